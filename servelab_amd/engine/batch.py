@@ -1,0 +1,123 @@
+"""One step's batch: the tokens to run and the metadata the kernels read.
+
+Reference: ``LLMEngine.step`` flattens the scheduled prefill chunks, then the
+decode tokens, into parallel lists tokens/positions/slots/metas/logit_rows
+(servelab/engine/engine.py:176-209) and copies three of them to the device
+(:213-215); block tables stay Python lists and are re-uploaded per layer.
+Here every array of a step is packed into one int32 buffer that is copied to
+the device once: ids, positions, the sequence of each token, cumulative query
+lengths, context lengths, state slots, wanted rows, and per page group the
+slot of each token and the block tables.
+"""
+from dataclasses import dataclass, field
+from typing import Any, Dict, Hashable, List, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens; ``want`` are the places among these tokens
+    whose logits are asked for."""
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class GroupMeta:
+    slots: torch.Tensor          # [T] flat cache row of each token in this group
+    block_tables: torch.Tensor   # [S, max_pages]
+    max_pages: int
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_seqs: int
+    num_prefill_seqs: int        # sequences with more than one token come first
+    num_prefill_tokens: int
+    num_logit_rows: int
+    max_q_len: int
+    max_ctx_len: int
+    # device int32
+    ids: torch.Tensor
+    positions: torch.Tensor
+    tok_seq: torch.Tensor        # [T] sequence index of each token
+    cu_q: torch.Tensor           # [S + 1]
+    ctx_len: torch.Tensor        # [S] tokens cached after this step
+    state_slots: torch.Tensor    # [S]
+    logit_rows: torch.Tensor     # [R]
+    groups: List[GroupMeta]
+    # host copies for parts that plan on the host
+    q_lens: List[int] = field(default_factory=list)
+    starts: List[int] = field(default_factory=list)
+    requests: List[Hashable] = field(default_factory=list)
+    host_state_slots: List[int] = field(default_factory=list)
+
+
+def pack_batch(entries: List[StepEntry], starts: List[int], rows: List[int], manager, device,
+               pad_pages_to: int = 8) -> StepBatch:
+    """Build the batch of ``entries`` (already ordered: multi-token first) whose
+    requests have ``starts[i]`` tokens cached and room for the new ones;
+    ``rows`` are the packed rows whose logits are wanted."""
+    bs = manager.page_size
+    S = len(entries)
+    q_lens = [len(e.tokens) for e in entries]
+    T = sum(q_lens)
+    cu = np.zeros(S + 1, dtype=np.int32)
+    np.cumsum(q_lens, out=cu[1:])
+    ids = np.empty(T, dtype=np.int32)
+    pos = np.empty(T, dtype=np.int32)
+    tok_seq = np.empty(T, dtype=np.int32)
+    for i, e in enumerate(entries):
+        a, b = cu[i], cu[i + 1]
+        ids[a:b] = np.asarray(e.tokens, dtype=np.int64)
+        pos[a:b] = np.arange(starts[i], starts[i] + q_lens[i], dtype=np.int32)
+        tok_seq[a:b] = i
+    ctx = np.asarray([starts[i] + q_lens[i] for i in range(S)], dtype=np.int32)
+    slots_host = [manager.state_slot(e.request) for e in entries]
+
+    parts = [ids, pos, tok_seq, cu, ctx, np.asarray(slots_host, dtype=np.int32),
+             np.asarray(rows, dtype=np.int32)]
+    group_shapes = []
+    for gi, g in enumerate(manager.page_groups):
+        max_pages = max(manager.pages_for(int(c)) for c in ctx)
+        max_pages = -(-max_pages // pad_pages_to) * pad_pages_to
+        tables = np.zeros((S, max_pages), dtype=np.int32)
+        slots = np.empty(T, dtype=np.int32)
+        for i, e in enumerate(entries):
+            table = np.asarray(g.tables[e.request], dtype=np.int32)
+            n = min(len(table), max_pages)
+            tables[i, :n] = np.maximum(table[:n], 0)     # released entries are never read
+            p = pos[cu[i]:cu[i + 1]]
+            page = table[p // bs]
+            if (page < 0).any():
+                raise AssertionError(f"request {e.request!r} writes into a released page")
+            slots[cu[i]:cu[i + 1]] = page * bs + p % bs
+        parts += [slots, tables.reshape(-1)]
+        group_shapes.append(max_pages)
+
+    sizes = [p.size for p in parts]
+    offsets = np.concatenate([[0], np.cumsum([-(-s // 4) * 4 for s in sizes])])   # 16-byte aligned
+    host = torch.empty(int(offsets[-1]), dtype=torch.int32,
+                       pin_memory=(torch.device(device).type == "cuda"))
+    host_np = host.numpy()
+    for p, o in zip(parts, offsets[:-1]):
+        host_np[o:o + p.size] = p
+    dev = host.to(device, non_blocking=True)
+    views = [dev[int(o):int(o) + s] for o, s in zip(offsets[:-1], sizes)]
+
+    groups = []
+    for gi, max_pages in enumerate(group_shapes):
+        groups.append(GroupMeta(views[7 + 2 * gi], views[8 + 2 * gi].view(S, max_pages), max_pages))
+    n_prefill = sum(1 for q in q_lens if q > 1)
+    return StepBatch(
+        num_tokens=T, num_seqs=S, num_prefill_seqs=n_prefill,
+        num_prefill_tokens=int(cu[n_prefill]), num_logit_rows=len(rows),
+        max_q_len=max(q_lens), max_ctx_len=int(ctx.max()),
+        ids=views[0], positions=views[1], tok_seq=views[2], cu_q=views[3], ctx_len=views[4],
+        state_slots=views[5], logit_rows=views[6], groups=groups,
+        q_lens=q_lens, starts=list(starts), requests=[e.request for e in entries],
+        host_state_slots=slots_host)

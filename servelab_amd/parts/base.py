@@ -1,0 +1,126 @@
+"""What every part is made of: parameter and cache declarations, the runtime a
+part computes with, and the interfaces of the five kinds of part.
+
+A part owns its sizes and constants as constructor parameters, declares the
+checkpoint tensors it needs under names *relative to itself* (the model puts
+the prefix in front), says what it needs cached per request, and computes
+through the kernel table of the runtime.  No part knows which model it is in.
+"""
+from dataclasses import dataclass
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One checkpoint tensor a part needs."""
+    shape: Tuple[int, ...]
+    init: str = "normal"       # random-weights mode: "normal" N(0, std) | "gain" 1 + N(0, norm_std)
+
+
+@dataclass(frozen=True)
+class PagedKVSpec:
+    """Cache need: keys and values of past tokens, in pages.  ``window`` None
+    keeps every token; a window W keeps the last W."""
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Cache need: one fixed-size state per request."""
+    shape: Tuple[int, ...]
+    dtype: str = "float32"
+
+
+class Runtime:
+    """Device, activation dtype and kernel table that parts compute with."""
+
+    def __init__(self, ops, device, act_dtype: torch.dtype):
+        self.ops = ops
+        self.device = torch.device(device)
+        self.act_dtype = act_dtype
+
+    def matrix(self, t: torch.Tensor) -> torch.Tensor:
+        """A matrix or table in the activation dtype, on the device."""
+        return t.to(device=self.device, dtype=self.act_dtype).contiguous()
+
+    def vector(self, t: torch.Tensor) -> torch.Tensor:
+        """A gain or bias: always float32 on the device (they enter float32 math)."""
+        return t.to(device=self.device, dtype=torch.float32).contiguous()
+
+
+TensorSource = Callable[[str], torch.Tensor]
+
+
+def prefixed(prefix: str, source: TensorSource) -> TensorSource:
+    return lambda name: source(prefix + name)
+
+
+class Part:
+    """Base of all parts."""
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def load(self, tensors: TensorSource, rt: Runtime) -> None:
+        """Fetch the declared tensors by relative name and keep device copies."""
+        self.rt = rt
+
+
+class Norm(Part):
+    """forward(resid, delta) adds ``delta`` (or nothing) into the float32
+    residual stream in place and returns the normed rows in the activation
+    dtype; forward_rows does the same for selected rows without changing the
+    stream."""
+
+    def forward(self, resid, delta):
+        raise NotImplementedError
+
+    def forward_rows(self, resid, delta, rows):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """A parameter of a mixer.  ``tables(batch, shared)`` returns what the
+    mixer's kernels need for this step's positions; ``shared`` is a per-step
+    dict so that equal encodings in many layers are prepared once."""
+
+    def tables(self, batch, shared):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Sequence mixer.  ``cache_spec`` declares its per-request cache need
+    (PagedKVSpec, StateSpec or None); ``forward(x, batch, cache, shared)`` maps
+    normed rows [T, H] to rows [T, H].  ``cache`` is the binding the cache
+    manager made for the layer call: pages plus block tables, or state plus
+    slot ids; ``cache.write`` is False when the call reads another call's
+    cache."""
+
+    def cache_spec(self):
+        return None
+
+    def forward(self, x, batch, cache, shared):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(x [T, H]) -> [T, H]."""
+
+    def forward(self, x):
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of norms, a mixer and a feed-forward around the residual
+    stream.  ``forward(resid, delta, batch, cache, shared) -> delta``: ``resid``
+    is the float32 stream (updated in place), ``delta`` the not yet added
+    output of what ran before (None at the start)."""
+
+    mixer: Mixer
+
+    def forward(self, resid, delta, batch, cache, shared):
+        raise NotImplementedError

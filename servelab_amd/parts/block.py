@@ -1,0 +1,36 @@
+"""Arrangements of parts in a block.
+
+PreNormBlock: h += Mixer(Norm1(h)); h += FeedForward(Norm2(h))
+(servelab/parallel/tp_model.py:124-133).  The adds are fused into the norm
+that follows them, so a block returns its feed-forward output as a pending
+delta for the next norm to add.
+"""
+from .base import Block, prefixed
+
+
+class PreNormBlock(Block):
+    def __init__(self, norm1, mixer, norm2, feedforward,
+                 names=("input_layernorm.", "self_attn.", "post_attention_layernorm.", "mlp.")):
+        self.norm1, self.mixer, self.norm2, self.feedforward = norm1, mixer, norm2, feedforward
+        self.names = tuple(names)
+
+    def _children(self):
+        return list(zip(self.names, (self.norm1, self.mixer, self.norm2, self.feedforward)))
+
+    def param_specs(self):
+        specs = {}
+        for prefix, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[prefix + name] = spec
+        return specs
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        for prefix, part in self._children():
+            part.load(prefixed(prefix, tensors), rt)
+
+    def forward(self, resid, delta, batch, cache, shared):
+        x = self.norm1.forward(resid, delta)
+        a = self.mixer.forward(x, batch, cache, shared)
+        x2 = self.norm2.forward(resid, a)
+        return self.feedforward.forward(x2)

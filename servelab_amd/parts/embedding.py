@@ -1,0 +1,45 @@
+"""Token embedding and output head.
+
+Embedding lookup servelab/parallel/tp_model.py:123; head = embedding table when
+tied, else its own matrix, no bias, logits returned in float32
+(servelab/parallel/tp_model.py:115-119, servelab/engine/engine.py:218).
+"""
+from .base import Part, ParamSpec
+
+
+class TokenEmbedding(Part):
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        self.weight = rt.matrix(tensors("weight"))
+
+    def forward(self, ids):
+        """int32 ids [T] -> float32 residual stream [T, H]."""
+        return self.rt.ops.embed(ids, self.weight)
+
+
+class OutputHead(Part):
+    """``tied_to`` is the embedding part whose table the head shares, or None."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to=None):
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.tied_to = tied_to
+
+    def param_specs(self):
+        if self.tied_to is not None:
+            return {}
+        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        self.weight = self.tied_to.weight if self.tied_to is not None \
+            else rt.matrix(tensors("weight"))
+
+    def forward(self, rows):
+        """normed rows [R, H] -> float32 logits [R, V]."""
+        return self.rt.ops.linear(rows, self.weight, None, out_f32=True)
