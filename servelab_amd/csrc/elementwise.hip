@@ -1,0 +1,129 @@
+// Embedding gather, SiLU-multiply, rotary tables, and rotary + cache write.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// out[t, :] = float(table[ids[t], :]).  Replaces the embedding lookup of
+// servelab/parallel/tp_model.py:123; the residual stream it starts is float.
+__global__ void embed_kernel(const int* __restrict__ ids, const act_t* __restrict__ table,
+                             float* __restrict__ out, int H, int V) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);     // the host rejects such ids; never fault
+  const act_t* row = table + (size_t)id * H;
+  float* o = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f(row[i]);
+}
+
+extern "C" const char* sl_embed(const int* ids, const void* table, float* out, int T, int H,
+                                int V, hipStream_t stream) {
+  SL_CHECK(T >= 0 && H > 0 && V > 0, "embed: sizes must be positive");
+  if (T == 0) return nullptr;
+  embed_kernel<<<T, 256, 0, stream>>>(ids, (const act_t*)table, out, H, V);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------- silu * up
+// out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i], silu(z) = z * sigmoid(z)
+// (servelab/parallel/tp_model.py:68), float inside.
+__global__ void silu_mul_kernel(const act_t* __restrict__ gate_up, act_t* __restrict__ out,
+                                int I, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / I;
+    const int i = (int)(idx - t * I);
+    const float g = to_f(gate_up[t * 2 * I + i]);
+    const float u = to_f(gate_up[t * 2 * I + I + i]);
+    out[idx] = from_f<act_t>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" const char* sl_silu_mul(const void* gate_up, void* out, int T, int I,
+                                   hipStream_t stream) {
+  SL_CHECK(T >= 0 && I > 0, "silu_mul: sizes must be positive");
+  if (T == 0) return nullptr;
+  const size_t total = (size_t)T * I;
+  const int blocks = (int)((total + 255) / 256 < 65535 * 4 ? (total + 255) / 256 : 65535 * 4);
+  silu_mul_kernel<<<blocks, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, I, total);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------------------ rotary tables
+// cos/sin[t, j] of angle float(pos[t]) * inv_freq[j], float32 with the
+// accurate cosf/sinf.  Once per step; every layer reads the same table.
+__global__ void rope_tables_kernel(const int* __restrict__ pos, const float* __restrict__ inv_freq,
+                                   float* __restrict__ cosv, float* __restrict__ sinv,
+                                   int half, int total) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int t = idx / half, j = idx - t * half;
+  const float ang = (float)pos[t] * inv_freq[j];
+  cosv[idx] = cosf(ang);
+  sinv[idx] = sinf(ang);
+}
+
+extern "C" const char* sl_rope_tables(const int* pos, const float* inv_freq, float* cosv,
+                                      float* sinv, int T, int half, hipStream_t stream) {
+  SL_CHECK(T >= 0 && half > 0, "rope_tables: sizes must be positive");
+  if (T == 0) return nullptr;
+  const int total = T * half;
+  rope_tables_kernel<<<(total + 255) / 256, 256, 0, stream>>>(pos, inv_freq, cosv, sinv, half,
+                                                              total);
+  return sl_launch_status();
+}
+
+// ------------------------------------------------- rotary + write to pages
+// qkv rows are [q heads | k heads | v heads], head-major.  q and k are rotated
+// in place with pairs (j, j + D/2) (servelab/parallel/tp_model.py:128); the
+// rotated k and the v of each token go to its cache row (:129,
+// servelab/kv_cache/pool.py:68-78): K pages [page, nkv, page_size, D], V pages
+// [page, nkv, D, page_size].  One block per (token, head).
+__global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restrict__ cosv,
+                                  const float* __restrict__ sinv, const int* __restrict__ slots,
+                                  act_t* __restrict__ kc, act_t* __restrict__ vc, int nh, int nkv,
+                                  int D, int page) {
+  const int t = blockIdx.x, hd = blockIdx.y;
+  const int half = D / 2;
+  act_t* x = qkv + ((size_t)t * (nh + 2 * nkv) + hd) * D;
+  if (hd < nh + nkv) {
+    act_t* dst = nullptr;
+    if (hd >= nh && kc != nullptr) {
+      const int slot = slots[t];
+      dst = kc + (((size_t)(slot / page) * nkv + (hd - nh)) * page + slot % page) * D;
+    }
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+      float x1 = to_f(x[j]), x2 = to_f(x[j + half]);
+      if (cosv != nullptr) {
+        const float c = cosv[(size_t)t * half + j], s = sinv[(size_t)t * half + j];
+        const float r1 = x1 * c - x2 * s, r2 = x2 * c + x1 * s;
+        x1 = r1;
+        x2 = r2;
+        x[j] = from_f<act_t>(x1);
+        x[j + half] = from_f<act_t>(x2);
+      }
+      if (dst != nullptr) {
+        dst[j] = from_f<act_t>(x1);
+        dst[j + half] = from_f<act_t>(x2);
+      }
+    }
+  } else if (vc != nullptr) {
+    const int slot = slots[t];
+    act_t* dst = vc + ((size_t)(slot / page) * nkv + (hd - nh - nkv)) * D * page + slot % page;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[(size_t)d * page] = x[d];
+  }
+}
+
+extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* sinv,
+                                     const int* slots, void* kc, void* vc, int T, int nh, int nkv,
+                                     int D, int page, hipStream_t stream) {
+  SL_CHECK(T >= 0 && nh > 0 && nkv > 0, "rope_store: sizes must be positive");
+  SL_CHECK(D > 0 && D % 2 == 0, "rope_store: head_dim must be even");
+  SL_CHECK((cosv == nullptr) == (sinv == nullptr), "rope_store: cos and sin go together");
+  SL_CHECK((kc == nullptr) == (vc == nullptr), "rope_store: k and v pages go together");
+  SL_CHECK(kc == nullptr || (slots != nullptr && page > 0), "rope_store: pages need slots");
+  if (T == 0) return nullptr;
+  const int heads = kc != nullptr ? nh + 2 * nkv : nh + nkv;
+  if (cosv == nullptr && kc == nullptr) return nullptr;
+  rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, cosv, sinv, slots,
+                                                       (act_t*)kc, (act_t*)vc, nh, nkv, D, page);
+  return sl_launch_status();
+}

@@ -1,0 +1,2 @@
+from .build import BuildError, all_units, ensure
+from .ops import HipOps, KernelError

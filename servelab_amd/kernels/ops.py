@@ -1,0 +1,236 @@
+"""The kernel table: every device computation of the engine, as calls into the
+hand-written HIP libraries (ctypes, C ABI, the caller's current stream).
+
+There is no fallback: without a GPU, without hipcc-built libraries, or for a
+size a kernel refuses, a call raises.  Shapes, dtypes and contiguity are
+checked here on the host before any launch, because a kernel that reads out of
+bounds can take the GPU down.
+
+Large bfloat16 matrix products (more rows than the hand-written few-rows
+kernel takes) go to the library GEMM behind ``torch.addmm`` — where the
+reference calls ``F.linear`` (servelab/parallel/layers.py:164-180).  The
+float32 table never does: its products are the hand-written FMA kernels.
+"""
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+_c_int, _c_float, _c_void_p = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else _c_void_p(t.data_ptr())
+
+
+class HipOps:
+    ROWS_KERNEL_MAX_M = 16        # the few-rows GEMM takes up to this many rows per pass
+
+    def __init__(self, act_dtype: torch.dtype, device="cuda:0"):
+        if act_dtype not in (torch.bfloat16, torch.float32):
+            raise KernelError(f"kernels exist for bfloat16 and float32, not {act_dtype}")
+        if not torch.cuda.is_available():
+            raise KernelError("servelab_amd needs a GPU: the HIP kernels have no CPU fallback")
+        self.act_dtype = act_dtype
+        self.device = torch.device(device)
+        self.dtype_name = "float32" if act_dtype == torch.float32 else "bfloat16"
+        units = [build.unit(stem, self.dtype_name) for stem in build.DEFAULT_STEMS]
+        build.ensure(units)
+        self._lib = {stem: build.load(build.unit(stem, self.dtype_name))
+                     for stem in build.DEFAULT_STEMS}
+        self._fn = {}
+        self._bias_cache = {}
+
+    # ------------------------------------------------------------ plumbing
+    def _call(self, stem, name, *args):
+        fn = self._fn.get(name)
+        if fn is None:
+            fn = getattr(self._lib[stem], name)
+            fn.restype = ctypes.c_char_p
+            self._fn[name] = fn
+        err = fn(*args, _c_void_p(torch.cuda.current_stream().cuda_stream))
+        if err is not None:
+            raise KernelError(f"{name}: {err.decode()}")
+
+    def _check(self, t, dtype, shape=None, name="tensor"):
+        if t.device.type != "cuda":
+            raise KernelError(f"{name} is on {t.device}, not on the GPU")
+        if t.dtype != dtype:
+            raise KernelError(f"{name} has dtype {t.dtype}, expected {dtype}")
+        if not t.is_contiguous():
+            raise KernelError(f"{name} is not contiguous")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{name} has shape {list(t.shape)}, expected {list(shape)}")
+
+    def _new(self, shape, dtype=None):
+        return torch.empty(shape, dtype=dtype or self.act_dtype, device=self.device)
+
+    # ------------------------------------------------------------ embedding
+    def embed(self, ids, table):
+        T = ids.shape[0]
+        V, H = table.shape
+        self._check(ids, torch.int32, (T,), "ids")
+        self._check(table, self.act_dtype, None, "embedding table")
+        out = self._new((T, H), torch.float32)
+        self._call("elementwise", "sl_embed", _p(ids), _p(table), _p(out), T, H, V)
+        return out
+
+    # ---------------------------------------------------------------- norms
+    def add_rmsnorm(self, resid, delta, weight, eps):
+        T, H = resid.shape
+        self._check(resid, torch.float32, None, "residual stream")
+        self._check(weight, torch.float32, (H,), "norm weight")
+        if delta is not None:
+            self._check(delta, self.act_dtype, (T, H), "delta")
+        out = self._new((T, H))
+        self._call("norm", "sl_add_rmsnorm", _p(resid), _p(delta), None, _p(weight), _p(out),
+                   T, H, _c_float(eps))
+        return out
+
+    def rows_add_rmsnorm(self, resid, delta, rows, weight, eps):
+        T, H = resid.shape
+        R = rows.shape[0]
+        self._check(resid, torch.float32, None, "residual stream")
+        self._check(weight, torch.float32, (H,), "norm weight")
+        self._check(rows, torch.int32, (R,), "rows")
+        if delta is not None:
+            self._check(delta, self.act_dtype, (T, H), "delta")
+        out = self._new((R, H))
+        self._call("norm", "sl_add_rmsnorm", _p(resid), _p(delta), _p(rows), _p(weight), _p(out),
+                   R, H, _c_float(eps))
+        return out
+
+    # --------------------------------------------------------------- linear
+    def linear(self, x, w, bias, out_f32=False):
+        M, K = x.shape
+        N = w.shape[0]
+        self._check(x, self.act_dtype, None, "x")
+        self._check(w, self.act_dtype, (N, K), "weight")
+        if bias is not None:
+            self._check(bias, torch.float32, (N,), "bias")
+        vec = 4 if self.act_dtype == torch.float32 else 8
+        rows_ok = K % vec == 0
+        if rows_ok and M <= self.ROWS_KERNEL_MAX_M:
+            return self.linear_rows(x, w, bias, out_f32)
+        if self.act_dtype == torch.float32:
+            return self.linear_tiled(x, w, bias, out_f32)
+        if out_f32:
+            if rows_ok and M <= 4 * self.ROWS_KERNEL_MAX_M:
+                return self.linear_rows(x, w, bias, out_f32)
+            return self.linear_tiled(x, w, bias, out_f32)
+        return self.linear_library(x, w, bias)
+
+    def linear_rows(self, x, w, bias, out_f32=False):
+        M, K = x.shape
+        N = w.shape[0]
+        y = self._new((M, N), torch.float32 if out_f32 else None)
+        self._call("gemm", "sl_gemm_rows", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32))
+        return y
+
+    def linear_tiled(self, x, w, bias, out_f32=False):
+        M, K = x.shape
+        N = w.shape[0]
+        y = self._new((M, N), torch.float32 if out_f32 else None)
+        self._call("gemm", "sl_gemm_tiled", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32))
+        return y
+
+    def linear_library(self, x, w, bias):
+        if self.act_dtype != torch.bfloat16:
+            raise KernelError("the library GEMM is for the bfloat16 table only")
+        if bias is None:
+            return torch.mm(x, w.t())
+        key = bias.data_ptr()
+        b = self._bias_cache.get(key)
+        if b is None or b.shape != bias.shape:
+            b = bias.to(torch.bfloat16)
+            self._bias_cache[key] = b
+        return torch.addmm(b, x, w.t())
+
+    def silu_mul(self, gate_up):
+        T, two_i = gate_up.shape
+        if two_i % 2:
+            raise KernelError("silu_mul: the row must hold gate and up of equal width")
+        self._check(gate_up, self.act_dtype, None, "gate_up")
+        out = self._new((T, two_i // 2))
+        self._call("elementwise", "sl_silu_mul", _p(gate_up), _p(out), T, two_i // 2)
+        return out
+
+    # ----------------------------------------------------------------- rope
+    def rope_tables(self, positions, inv_freq):
+        T, half = positions.shape[0], inv_freq.shape[0]
+        self._check(positions, torch.int32, (T,), "positions")
+        self._check(inv_freq, torch.float32, (half,), "inv_freq")
+        cos = self._new((T, half), torch.float32)
+        sin = self._new((T, half), torch.float32)
+        self._call("elementwise", "sl_rope_tables", _p(positions), _p(inv_freq), _p(cos), _p(sin),
+                   T, half)
+        return cos, sin
+
+    def _check_pages(self, k_cache, v_cache, nkv, D, page_size):
+        pages = k_cache.shape[0]
+        self._check(k_cache, self.act_dtype, (pages, nkv, page_size, D), "K pages")
+        self._check(v_cache, self.act_dtype, (pages, nkv, D, page_size), "V pages")
+        return pages
+
+    def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size):
+        T = qkv.shape[0]
+        self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
+        if cos is not None:
+            self._check(cos, torch.float32, (T, D // 2), "cos")
+            self._check(sin, torch.float32, (T, D // 2), "sin")
+        if k_cache is not None:
+            self._check_pages(k_cache, v_cache, nkv, D, page_size)
+            self._check(slots, torch.int32, (T,), "slots")
+        self._call("elementwise", "sl_rope_store", _p(qkv), _p(cos), _p(sin), _p(slots),
+                   _p(k_cache), _p(v_cache), T, nh, nkv, D, page_size)
+
+    # ------------------------------------------------------------ attention
+    def paged_attention(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                        batch, scale, window):
+        T = qkv.shape[0]
+        S, max_pages = block_tables.shape
+        self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
+        self._check_pages(k_cache, v_cache, nkv, D, page_size)
+        self._check(block_tables, torch.int32, None, "block tables")
+        self._check(batch.tok_seq, torch.int32, (T,), "tok_seq")
+        self._check(batch.positions, torch.int32, (T,), "positions")
+        if S != batch.num_seqs:
+            raise KernelError(f"block tables hold {S} sequences, the batch {batch.num_seqs}")
+        if batch.max_ctx_len > max_pages * page_size:
+            raise KernelError(f"context {batch.max_ctx_len} exceeds the block table "
+                              f"({max_pages} pages of {page_size})")
+        out = self._new((T, nh * D))
+        self._call("attention", "sl_attention_general", _p(qkv), (nh + 2 * nkv) * D, _p(k_cache),
+                   _p(v_cache), _p(block_tables), max_pages, _p(batch.tok_seq),
+                   _p(batch.positions), T, nh, nkv, D, page_size, _c_float(scale),
+                   int(window or 0), _p(out))
+        return out
+
+    # ------------------------------------------------------------- sampling
+    def argmax(self, logits):
+        R, V = logits.shape
+        self._check(logits, torch.float32, None, "logits")
+        out = self._new((R,), torch.int32)
+        self._call("sampling", "sl_sample", _p(logits), R, V, None, None, None, None, None,
+                   _p(out))
+        return out
+
+    def sample(self, logits, temperature, top_k, top_p, seeds, draws):
+        """One token per row; rows with temperature 0 take the argmax."""
+        R, V = logits.shape
+        self._check(logits, torch.float32, None, "logits")
+        self._check(temperature, torch.float32, (R,), "temperature")
+        self._check(top_k, torch.int32, (R,), "top_k")
+        self._check(top_p, torch.float32, (R,), "top_p")
+        self._check(seeds, torch.int64, (R,), "seeds")
+        self._check(draws, torch.int64, (R,), "draws")
+        out = self._new((R,), torch.int32)
+        self._call("sampling", "sl_sample", _p(logits), R, V, _p(temperature), _p(top_k),
+                   _p(top_p), _p(seeds), _p(draws), _p(out))
+        return out

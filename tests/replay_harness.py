@@ -1,0 +1,70 @@
+"""Runs a schedule through the replay tool (in process or as the bin/trace_run
+program) and compares every written row with the plain implementation."""
+import argparse
+import io
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import torch
+
+import plain_qwen2 as plain
+from replay_schedules import expected_rows, max_tokens_needed
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_logits(folder, requests):
+    cfg, w = plain.load_folder(folder)
+    return {rid: plain.forward(cfg, w, toks).numpy() for rid, toks in requests.items()}
+
+
+def replay_in_process(folder, steps, out_dir, dtype, max_tokens, ops=None, device="cuda:0",
+                      block_size=16):
+    from servelab_amd.replay import run
+    args = argparse.Namespace(model=folder, dtype=dtype, out=out_dir, max_tokens=max_tokens,
+                              block_size=block_size, device=device)
+    stdin = io.StringIO("".join(json.dumps(s) + "\n" for s in steps))
+    stdout = io.StringIO()
+    assert run(args, stdin, stdout, ops=ops) == 0
+    assert stdout.getvalue().split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+
+
+def replay_program(folder, steps, out_dir, dtype, max_tokens, env=None):
+    """Through bin/trace_run, one step at a time, waiting for each 'done'."""
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder,
+           "--dtype", dtype, "--out", out_dir, "--max-tokens", str(max_tokens)]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=env)
+    try:
+        for s in steps:
+            proc.stdin.write(json.dumps(s) + "\n")
+            proc.stdin.flush()
+            line = proc.stdout.readline().strip()
+            assert line == f"done {s['step']}", f"got {line!r}"
+        proc.stdin.close()
+        assert proc.wait(timeout=120) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+
+
+def compare(out_dir, steps, reference, vocab):
+    """Largest absolute difference over all written rows."""
+    worst, where = 0.0, None
+    rows = expected_rows(steps)
+    for step, wanted in rows.items():
+        path = os.path.join(out_dir, f"{step}.f32")
+        assert os.path.exists(path), f"step {step} wrote no file"
+        got = np.fromfile(path, dtype="<f4").reshape(-1, vocab)
+        assert got.shape[0] == len(wanted), f"step {step}: {got.shape[0]} rows, wanted {len(wanted)}"
+        assert np.isfinite(got).all(), f"step {step}: logits are not finite"
+        for row, (rid, p) in zip(got, wanted):
+            err = float(np.abs(row - reference[rid][p]).max())
+            if err > worst:
+                worst, where = err, (step, rid, p)
+    for st in steps:
+        if st["step"] not in rows:
+            assert not os.path.exists(os.path.join(out_dir, f"{st['step']}.f32"))
+    return worst, where

@@ -1,0 +1,274 @@
+"""Each HIP kernel alone against the plain torch function of the same name
+(tests/emulated_ops.py), in float32 and in bfloat16, at sizes other than the
+tiny models': widths and vocabularies that are no power of two, several head
+sizes, group sizes and page sizes."""
+import math
+import types
+
+import pytest
+import torch
+
+from emulated_ops import EmulatedOps
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+# elementwise results are rounded once to the activation dtype: half an ulp
+ELEM_TOL = {torch.float32: 2e-6, torch.bfloat16: 2 ** -8}
+
+
+@pytest.fixture(scope="module", params=DTYPES, ids=["float32", "bfloat16"])
+def both(request):
+    from servelab_amd.kernels import HipOps
+    dt = request.param
+    return HipOps(dt, "cuda:0"), EmulatedOps(dt), dt
+
+
+def randn(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+def rel_err(got, ref):
+    got, ref = got.float(), ref.float()
+    return ((got - ref).abs().max() / ref.abs().max().clamp_min(1e-6)).item()
+
+
+def test_embed(both):
+    ops, emu, dt = both
+    table = randn(1000, 96, dtype=dt)
+    ids = torch.tensor([0, 999, 5, 5, 317], dtype=torch.int32).cuda()
+    assert torch.equal(ops.embed(ids, table), emu.embed(ids, table))
+
+
+@pytest.mark.parametrize("T,H", [(1, 64), (7, 3584), (33, 1000), (5, 130)])
+def test_add_rmsnorm(both, T, H):
+    ops, emu, dt = both
+    resid = randn(T, H, seed=1)
+    delta = randn(T, H, dtype=dt, seed=2)
+    w = 1 + 0.1 * randn(H, seed=3)
+    r1, r2 = resid.clone(), resid.clone()
+    got = ops.add_rmsnorm(r1, delta, w, 1e-5)
+    ref = emu.add_rmsnorm(r2, delta, w, 1e-5)
+    assert (r1 - r2).abs().max().item() < 1e-6
+    assert rel_err(got, ref) < ELEM_TOL[dt] * 2
+    # without a delta the stream is left alone
+    r3 = resid.clone()
+    got = ops.add_rmsnorm(r3, None, w, 1e-6)
+    assert torch.equal(r3, resid)
+    assert rel_err(got, emu.add_rmsnorm(resid.clone(), None, w, 1e-6)) < ELEM_TOL[dt] * 2
+
+
+def test_rows_add_rmsnorm(both):
+    ops, emu, dt = both
+    resid, delta = randn(20, 200, seed=1), randn(20, 200, dtype=dt, seed=2)
+    w = 1 + 0.1 * randn(200, seed=3)
+    rows = torch.tensor([19, 0, 7, 7], dtype=torch.int32).cuda()
+    before = resid.clone()
+    got = ops.rows_add_rmsnorm(resid, delta, rows, w, 1e-6)
+    assert torch.equal(resid, before)
+    assert rel_err(got, emu.rows_add_rmsnorm(resid, delta, rows, w, 1e-6)) < ELEM_TOL[dt] * 2
+    got = ops.rows_add_rmsnorm(resid, None, rows, w, 1e-6)
+    assert rel_err(got, emu.rows_add_rmsnorm(resid, None, rows, w, 1e-6)) < ELEM_TOL[dt] * 2
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 64), (3, 130, 200), (8, 512, 3584), (16, 96, 352),
+                                   (17, 200, 136), (70, 1000, 128), (130, 352, 64)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_linear(both, M, N, K, bias):
+    ops, emu, dt = both
+    x, w = randn(M, K, dtype=dt, seed=1), randn(N, K, dtype=dt, scale=0.05, seed=2)
+    b = randn(N, seed=3) if bias else None
+    tol = 1e-5 if dt == torch.float32 else 2 ** -7
+    for out_f32 in (False, True):
+        got = ops.linear(x, w, b, out_f32=out_f32)
+        ref = emu.linear(x, w, b, out_f32=out_f32)
+        assert got.dtype == ref.dtype and got.shape == ref.shape
+        assert rel_err(got, ref) < tol, (M, N, K, out_f32)
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 70, 24), (64, 64, 16), (65, 129, 37)])
+def test_linear_kernels_separately(both, M, N, K):
+    """The tiled kernel takes any K; the few-rows kernel any K that fills
+    16-byte vectors."""
+    ops, emu, dt = both
+    x, w = randn(M, K, dtype=dt, seed=4), randn(N, K, dtype=dt, scale=0.1, seed=5)
+    b = randn(N, seed=6)
+    tol = 1e-5 if dt == torch.float32 else 2 ** -7
+    ref = emu.linear(x, w, b)
+    assert rel_err(ops.linear_tiled(x, w, b), ref) < tol
+    if K % 8 == 0:
+        assert rel_err(ops.linear_rows(x, w, b), ref) < tol
+    else:
+        from servelab_amd.kernels import KernelError
+        with pytest.raises(KernelError):
+            ops.linear_rows(x, w, b)
+
+
+def test_silu_mul(both):
+    ops, emu, dt = both
+    gu = randn(9, 2 * 353, dtype=dt, scale=3.0)
+    assert rel_err(ops.silu_mul(gu), emu.silu_mul(gu)) < ELEM_TOL[dt] * 2
+    gu[:, :353] = 0          # gate 0 => output 0
+    assert ops.silu_mul(gu).abs().max().item() == 0
+
+
+def test_rope_tables(both):
+    ops, emu, dt = both
+    D, theta = 48, 1e6
+    inv = (1.0 / theta ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
+    pos = torch.tensor([0, 1, 17, 4095, 32767], dtype=torch.int32).cuda()
+    cos, sin = ops.rope_tables(pos, inv)
+    # against float64 angles of the same float32 products
+    ang = (pos.float()[:, None] * inv[None, :]).double()
+    assert (cos.double() - torch.cos(ang)).abs().max().item() < 2e-7
+    assert (sin.double() - torch.sin(ang)).abs().max().item() < 2e-7
+
+
+@pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (6, 1, 48, 32), (7, 7, 128, 64)])
+def test_rope_store(both, nh, nkv, D, page):
+    ops, emu, dt = both
+    T, pages = 37, 9
+    qkv = randn(T, (nh + 2 * nkv) * D, dtype=dt, seed=1)
+    inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
+    pos = torch.arange(100, 100 + T, dtype=torch.int32).cuda()
+    cos, sin = emu.rope_tables(pos, inv)
+    slots = torch.randperm(pages * page)[:T].to(torch.int32).cuda()
+    kc = [randn(pages, nkv, page, D, dtype=dt, seed=7) for _ in range(2)]
+    vc = [randn(pages, nkv, D, page, dtype=dt, seed=8) for _ in range(2)]
+    q1, q2 = qkv.clone(), qkv.clone()
+    ops.rope_store(q1, nh, nkv, D, cos, sin, slots, kc[0], vc[0], page)
+    emu.rope_store(q2, nh, nkv, D, cos, sin, slots, kc[1], vc[1], page)
+    assert rel_err(q1, q2) < ELEM_TOL[dt] * 2
+    assert rel_err(kc[0], kc[1]) < ELEM_TOL[dt] * 2
+    assert torch.equal(vc[0], vc[1])
+    # no tables: nothing rotates; no pages: nothing is written
+    q3 = qkv.clone()
+    ops.rope_store(q3, nh, nkv, D, None, None, slots, kc[0], vc[0], page)
+    assert torch.equal(q3, qkv)
+    k_before = kc[0].clone()
+    ops.rope_store(qkv.clone(), nh, nkv, D, cos, sin, None, None, None, page)
+    assert torch.equal(kc[0], k_before)
+
+
+def make_attention_case(dt, nh, nkv, D, page, seqs, seed=0):
+    """``seqs``: list of (context length after the step, query length).  Builds
+    a cache with shuffled pages and garbage in unused rows."""
+    g = torch.Generator().manual_seed(seed)
+    bs = page
+    n_pages = sum(-(-c // bs) for c, _ in seqs) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kc = randn(n_pages, nkv, bs, D, dtype=dt, seed=seed + 1)
+    vc = randn(n_pages, nkv, D, bs, dtype=dt, seed=seed + 2)
+    max_pages = max(-(-c // bs) for c, _ in seqs) + 1
+    tables = torch.zeros(len(seqs), max_pages, dtype=torch.int32)
+    tok_seq, positions, cu = [], [], [0]
+    for s, (ctx, q) in enumerate(seqs):
+        n = -(-ctx // bs)
+        tables[s, :n] = torch.tensor([perm.pop() for _ in range(n)], dtype=torch.int32)
+        tok_seq += [s] * q
+        positions += list(range(ctx - q, ctx))
+        cu.append(cu[-1] + q)
+    T = cu[-1]
+    qkv = randn(T, (nh + 2 * nkv) * D, dtype=dt, seed=seed + 3)
+    batch = types.SimpleNamespace(
+        num_seqs=len(seqs), num_tokens=T,
+        tok_seq=torch.tensor(tok_seq, dtype=torch.int32).cuda(),
+        positions=torch.tensor(positions, dtype=torch.int32).cuda(),
+        cu_q=torch.tensor(cu, dtype=torch.int32).cuda(),
+        ctx_len=torch.tensor([c for c, _ in seqs], dtype=torch.int32).cuda(),
+        max_ctx_len=max(c for c, _ in seqs), max_q_len=max(q for _, q in seqs),
+        num_prefill_seqs=sum(1 for _, q in seqs if q > 1))
+    return qkv, kc, vc, tables.cuda(), batch
+
+
+ATTN_TOL = {torch.float32: 2e-5, torch.bfloat16: 2 ** -7}
+
+
+@pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (8, 1, 32, 16), (7, 7, 48, 32),
+                                           (28, 4, 128, 16), (6, 2, 256, 64), (5, 5, 80, 16)])
+@pytest.mark.parametrize("window", [None, 16, 50])
+def test_paged_attention(both, nh, nkv, D, page, window):
+    ops, emu, dt = both
+    seqs = [(130, 130), (77, 5), (64, 64), (200, 2), (16, 1), (145, 1), (1, 1), (333, 1)]
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs)
+    scale = 1.0 / math.sqrt(D)
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
+    ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                              types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                       for k, v in vars(batch).items()}),
+                              scale, window)
+    assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+
+
+def test_attention_finds_a_far_key(both):
+    """One key among hundreds carries all the weight: scale one query and that
+    key so its score stands out; the output must be that key's value."""
+    ops, emu, dt = both
+    nh, nkv, D, page = 4, 2, 32, 16
+    seqs = [(400, 1)]
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=3)
+    target = 37
+    pg, off = int(tables[0, target // page]), target % page
+    q = torch.zeros(D)
+    q[0] = 30.0
+    qkv[0, :nh * D] = q.repeat(nh).to(dt)
+    kc[:, :, :, 0] = 0
+    kc[pg, :, off, 0] = 30.0
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, None)
+    for h in range(nh):
+        want = vc[pg, h // 2, :, off].float()
+        assert (got[0, h * D:(h + 1) * D].float() - want).abs().max().item() < 2e-2
+    # with a window that ends before the target the key is invisible
+    got_w = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, 100)
+    assert (got_w.float() - got.float()).abs().max().item() > 0.1
+
+
+def test_argmax_and_sampling():
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.float32, "cuda:0")
+    V = 152064 // 8 + 7
+    logits = randn(5, V, seed=1)
+    logits[2, 77] = 50.0
+    logits[2, 9000] = 50.0            # ties resolve to the first index
+    assert ops.argmax(logits).tolist() == torch.argmax(logits, -1).tolist()
+    assert ops.argmax(logits)[2].item() == 77
+
+    # temperature sampling follows softmax(logits / T)
+    V, n = 11, 20000
+    base = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, 3.0, 0.1, 0.2, -3.0, 1.5, 2.5])
+    logits = base.repeat(n, 1).cuda()
+    T = 0.7
+    temp = torch.full((n,), T).cuda()
+    top_k = torch.full((n,), -1, dtype=torch.int32).cuda()
+    top_p = torch.ones(n).cuda()
+    seeds = torch.full((n,), 1234, dtype=torch.int64).cuda()
+    draws = torch.arange(n, dtype=torch.int64).cuda()
+    toks = ops.sample(logits, temp, top_k, top_p, seeds, draws)
+    freq = torch.bincount(toks.long().cpu(), minlength=V).float() / n
+    want = torch.softmax(base / T, -1)
+    assert (freq - want).abs().max().item() < 0.015
+    # same seed and draw => same token; temperature 0 rows take the argmax
+    assert torch.equal(toks, ops.sample(logits, temp, top_k, top_p, seeds, draws))
+    temp0 = torch.zeros(n).cuda()
+    assert set(ops.sample(logits, temp0, top_k, top_p, seeds, draws).tolist()) == {5}
+    # top-k 3 draws only the three largest, renormalised
+    k3 = torch.full((n,), 3, dtype=torch.int32).cuda()
+    toks = ops.sample(logits, temp, k3, top_p, seeds, draws)
+    freq = torch.bincount(toks.long().cpu(), minlength=V).float() / n
+    keep = torch.zeros(V)
+    keep[[5, 10, 0]] = 1
+    want3 = torch.softmax(base / T, -1) * keep
+    want3 /= want3.sum()
+    assert (freq - want3).abs().max().item() < 0.015
+    # top-p: sorted prefix with cumulative probability <= p (first always kept)
+    p = 0.8
+    probs = torch.softmax(base / T, -1)
+    sp, si = torch.sort(probs, descending=True)
+    kept = si[(torch.cumsum(sp, 0) <= p) | (torch.arange(V) == 0)]
+    wantp = torch.zeros(V)
+    wantp[kept] = probs[kept]
+    wantp /= wantp.sum()
+    toks = ops.sample(logits, temp, top_k, torch.full((n,), p).cuda(), seeds, draws)
+    freq = torch.bincount(toks.long().cpu(), minlength=V).float() / n
+    assert (freq - wantp).abs().max().item() < 0.015

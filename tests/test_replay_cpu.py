@@ -1,0 +1,40 @@
+"""The replay tool over the engine's host side (cache manager, batch packing,
+step function) with the kernels emulated in torch on the CPU: every cutting of
+the same requests gives the plain implementation's logits."""
+import random
+
+import pytest
+import torch
+
+import replay_schedules as rs
+from emulated_ops import EmulatedOps
+from replay_harness import compare, plain_logits, replay_in_process
+from tiny_configs import TINY, make_folder
+
+
+def make_requests(vocab, lengths, seed):
+    rng = random.Random(seed)
+    return {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(lengths)}
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+def test_replay_matches_plain(tmp_path, which, schedule):
+    folder = make_folder(tmp_path, which, seed=11)
+    vocab = TINY[which]["vocab_size"]
+    lengths = [37, 70, 49, 96, 130, 41, 66] if which == "A" else [41, 109, 56, 200, 33, 77]
+    requests = make_requests(vocab, lengths, seed=5)
+    reference = plain_logits(folder, requests)
+    if schedule == "whole":
+        steps = rs.whole(requests)
+    elif schedule == "tail":
+        steps = rs.tail_decoded(requests)
+    elif schedule == "portions":
+        steps = rs.portions(requests)
+    else:
+        steps = rs.mixed(requests, {r: max(2, len(t) - 32) for r, t in requests.items()})
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, "float32", rs.max_tokens_needed(steps),
+                      ops=EmulatedOps(torch.float32), device="cpu")
+    worst, where = compare(out, steps, reference, vocab)
+    assert worst < 1e-4, f"max abs err {worst} at {where}"
