@@ -10,7 +10,8 @@ from . import models as _models  # registers the architectures  # noqa: F401
 from .config import (CacheConfig, ConfigError, EngineConfig, ModelConfig, Qwen2Config,
                      SchedulerConfig, register_architecture)
 from .weights import WeightError, load_config, load_model, write_random_model
+from .engine import LLMEngine, RequestOutput, SamplingParams
 
 __all__ = ["CacheConfig", "ConfigError", "EngineConfig", "ModelConfig", "Qwen2Config",
            "SchedulerConfig", "register_architecture", "WeightError", "load_config",
-           "load_model", "write_random_model"]
+           "load_model", "write_random_model", "LLMEngine", "RequestOutput", "SamplingParams"]

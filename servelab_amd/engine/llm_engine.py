@@ -1,0 +1,151 @@
+"""The engine: scheduler, cache manager, step function and sampler together.
+
+Reference: ``LLMEngine`` (servelab/engine/engine.py:42-297) with the same
+entry points — add_request, abort_request, has_unfinished, step, generate,
+stats — and the same constructor arguments where they apply to one GPU.
+"""
+import time
+from typing import Callable, Dict, List, Optional
+
+import torch
+
+from ..config import CacheConfig, SchedulerConfig
+from ..sampling import Sampler
+from .batch import StepEntry
+from .output import RequestOutput
+from .sampling_params import SamplingParams
+from .scheduler import Scheduler
+from .sequence import Sequence
+from .session import load_model_on_device, make_runner
+
+
+class LLMEngine:
+    def __init__(self, model_config, cache_config: Optional[CacheConfig] = None,
+                 scheduler_config: Optional[SchedulerConfig] = None, seed: int = 1234,
+                 device: str = "cuda:0", tokenizer=None,
+                 clock: Optional[Callable[[], float]] = None, dtype: str = "auto",
+                 model=None, ops=None):
+        """``model_config.path`` names the model folder (as in the reference,
+        servelab/engine/engine.py:86-87); ``model`` may pass an already loaded
+        DecoderModel instead."""
+        self.model_config = model_config
+        self.cache_config = cache_config or CacheConfig()
+        self.scheduler_config = scheduler_config or SchedulerConfig()
+        self.tokenizer = tokenizer
+        self.clock = clock or time.monotonic
+        if device == "auto":
+            device = "cuda:0"
+        if model is None:
+            if not getattr(model_config, "path", ""):
+                raise ValueError("model_config.path must name a model folder "
+                                 "(write_random_model makes one from a configuration and a seed)")
+            _, model = load_model_on_device(model_config.path, dtype, device, ops=ops,
+                                            config=model_config)
+        self.model = model
+        self.device = model.rt.device
+        self.dtype = model.rt.act_dtype
+        self.runner = make_runner(model, self.cache_config.num_blocks,
+                                  self.cache_config.block_size,
+                                  self.scheduler_config.max_num_seqs,
+                                  self.cache_config.gpu_memory_utilization)
+        self.num_blocks = self.runner.manager.num_pages
+        self.scheduler = Scheduler(self.scheduler_config, self.runner.manager, self.clock,
+                                   eos_token_id=model.spec.eos_token_id,
+                                   max_positions=model.spec.max_position_embeddings)
+        self.sampler = Sampler(model.rt.ops, self.device, seed)
+        self._req_counter = 0
+        self._draws: Dict[str, int] = {}
+        self.num_steps = 0
+
+    # -------------------------------------------------------------- intake
+    def add_request(self, prompt: Optional[str] = None,
+                    sampling_params: Optional[SamplingParams] = None,
+                    prompt_token_ids: Optional[List[int]] = None,
+                    request_id: Optional[str] = None, priority: int = 0) -> str:
+        """servelab/engine/engine.py:138-160."""
+        if prompt_token_ids is None:
+            if self.tokenizer is None or prompt is None:
+                raise ValueError("need prompt_token_ids, or a tokenizer + prompt")
+            prompt_token_ids = self.tokenizer.encode(prompt)
+        vocab = self.model.spec.vocab_size
+        bad = [t for t in prompt_token_ids if not 0 <= int(t) < vocab]
+        if bad:
+            raise ValueError(f"token id {bad[0]} is outside the vocabulary of {vocab}")
+        self._req_counter += 1
+        request_id = request_id or f"req-{self._req_counter}"
+        seq = Sequence(request_id, list(prompt_token_ids), sampling_params or SamplingParams(),
+                       priority=priority, arrival_time=self.clock(), number=self._req_counter)
+        self.scheduler.add_request(seq)
+        return request_id
+
+    def abort_request(self, request_id: str) -> bool:
+        return self.scheduler.abort_request(request_id)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    # ---------------------------------------------------------------- step
+    def step(self) -> List[RequestOutput]:
+        """One scheduler pass, one model step, one sampling call.  Returns the
+        requests that finished (or were aborted) in this step
+        (servelab/engine/engine.py:169-241)."""
+        plan = self.scheduler.schedule()
+        outputs = [RequestOutput.from_sequence(s, self._detokenize) for s in plan.aborted]
+        if plan.is_empty():
+            if not outputs and self.scheduler.has_unfinished():
+                raise RuntimeError("nothing can be scheduled although requests are unfinished")
+            return outputs
+        entries: List[StepEntry] = []
+        sampling: List[Sequence] = []
+        for ps in plan.prefills:                 # prompt portions first, then decode tokens
+            seq, start, n = ps.seq, ps.num_computed, ps.num_new_tokens
+            last = start + n == seq.prefill_target
+            entries.append(StepEntry(seq.request_id, seq.token_ids[start:start + n],
+                                     [n - 1] if last else []))
+            if last:
+                sampling.append(seq)
+            seq.num_computed_tokens = start + n
+        for seq in plan.decodes:
+            entries.append(StepEntry(seq.request_id, [seq.token_ids[-1]], [0]))
+            sampling.append(seq)
+            seq.num_computed_tokens = seq.get_len()      # this token's cache is written below
+        logits = self.runner.step(entries)
+        tokens = self.sampler.sample(
+            logits, [s.sampling_params for s in sampling], [s.number for s in sampling],
+            [s.num_output_tokens for s in sampling])
+        sampled = {s.request_id: t for s, t in zip(sampling, tokens)}
+        finished = self.scheduler.update_after_exec(sampled, now=self.clock())
+        self.num_steps += 1
+        return outputs + [RequestOutput.from_sequence(s, self._detokenize) for s in finished]
+
+    def _detokenize(self, token_ids: List[int]) -> str:
+        return "" if self.tokenizer is None else self.tokenizer.decode(token_ids)
+
+    # ------------------------------------------------------------ generate
+    def generate(self, prompts: List, sampling_params: Optional[SamplingParams] = None,
+                 verbose: bool = False) -> List[RequestOutput]:
+        """Offline generation; prompts are strings (needs a tokenizer) or lists
+        of token ids; outputs come back in input order
+        (servelab/engine/engine.py:249-270)."""
+        params = sampling_params or SamplingParams()
+        ids = []
+        for p in prompts:
+            ids.append(self.add_request(
+                prompt=p if isinstance(p, str) else None,
+                prompt_token_ids=None if isinstance(p, str) else list(p),
+                sampling_params=params))
+        results: Dict[str, RequestOutput] = {}
+        while self.has_unfinished():
+            for out in self.step():
+                results[out.request_id] = out
+            if verbose:
+                st = self.scheduler.stats()
+                print(f"[step] running={st['running']} waiting={st['waiting']} "
+                      f"cache={st['gpu_cache_usage']:.0%}")
+        return [results.get(i) for i in ids]
+
+    def stats(self) -> dict:
+        return {**self.scheduler.stats(), **self.runner.manager.stats(),
+                "num_blocks": self.num_blocks, "block_size": self.cache_config.block_size,
+                "dtype": str(self.dtype).replace("torch.", ""), "device": str(self.device),
+                "steps": self.num_steps}

@@ -1,0 +1,50 @@
+"""Logits -> tokens, on the device.
+
+Reference: ``Sampler`` (servelab/engine/sampler.py:10-45) handles rows one at a
+time on the host: temperature 0 is argmax; else softmax(logits / T), top-k
+(which ignores top-p) or top-p, multinomial from one engine-wide generator, or
+from a fresh generator per call when the request has a seed.  Here one kernel
+call samples all rows; a row's random stream is keyed by (seed, number of
+tokens the request has drawn), so it does not depend on the batch it shares.
+"""
+from typing import List, Sequence
+
+import torch
+
+
+def _mix(seed: int, number: int) -> int:
+    """A 63-bit key from the engine seed and the request's submission number."""
+    z = (seed * 0x9E3779B97F4A7C15 + (number + 1) * 0xBF58476D1CE4E5B9) & 0xFFFFFFFFFFFFFFFF
+    z ^= z >> 31
+    return z & 0x7FFFFFFFFFFFFFFF
+
+
+class Sampler:
+    def __init__(self, ops, device, seed: int = 0):
+        self.ops = ops
+        self.device = torch.device(device)
+        self.seed = int(seed)
+
+    def row_seed(self, params, number: int) -> int:
+        return int(params.seed) if params.seed >= 0 else _mix(self.seed, number)
+
+    def sample(self, logits: torch.Tensor, params: Sequence, numbers: Sequence[int],
+               draws: Sequence[int]) -> List[int]:
+        """``logits`` [B, V] float32; ``params[i]`` the SamplingParams of row i,
+        ``numbers[i]`` its request's submission number, ``draws[i]`` how many
+        tokens that request has sampled before."""
+        if logits.shape[0] == 0:
+            return []
+        if all(p.temperature == 0.0 for p in params):
+            return self.ops.argmax(logits).tolist()
+        host = torch.tensor(
+            [[p.temperature, p.top_p] for p in params], dtype=torch.float32)
+        ints = torch.tensor([[self.row_seed(p, n), d] for p, n, d in zip(params, numbers, draws)],
+                            dtype=torch.int64)
+        top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32)
+        temperature = host[:, 0].contiguous().to(self.device)
+        top_p = host[:, 1].contiguous().to(self.device)
+        seeds = ints[:, 0].contiguous().to(self.device)
+        counters = ints[:, 1].contiguous().to(self.device)
+        return self.ops.sample(logits, temperature, top_k.to(self.device), top_p, seeds,
+                               counters).tolist()

@@ -1,0 +1,128 @@
+"""The engine above the kernels (entry point, scheduler, step function, cache)
+with the kernels emulated on the CPU: greedy generation equals the plain
+implementation's however the work is cut (no GPU).  After the reference's
+tests/test_engine_smoke.py:57-134 and tests/test_speculative.py:41-49."""
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from emulated_ops import EmulatedOps
+from servelab_amd import CacheConfig, LLMEngine, SamplingParams, SchedulerConfig, load_config
+from servelab_amd.engine import ModelRunner, OutOfPages, StepEntry
+from servelab_amd.engine.session import load_model_on_device
+from tiny_configs import make_folder
+
+
+def make_engine(folder, num_blocks=64, max_batched=256, max_seqs=8, block_size=16):
+    return LLMEngine(load_config(folder), CacheConfig(block_size=block_size, num_blocks=num_blocks),
+                     SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched),
+                     device="cpu", dtype="float32", ops=EmulatedOps())
+
+
+PROMPTS = [list(range(10, 40)), [5, 9, 200, 31], list(range(300, 377)), [7]]
+
+
+@pytest.fixture(scope="module")
+def folder_and_plain(tmp_path_factory):
+    folder = make_folder(tmp_path_factory.mktemp("m"), "B", seed=21)
+    cfg, w = plain.load_folder(folder)
+    want = [plain.greedy_generate(cfg, w, p, 12) for p in PROMPTS]
+    return folder, want
+
+
+def test_greedy_generation_matches_plain(folder_and_plain):
+    folder, want = folder_and_plain
+    outs = make_engine(folder).generate(PROMPTS, SamplingParams.greedy(12))
+    assert [o.outputs[0].token_ids for o in outs] == want
+    assert all(o.finished and o.outputs[0].finish_reason == "length" for o in outs)
+    assert [o.prompt_token_ids for o in outs] == PROMPTS
+
+
+@pytest.mark.parametrize("max_batched,max_seqs", [(8, 8), (48, 2), (3, 4)])
+def test_any_cutting_gives_the_same_tokens(folder_and_plain, max_batched, max_seqs):
+    folder, want = folder_and_plain
+    eng = make_engine(folder, max_batched=max_batched, max_seqs=max_seqs)
+    outs = eng.generate(PROMPTS, SamplingParams.greedy(12))
+    assert [o.outputs[0].token_ids for o in outs] == want
+
+
+def test_preemption_keeps_outputs_whole(folder_and_plain):
+    folder, want = folder_and_plain
+    eng = make_engine(folder, num_blocks=9, max_batched=64)      # 144 tokens of cache for 4 requests
+    outs = eng.generate(PROMPTS, SamplingParams.greedy(12))
+    assert [o.outputs[0].token_ids for o in outs] == want
+    assert eng.stats()["num_preemptions_total"] > 0
+    assert sum(o.metrics["preemptions"] for o in outs) == eng.stats()["num_preemptions_total"]
+    eng.runner.manager.check()
+    assert eng.runner.manager.num_free_pages() == 9
+
+
+def test_running_requests_keep_the_invariant(folder_and_plain):
+    folder, _ = folder_and_plain
+    eng = make_engine(folder, max_batched=16)
+    for p in PROMPTS:
+        eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(5))
+    while eng.has_unfinished():
+        eng.step()
+        for s in eng.scheduler.running:               # tests/test_engine_smoke.py:113-127
+            if s.is_prefill_done():
+                assert s.num_computed_tokens == s.get_len() - 1
+            assert eng.runner.manager.length(s.request_id) == s.num_computed_tokens
+
+
+def test_eos_stops_and_stays_in_the_output(folder_and_plain):
+    folder, want = folder_and_plain
+    eng = make_engine(folder)
+    stop = want[0][3]
+    first = want[0].index(stop)
+    out = eng.generate([PROMPTS[0]], SamplingParams(temperature=0.0, max_tokens=12,
+                                                    stop_token_ids=(stop,)))[0]
+    assert out.outputs[0].token_ids == want[0][:first + 1] and out.outputs[0].finish_reason == "eos"
+
+
+def test_abort_and_oversize(folder_and_plain):
+    folder, _ = folder_and_plain
+    eng = make_engine(folder, num_blocks=4)
+    rid = eng.add_request(prompt_token_ids=PROMPTS[0], sampling_params=SamplingParams.greedy(4))
+    eng.step()
+    assert eng.abort_request(rid) and not eng.has_unfinished()
+    assert eng.runner.manager.num_free_pages() == 4
+    outs = eng.generate([list(range(100)), [1, 2, 3]], SamplingParams.greedy(2))
+    assert outs[0].outputs[0].finish_reason == "aborted" and outs[0].outputs[0].token_ids == []
+    assert outs[1].outputs[0].finish_reason == "length"
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request(prompt_token_ids=[1000])
+    with pytest.raises(ValueError, match="tokenizer"):
+        eng.add_request(prompt="text")
+
+
+def test_step_function_errors(folder_and_plain):
+    folder, _ = folder_and_plain
+    _, model = load_model_on_device(folder, "float32", "cpu", ops=EmulatedOps())
+    runner = ModelRunner(model, num_pages=2, page_size=16)
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("a", list(range(40)), [0])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.step([StepEntry("b", [1], [0]), StepEntry("b", [2], [0])])
+    with pytest.raises(ValueError, match="outside"):
+        runner.step([StepEntry("c", [1, 2], [2])])
+    runner.close("a"), runner.close("b"), runner.close("c")
+    out = runner.step([StepEntry("d", [1, 2, 3], [])])           # nothing wanted: no logits
+    assert out.shape == (0, 1000)
+    out = runner.step([StepEntry("d", [4], [0])])
+    assert out.shape == (1, 1000)
+    runner.manager.check()
+
+
+def test_cli_smoke(folder_and_plain, capsys, monkeypatch):
+    folder, want = folder_and_plain
+    import servelab_amd.cli as cli
+    import servelab_amd.engine.llm_engine as le
+    real = le.load_model_on_device
+    monkeypatch.setattr(le, "load_model_on_device",
+                        lambda f, dtype, device, ops=None, config=None:
+                        real(f, "float32", "cpu", ops=EmulatedOps(), config=config))
+    assert cli.main(["--model", folder, "--max-tokens", "12", "--temperature", "0",
+                     "--num-blocks", "32"]) == 0
+    printed = capsys.readouterr().out
+    assert f"[req-1] finish=length -> {want[0]}" in printed and "stats:" in printed

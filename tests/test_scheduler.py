@@ -1,0 +1,241 @@
+"""Scheduler decisions with a fake executor and a fake clock (no GPU), after
+the reference's tests/test_scheduler.py:29-154."""
+import pytest
+
+from servelab_amd.cache import CacheManager
+from servelab_amd.config import SchedulerConfig
+from servelab_amd.engine import SamplingParams, Scheduler, Sequence, SequenceStatus
+from servelab_amd.parts import PagedKVSpec
+
+
+class FakeClock:
+    def __init__(self):
+        self.t = 0.0
+
+    def __call__(self):
+        return self.t
+
+
+class Driver:
+    """Executes whatever the scheduler plans: advances the computed counts,
+    'samples' token 7, and checks the invariants after every step."""
+
+    def __init__(self, num_pages=16, page_size=4, max_batched=32, max_seqs=8, policy="fcfs",
+                 chunked=True, eos=-1, max_positions=None, window=None):
+        self.clock = FakeClock()
+        specs = {0: PagedKVSpec(1, 16, None)}
+        if window:
+            specs[1] = PagedKVSpec(1, 16, window)
+        self.manager = CacheManager(specs, num_pages, page_size, num_state_slots=max_seqs)
+        self.scheduler = Scheduler(
+            SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched,
+                            chunked_prefill=chunked, policy=policy),
+            self.manager, self.clock, eos_token_id=eos, max_positions=max_positions)
+        self.finished, self.aborted, self.n, self.plans = [], [], 0, []
+        self.token = 7
+
+    def submit(self, rid, prompt_len, output_len, priority=0, ignore_eos=True):
+        self.n += 1
+        seq = Sequence(rid, list(range(1000, 1000 + prompt_len)),
+                       SamplingParams(max_tokens=output_len, ignore_eos=ignore_eos),
+                       priority=priority, arrival_time=self.clock.t, number=self.n)
+        self.scheduler.add_request(seq)
+        return seq
+
+    def step(self):
+        out = self.scheduler.schedule()
+        self.plans.append(out)
+        sampled = {}
+        assert out.num_batched_tokens <= max(self.scheduler.cfg.max_num_batched_tokens, 1) \
+            or not self.scheduler.cfg.chunked_prefill
+        for ps in out.prefills:
+            assert ps.num_computed == ps.seq.num_computed_tokens
+            ps.seq.num_computed_tokens += ps.num_new_tokens
+            self.manager.commit(ps.seq.request_id, ps.seq.num_computed_tokens)
+            if ps.seq.is_prefill_done():
+                sampled[ps.seq.request_id] = self.token
+        for seq in out.decodes:
+            seq.num_computed_tokens = seq.get_len()
+            self.manager.commit(seq.request_id, seq.num_computed_tokens)
+            sampled[seq.request_id] = self.token
+        self.clock.t += 0.01
+        self.finished += self.scheduler.update_after_exec(sampled)
+        self.aborted += out.aborted
+        self.manager.check()
+        # servelab's invariant (tests/test_engine_smoke.py:113-127)
+        for s in self.scheduler.running:
+            if s.is_prefill_done():
+                assert s.num_computed_tokens == s.get_len() - 1
+        assert set(self.manager.lengths) == {s.request_id for s in self.scheduler.running}
+        return out
+
+    def run(self, max_steps=2000):
+        steps = 0
+        while self.scheduler.has_unfinished():
+            steps += 1
+            assert steps < max_steps, "scheduler makes no progress"
+            out = self.step()
+            assert not out.is_empty() or out.aborted
+        assert self.manager.num_free_pages() == self.manager.num_pages
+        return steps
+
+
+def test_all_finish_with_exact_counts():
+    d = Driver()
+    for i in range(5):
+        d.submit(f"r{i}", 10, 5)
+    d.run()
+    assert {s.request_id: s.num_output_tokens for s in d.finished} == {f"r{i}": 5 for i in range(5)}
+    assert all(s.status == SequenceStatus.FINISHED_LENGTH for s in d.finished)
+
+
+def test_portions_respect_the_budget():
+    d = Driver(max_batched=8)
+    d.submit("big", 40, 1)
+    out = d.scheduler.schedule()
+    assert len(out.prefills) == 1 and out.prefills[0].num_new_tokens == 8
+    assert out.prefills[0].num_computed == 0
+
+
+def test_decodes_first_then_portions_share_the_budget():
+    d = Driver(max_batched=16, num_pages=64)
+    d.submit("a", 6, 4)
+    d.step()                               # a: whole prompt, first token sampled
+    d.submit("b", 40, 2)
+    out = d.step()
+    assert [s.request_id for s in out.decodes] == ["a"]
+    assert out.prefills[0].seq.request_id == "b" and out.prefills[0].num_new_tokens == 15
+    out = d.step()
+    assert out.prefills[0].num_computed == 15 and out.prefills[0].num_new_tokens == 15
+
+
+def test_several_prompts_are_cut_in_one_step():
+    d = Driver(max_batched=20, num_pages=64)
+    d.submit("a", 12, 1)
+    d.submit("b", 12, 1)
+    out = d.scheduler.schedule()
+    assert [(p.seq.request_id, p.num_new_tokens) for p in out.prefills] == [("a", 12), ("b", 8)]
+
+
+def test_fcfs_and_priority_order():
+    d = Driver(max_batched=12)
+    for i in range(4):
+        d.submit(f"r{i}", 20, 1)
+    assert d.scheduler.schedule().prefills[0].seq.request_id == "r0"
+    d = Driver(max_batched=12, policy="priority")
+    d.submit("low", 20, 1, priority=5)
+    d.submit("high", 20, 1, priority=0)
+    assert d.scheduler.schedule().prefills[0].seq.request_id == "high"
+
+
+def test_request_numbers_not_id_strings_break_ties():
+    d = Driver(max_batched=4)
+    d.submit("req-10", 4, 1)
+    d.submit("req-2", 4, 1)
+    assert d.scheduler.schedule().prefills[0].seq.request_id == "req-10"
+
+
+def test_preemption_when_pages_run_out():
+    # 8 pages of 4 tokens; four requests need 18 tokens each
+    d = Driver(num_pages=8, page_size=4, max_batched=64, max_seqs=4)
+    seqs = [d.submit(f"r{i}", 8, 10) for i in range(4)]
+    d.run()
+    assert len(d.finished) == 4
+    assert sum(s.metrics.num_preemptions for s in d.finished) > 0
+    # outputs survive a preemption: ten tokens each, the prompt untouched
+    assert all(s.num_output_tokens == 10 and s.num_prompt_tokens == 8 for s in seqs)
+    # the victim is the request that came last, and it goes to the front of the queue
+    first = next(p for p in d.plans if p.preempted)
+    assert first.preempted[0] == "r3" or first.preempted[0] == "r2"
+
+
+def test_the_victim_is_the_last_in_policy_order_and_requeues_first():
+    d = Driver(num_pages=4, page_size=4, max_batched=64, max_seqs=4)
+    a = d.submit("a", 7, 8)
+    b = d.submit("b", 7, 8)
+    d.step()                         # both prompts (2 pages each), first tokens
+    d.step()                         # position 7 still fits the second page
+    out = d.step()                   # a needs position 8 -> a third page: b is evicted
+    assert out.preempted == ["b"] and [s.request_id for s in out.decodes] == ["a"]
+    assert b.status == SequenceStatus.WAITING and d.scheduler.waiting[0] is b
+    assert b.num_computed_tokens == 0 and b.prefill_target == 9 and b.num_prompt_tokens == 7
+    d.run()
+    assert a.num_output_tokens == 8 and b.num_output_tokens == 8
+
+
+def test_a_single_request_too_big_for_what_is_left_preempts_itself_then_aborts_or_finishes():
+    d = Driver(num_pages=3, page_size=4, max_batched=64, max_seqs=2)
+    s = d.submit("a", 10, 8)         # grows to 18 tokens > 12
+    d.run()
+    assert s.status == SequenceStatus.FINISHED_ABORTED and d.aborted == [s]
+    assert s.metrics.num_preemptions == 1
+
+
+def test_oversize_and_overlong_requests_abort_at_admission():
+    d = Driver(num_pages=4, page_size=4, max_positions=64)
+    big = d.submit("big", 17, 2)
+    ok = d.submit("ok", 8, 2)
+    out = d.step()
+    assert out.aborted == [big] and big.status == SequenceStatus.FINISHED_ABORTED
+    assert out.prefills[0].seq is ok
+    d = Driver(num_pages=64, page_size=4, max_positions=12)
+    assert d.submit("long", 13, 1) and d.step().aborted[0].request_id == "long"
+    s = d.submit("edge", 10, 20)
+    d.run()
+    assert s.get_len() == 12 and s.status == SequenceStatus.FINISHED_LENGTH
+
+
+def test_head_of_line_blocking_and_max_num_seqs():
+    d = Driver(num_pages=6, page_size=4, max_batched=64, max_seqs=8)
+    d.submit("a", 16, 1)
+    d.submit("b", 12, 1)             # does not fit beside a
+    d.submit("c", 2, 1)              # would fit, but waits behind b
+    out = d.scheduler.schedule()
+    assert [p.seq.request_id for p in out.prefills] == ["a"]
+    d = Driver(max_seqs=2, max_batched=64)
+    for i in range(5):
+        d.submit(f"r{i}", 4, 3)
+    assert len(d.scheduler.schedule().prefills) == 2
+    d.run()
+
+
+def test_eos_and_stop_tokens():
+    d = Driver(eos=7)
+    s = d.submit("a", 4, 10, ignore_eos=False)
+    t = d.submit("b", 4, 3, ignore_eos=True)
+    d.run()
+    assert s.status == SequenceStatus.FINISHED_EOS and s.output_token_ids == [7]
+    assert t.status == SequenceStatus.FINISHED_LENGTH and t.num_output_tokens == 3
+
+
+def test_abort():
+    d = Driver()
+    d.submit("x", 10, 10)
+    d.submit("y", 10, 10)
+    d.step()
+    assert d.scheduler.abort_request("x") and d.scheduler.abort_request("y")
+    assert not d.scheduler.abort_request("z")
+    assert not d.scheduler.has_unfinished()
+    d.manager.check()
+    assert d.manager.num_free_pages() == 16
+
+
+def test_unchunked_mode_runs_whole_prompts_and_holds_decodes_while_any_waits():
+    d = Driver(chunked=False, max_batched=8, num_pages=64, max_seqs=1)
+    d.submit("a", 20, 3)
+    d.submit("b", 20, 2)
+    out = d.step()
+    assert out.prefills[0].num_new_tokens == 20
+    out = d.scheduler.schedule()
+    assert out.is_empty()            # b waits, max_seqs is 1: servelab/engine/scheduler.py:177
+    d.scheduler.abort_request("b")
+    d.run()
+
+
+def test_window_groups_keep_few_pages_during_long_decoding():
+    d = Driver(num_pages=12, page_size=4, max_batched=64, window=8)
+    s = d.submit("a", 6, 40)
+    d.run()
+    assert s.num_output_tokens == 40
+    assert d.manager.page_groups[1].allocator.high_water <= 4
+    assert d.manager.page_groups[0].allocator.high_water == 12
