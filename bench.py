@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+Default run: the layer sizes of the Qwen2.5-7B shape with random weights,
+bfloat16, a batch of 8 requests whose context ends at 4,096 tokens, 16-token
+pages.  A "step" is one decode step of the whole batch through the engine's
+step function and greedy sampling; ``value`` is decoded tokens per second.
+The same line carries a 2,048-token prefill, the decode step's HBM roofline
+(every weight the step uses once plus the cache of the live requests, over its
+time) and decode at batch 1 and 64.
+
+The reference has no recorded numbers; its harness measures the same kind of
+quantities over synthetic random-id prompts (servelab/bench/benchmark_serving.py:102-121,
+servelab/bench/datasets.py:8-20, 10 warm-up + 50 timed iterations with device
+events in servelab/bench/kernel_bench.py:12-23).
+
+    python bench.py --gpus 1 --steps 20 --warmup 3
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN25_7B = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=28,
+    hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
+    intermediate_size=18944, vocab_size=152064, rope_theta=1000000.0, rms_norm_eps=1e-6,
+    tie_word_embeddings=False, use_sliding_window=False, max_position_embeddings=32768,
+    torch_dtype="bfloat16", eos_token_id=151645)
+
+
+class RandomCheckpoint:
+    """Seeded random tensors made on the device when a part asks for them, so
+    that a 15 GB model needs no file: N(0, 0.02), norm gains 1 + N(0, 0.05)."""
+
+    def __init__(self, specs, seed, device, dtype):
+        self.specs, self.seed, self.device, self.dtype = specs, seed, device, dtype
+        self.order = {n: i for i, n in enumerate(specs)}
+
+    def shapes(self):
+        return {n: s.shape for n, s in self.specs.items()}
+
+    def get(self, name):
+        import torch
+        spec = self.specs[name]
+        gen = torch.Generator(device=self.device)
+        gen.manual_seed(self.seed * 100003 + self.order[name])
+        t = torch.randn(spec.shape, generator=gen, device=self.device, dtype=torch.float32)
+        t = 1.0 + 0.05 * t if spec.init == "gain" else 0.02 * t
+        return t.to(self.dtype) if len(spec.shape) > 1 else t
+
+
+def build(args):
+    import torch
+    import servelab_amd  # noqa: F401
+    from servelab_amd import Qwen2Config
+    from servelab_amd.engine.session import make_runtime, resolve_dtype
+    from servelab_amd.parts import DecoderModel, build_model_spec
+
+    raw = dict(QWEN25_7B)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    cfg = Qwen2Config.from_hf(raw)
+    dtype = resolve_dtype(args.dtype)
+    rt = make_runtime(dtype, "cuda:0")
+    model = DecoderModel(build_model_spec(cfg), rt)
+    model.load(RandomCheckpoint(model.spec.param_specs(), args.seed, rt.device, dtype))
+    torch.cuda.synchronize()
+    return cfg, model, full_layers
+
+
+def weight_bytes_per_step(cfg, itemsize):
+    """Bytes of weights one decode step reads: every matrix, bias and gain of
+    every layer once, the final gain and the head; of the embedding only the
+    batch's rows (counted with the activations, not here)."""
+    h, d = cfg.hidden_size, cfg.head_dim
+    qkv = (cfg.num_heads + 2 * cfg.num_kv_heads) * d
+    per_layer = (qkv * h + cfg.num_heads * d * h + 3 * h * cfg.intermediate_size) * itemsize \
+        + (qkv + 2 * h) * 4
+    return cfg.num_layers * per_layer + h * 4 + cfg.vocab_size * h * itemsize
+
+
+def cache_bytes_per_token(cfg, itemsize):
+    return 2 * cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * itemsize
+
+
+def prefill_flops(cfg, T):
+    h, d = cfg.hidden_size, cfg.head_dim
+    qkv = (cfg.num_heads + 2 * cfg.num_kv_heads) * d
+    linear = cfg.num_layers * (qkv * h + cfg.num_heads * d * h + 3 * h * cfg.intermediate_size)
+    attn = 2 * cfg.num_heads * d * T * T * cfg.num_layers          # causal half of 4 T^2 nh D
+    return 2 * T * linear + attn + 2 * cfg.vocab_size * h
+
+
+def fill_cache(runner, requests, ctx, seed):
+    """Open ``requests`` with ``ctx`` tokens of random K/V already cached."""
+    import torch
+    gen = torch.Generator(device=runner.rt.device)
+    gen.manual_seed(seed)
+    for t in runner.pool.k + runner.pool.v:
+        for s in range(t.shape[0]):                   # stream by stream: bounded temporaries
+            t[s].copy_(torch.randn(t[s].shape, generator=gen, device=t.device,
+                                   dtype=torch.float32).mul_(0.5))
+    for r in requests:
+        assert runner.open(r) and runner.manager.grow(r, ctx)
+        runner.manager.commit(r, ctx)
+
+
+def time_decode(model, batch, ctx_end, steps, warmup, page, seed=0):
+    """Median-free, contract timing: ``warmup`` untimed steps, then exactly
+    ``steps`` steps between two synchronisations.  The context of every request
+    reaches ``ctx_end`` at the last step."""
+    import torch
+    from servelab_amd.engine import ModelRunner, StepEntry
+    total = warmup + steps
+    start = ctx_end - total
+    pages = batch * (-(-ctx_end // page)) + 8
+    runner = ModelRunner(model, pages, page, max_num_seqs=batch)
+    requests = [f"b{i}" for i in range(batch)]
+    fill_cache(runner, requests, start, seed)
+    vocab = model.spec.vocab_size
+    tokens = torch.randint(0, vocab, (batch,), generator=torch.Generator().manual_seed(seed)).tolist()
+    ops = model.rt.ops
+
+    def one_step(toks):
+        logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(requests, toks)])
+        return ops.argmax(logits).tolist()             # the engine needs the token on the host
+
+    for _ in range(warmup):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert runner.manager.length(requests[0]) == ctx_end
+    mean_ctx = ctx_end - (steps + 1) / 2.0
+    del runner
+    torch.cuda.empty_cache()
+    return dt / steps, mean_ctx
+
+
+def time_prefill(model, T, page, repeats, max_chunk, seed=1):
+    """A prompt of T tokens from an empty cache, in portions of at most
+    ``max_chunk`` tokens (one portion when T fits)."""
+    import torch
+    from servelab_amd.engine import ModelRunner, StepEntry
+    runner = ModelRunner(model, -(-T // page) + 8, page, max_num_seqs=4)
+    vocab = model.spec.vocab_size
+    toks = torch.randint(0, vocab, (T,), generator=torch.Generator().manual_seed(seed)).tolist()
+    ops = model.rt.ops
+
+    def once(tag):
+        pos = 0
+        while pos < T:
+            n = min(max_chunk, T - pos)
+            logits = runner.step([StepEntry(tag, toks[pos:pos + n], [n - 1] if pos + n == T else [])])
+            pos += n
+        first = ops.argmax(logits).tolist()
+        runner.close(tag)
+        return first
+
+    once("w")
+    torch.cuda.synchronize()
+    best = float("inf")
+    for i in range(repeats):
+        t0 = time.perf_counter()
+        once(f"p{i}")
+        torch.cuda.synchronize()
+        best = min(best, time.perf_counter() - t0)
+    del runner
+    torch.cuda.empty_cache()
+    return best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--prefill-chunk", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
+        return 2
+
+    cfg, model, full_layers = build(args)
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    itemsize = 2 if short == "bf16" else 4
+    page = args.block_size
+
+    step_s, mean_ctx = time_decode(model, args.batch, args.context, args.steps, args.warmup, page)
+    value = args.batch / step_s
+    step_bytes = weight_bytes_per_step(cfg, itemsize) + \
+        args.batch * mean_ctx * cache_bytes_per_token(cfg, itemsize)
+    achieved = step_bytes / step_s / 1e9
+
+    line = {
+        "metric": "decode_tokens_per_s", "value": round(value, 2), "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short,
+        "data": "synthetic: seeded random weights, uniform random token ids, cache filled with "
+                "random keys and values up to the context",
+        "config": {
+            "model": "Qwen2.5-7B shape", "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "none", "layers": cfg.num_layers, "layers_of_shape": full_layers,
+            "hidden_size": cfg.hidden_size, "num_heads": cfg.num_heads,
+            "num_kv_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "page_size": page, "prefill_tokens": args.prefill_tokens,
+            "decode_mean_context": round(mean_ctx, 1), "sampling": "greedy",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
+    }
+    if not args.no_prefill:
+        T = args.prefill_tokens
+        pre_s = time_prefill(model, T, page, repeats=3, max_chunk=args.prefill_chunk)
+        line["prefill"] = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
+                           "frac": round(prefill_flops(cfg, T) / pre_s / PEAK_FLOPS[short], 4)}
+    if not args.no_points:
+        points = {}
+        for b in (1, 64):
+            s, _ = time_decode(model, b, args.context, max(5, args.steps // 2), 2, page)
+            points[f"decode_b{b}"] = round(b / s, 2)
+        line["points"] = points
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
