@@ -162,4 +162,7 @@ def all_units(head_dims=(16, 32, 64, 128)) -> List[Unit]:
     for dtype in ("bfloat16", "float32"):
         for stem in DEFAULT_STEMS:
             units.append(unit(stem, dtype))
+    for d in head_dims:
+        if d % 32 == 0:
+            units.append(unit("attention_mfma", "bfloat16", SL_HEAD_DIM=d))
     return units

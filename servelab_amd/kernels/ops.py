@@ -46,6 +46,7 @@ class HipOps:
                      for stem in build.DEFAULT_STEMS}
         self._fn = {}
         self._bias_cache = {}
+        self.use_mfma_attention = True
 
     # ------------------------------------------------------------ plumbing
     def _call(self, stem, name, *args):
@@ -203,14 +204,69 @@ class HipOps:
         if S != batch.num_seqs:
             raise KernelError(f"block tables hold {S} sequences, the batch {batch.num_seqs}")
         if batch.max_ctx_len > max_pages * page_size:
-            raise KernelError(f"context {batch.max_ctx_len} exceeds the block table "
-                              f"({max_pages} pages of {page_size})")
+            raise KernelError("block table is shorter than the context")
         out = self._new((T, nh * D))
+        if self._mfma_attention_fits(D, nh // nkv, max_pages, page_size, batch):
+            self._attention_mfma(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                                 batch, scale, window, out)
+            return out
         self._call("attention", "sl_attention_general", _p(qkv), (nh + 2 * nkv) * D, _p(k_cache),
                    _p(v_cache), _p(block_tables), max_pages, _p(batch.tok_seq),
                    _p(batch.positions), T, nh, nkv, D, page_size, _c_float(scale),
                    int(window or 0), _p(out))
         return out
+
+    TARGET_WAVES = 1024           # wavefronts a decode launch aims for when it splits the context
+
+    def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
+        """The matrix-core kernels take bfloat16, head sizes that are multiples
+        of 32, and block tables that cover the context rounded up to a whole
+        32-key block; everything else goes to the general kernel."""
+        if self.act_dtype != torch.bfloat16 or not self.use_mfma_attention:
+            return False
+        if D % 32 or D > 256 or group > 64:
+            return False
+        return max_pages * page_size >= -(-batch.max_ctx_len // 32) * 32
+
+    def _attention_lib(self, D):
+        key = ("attention_mfma", D)
+        lib = self._lib.get(key)
+        if lib is None:
+            lib = build.load(build.unit("attention_mfma", "bfloat16", SL_HEAD_DIM=D))
+            self._lib[key] = lib
+        return key
+
+    def _attention_mfma(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables, batch,
+                        scale, window, out):
+        lib = self._attention_lib(D)
+        self._check(batch.cu_q, torch.int32, (batch.num_seqs + 1,), "cu_q")
+        max_pages = block_tables.shape[1]
+        n_pre, n_pre_tok = batch.num_prefill_seqs, batch.num_prefill_tokens
+        n_dec = batch.num_seqs - n_pre
+        if n_dec and n_pre_tok + n_dec != batch.num_tokens:
+            raise KernelError("single-token sequences must come last in the batch")
+        common = (_p(qkv), (nh + 2 * nkv) * D, _p(k_cache), _p(v_cache), _p(block_tables),
+                  max_pages, _p(batch.cu_q), _p(batch.positions))
+        tail = (nh, nkv, D, page_size, _c_float(scale), int(window or 0))
+        name = f"sl_attention_mfma@{D}"
+        if name not in self._fn:
+            fn = self._lib[lib].sl_attention_mfma
+            fn.restype = ctypes.c_char_p
+            self._fn[name] = fn
+        if n_pre:
+            self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, 1, _p(out),
+                       None, None, 0, 0)
+        if n_dec:
+            blocks = -(-batch.max_ctx_len // 32)
+            if window:
+                blocks = min(blocks, -(-int(window) // 32) + 1)
+            nsplit = max(1, min(blocks // 2, -(-self.TARGET_WAVES // (n_dec * nkv))))
+            part_o = part_ml = None
+            if nsplit > 1:
+                part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
+                part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
+            self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, _p(out),
+                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0)
 
     # ------------------------------------------------------------- sampling
     def argmax(self, logits):

@@ -178,7 +178,8 @@ def make_attention_case(dt, nh, nkv, D, page, seqs, seed=0):
         cu_q=torch.tensor(cu, dtype=torch.int32).cuda(),
         ctx_len=torch.tensor([c for c, _ in seqs], dtype=torch.int32).cuda(),
         max_ctx_len=max(c for c, _ in seqs), max_q_len=max(q for _, q in seqs),
-        num_prefill_seqs=sum(1 for _, q in seqs if q > 1))
+        num_prefill_seqs=sum(1 for _, q in seqs if q > 1),
+        num_prefill_tokens=sum(q for _, q in seqs if q > 1))
     return qkv, kc, vc, tables.cuda(), batch
 
 
@@ -186,7 +187,8 @@ ATTN_TOL = {torch.float32: 2e-5, torch.bfloat16: 2 ** -7}
 
 
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (8, 1, 32, 16), (7, 7, 48, 32),
-                                           (28, 4, 128, 16), (6, 2, 256, 64), (5, 5, 80, 16)])
+                                           (28, 4, 128, 16), (6, 2, 256, 64), (5, 5, 80, 16),
+                                           (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16)])
 @pytest.mark.parametrize("window", [None, 16, 50])
 def test_paged_attention(both, nh, nkv, D, page, window):
     ops, emu, dt = both
