@@ -219,35 +219,41 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const AttnParams P) 
   }
 }
 
-// out[row, head, :] = sum_j w_j o_j / sum_j w_j l_j,  w_j = exp(m_j - max m)
+// out[row, head, :] = sum_j w_j o_j / sum_j w_j l_j,  w_j = exp(m_j - max m).
+// One wavefront per (row, head); lane j takes split j's (m, l), so nsplit <= 64;
+// then the lanes split the channels and sum the partial outputs with the loads
+// of eight splits in flight at a time.
 __global__ __launch_bounds__(64) void attention_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int nsplit, int nh,
     int part_row0, __bf16* __restrict__ out) {
-  const int r = blockIdx.x, h = blockIdx.y;
+  __shared__ float ws[64];
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)r * nh + h) * nsplit;
-  float mx = -INFINITY;
-  for (int j = 0; j < nsplit; ++j) mx = fmaxf(mx, part_ml[(base + j) * 2]);
-  float denom = 0.f;
-  float acc[(D + 63) / 64];
-#pragma unroll
-  for (int i = 0; i < (D + 63) / 64; ++i) acc[i] = 0.f;
-  for (int j = 0; j < nsplit; ++j) {
-    const float m = part_ml[(base + j) * 2];
-    if (m == -INFINITY) continue;
-    const float w = __expf(m - mx);
-    denom += w * part_ml[(base + j) * 2 + 1];
-#pragma unroll
-    for (int i = 0; i < (D + 63) / 64; ++i) {
-      const int d = threadIdx.x + 64 * i;
-      if (d < D) acc[i] += w * part_o[(base + j) * D + d];
-    }
+  float m = -INFINITY, l = 0.f;
+  if (lane < nsplit) {
+    m = part_ml[(base + lane) * 2];
+    l = part_ml[(base + lane) * 2 + 1];
   }
+  const float mx = wave_max(m);
+  const float w = m == -INFINITY ? 0.f : __expf(m - mx);
+  const float denom = wave_sum(w * l);
+  ws[lane] = w;
+  __syncthreads();
   const float inv = 1.f / denom;
+  const float* po = part_o + base * D;
   __bf16* o = out + ((size_t)(part_row0 + r) * nh + h) * D;
+  for (int d = lane; d < D; d += 64) {
+    float acc = 0.f;
+    int j = 0;
+    for (; j + 8 <= nsplit; j += 8) {
+      float v[8];
 #pragma unroll
-  for (int i = 0; i < (D + 63) / 64; ++i) {
-    const int d = threadIdx.x + 64 * i;
-    if (d < D) o[d] = (__bf16)(acc[i] * inv);
+      for (int u = 0; u < 8; ++u) v[u] = po[(size_t)(j + u) * D + d];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc += ws[j + u] * v[u];
+    }
+    for (; j < nsplit; ++j) acc += ws[j] * po[(size_t)j * D + d];
+    o[d] = (__bf16)(acc * inv);
   }
 }
 
@@ -280,6 +286,7 @@ extern "C" const char* sl_attention_mfma(
     SL_CHECK(part_o != nullptr && part_ml != nullptr && part_rows == num_seqs,
              "attention_mfma: a split launch needs partial buffers for its rows");
     SL_CHECK(g <= 64, "attention_mfma: more than 64 query heads per kv head");
+    SL_CHECK(nsplit <= 64, "attention_mfma: at most 64 splits of the context");
     const dim3 grid(nsplit, nkv, num_seqs);
     if (g <= 16) attention_mfma_kernel<1, true><<<grid, 64, 0, stream>>>(P);
     else if (g <= 32) attention_mfma_kernel<2, true><<<grid, 64, 0, stream>>>(P);

@@ -147,3 +147,116 @@ extern "C" const char* sl_gemm_tiled(const void* x, const void* w, const float* 
                                               out_f32);
   return sl_launch_status();
 }
+
+// ------------------------------------------------ few rows on the matrix cores
+#if !defined(SL_F32)
+// y[M, N] for M <= 64 in bfloat16: bound by streaming W from HBM once.
+// A workgroup of 8 wavefronts owns 16 * NT columns of y (rows of W); each
+// wavefront takes an eighth of K, so that every row of W is read in long
+// contiguous runs and every wavefront has many loads in flight at once; the
+// eight partial tiles are summed through LDS.  Per 32 values of k one
+// mfma 16x16x32 per (16 rows of W) x (16 rows of x): A = W, B = x; the rows of
+// x are loaded once per k-step and used for all NT tiles of W.  Rows beyond M
+// or N repeat the last row and are not stored; k-steps beyond the wavefront's
+// share are loaded from its last step and zeroed, so the loop has no serial tail.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 load_stream(const __bf16* p) {
+  // W is read once per call: a non-temporal load keeps it from displacing x in the caches
+  const i32x4 v = __builtin_nontemporal_load((const i32x4*)p);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+template <int MB, int WAVES, bool NT_LOAD>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
+    const __bf16* __restrict__ x, const __bf16* __restrict__ w, const float* __restrict__ bias,
+    void* __restrict__ y, int M, int N, int K, int out_f32) {
+  constexpr int U = 8;
+  __shared__ f32x4 red[WAVES][MB][64];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int KT = K / 32;
+  const int ks0 = (int)((long long)KT * wave / WAVES), ks1 = (int)((long long)KT * (wave + 1) / WAVES);
+  const int nrow = n0 + i < N ? n0 + i : N - 1;
+  const __bf16* wp = w + (size_t)nrow * K + 8 * gq;
+  const __bf16* xp[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int m = 16 * b + i < M ? 16 * b + i : M - 1;
+    xp[b] = x + (size_t)m * K + 8 * gq;
+  }
+  f32x4 acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int ks = ks0;
+  for (; ks + U <= ks1; ks += U) {
+    bf16x8 a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      a[u] = NT_LOAD ? load_stream(wp + 32 * (size_t)(ks + u)) : *(const bf16x8*)(wp + 32 * (size_t)(ks + u));
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const bf16x8 bv = *(const bf16x8*)(xp[b] + 32 * (size_t)(ks + u));
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[b], 0, 0, 0);
+      }
+  }
+  for (; ks < ks1; ++ks) {
+    const bf16x8 a = NT_LOAD ? load_stream(wp + 32 * (size_t)ks) : *(const bf16x8*)(wp + 32 * (size_t)ks);
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const bf16x8 bv = *(const bf16x8*)(xp[b] + 32 * (size_t)ks);
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bv, acc[b], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < MB; ++b) red[wave][b][lane] = acc[b];
+  __syncthreads();
+  // lane (m_local + 16 (n_local / 4)) holds y[m_local, n_local] in element n_local % 4
+  for (int idx = threadIdx.x; idx < MB * 256; idx += WAVES * 64) {
+    const int b = idx / 256, rem = idx % 256, m_local = rem / 16, n_local = rem % 16;
+    const int m = 16 * b + m_local, n = n0 + n_local;
+    if (m < M && n < N) {
+      float s = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) s += red[wv][b][m_local + 16 * (n_local / 4)][n_local % 4];
+      if (bias != nullptr) s += bias[n];
+      if (out_f32) ((float*)y)[(size_t)m * N + n] = s;
+      else ((__bf16*)y)[(size_t)m * N + n] = (__bf16)s;
+    }
+  }
+}
+
+template <int MB>
+static const char* launch_skinny(int variant, const __bf16* x, const __bf16* w, const float* bias,
+                                 void* y, int M, int N, int K, int out_f32, hipStream_t stream) {
+  const dim3 grid((N + 15) / 16);
+  switch (variant) {
+    case 1: gemm_skinny_kernel<MB, 8, true><<<grid, 512, 0, stream>>>(x, w, bias, y, M, N, K, out_f32); break;
+    case 2: gemm_skinny_kernel<MB, 4, false><<<grid, 256, 0, stream>>>(x, w, bias, y, M, N, K, out_f32); break;
+    case 3: gemm_skinny_kernel<MB, 16, false><<<grid, 1024, 0, stream>>>(x, w, bias, y, M, N, K, out_f32); break;
+    case 4: gemm_skinny_kernel<MB, 4, true><<<grid, 256, 0, stream>>>(x, w, bias, y, M, N, K, out_f32); break;
+    default: gemm_skinny_kernel<MB, 8, false><<<grid, 512, 0, stream>>>(x, w, bias, y, M, N, K, out_f32);
+  }
+  return sl_launch_status();
+}
+
+extern "C" const char* sl_gemm_skinny(const void* x, const void* w, const float* bias, void* y,
+                                      int M, int N, int K, int out_f32, int nt,
+                                      hipStream_t stream) {
+  SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
+  SL_CHECK(M <= 64, "gemm_skinny: at most 64 rows");
+  SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
+  SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
+           "gemm_skinny: x and W must be 16-byte aligned");
+  if (M == 0) return nullptr;
+  const __bf16* xx = (const __bf16*)x;
+  const __bf16* ww = (const __bf16*)w;
+  if (M <= 16) return launch_skinny<1>(nt, xx, ww, bias, y, M, N, K, out_f32, stream);
+  if (M <= 32) return launch_skinny<2>(nt, xx, ww, bias, y, M, N, K, out_f32, stream);
+  return launch_skinny<4>(nt, xx, ww, bias, y, M, N, K, out_f32, stream);
+}
+#endif

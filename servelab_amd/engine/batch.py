@@ -57,11 +57,29 @@ class StepBatch:
     host_state_slots: List[int] = field(default_factory=list)
 
 
-def pack_batch(entries: List[StepEntry], starts: List[int], rows: List[int], manager, device,
-               pad_pages_to: int = 8) -> StepBatch:
-    """Build the batch of ``entries`` (already ordered: multi-token first) whose
+@dataclass
+class BatchArrays:
+    """A step's metadata on the host: one flat int32 array and where each piece
+    lies in it.  The layout depends only on (tokens, sequences, rows, pages per
+    table), so a captured graph can be fed by overwriting its buffer."""
+    flat: np.ndarray
+    offsets: List[int]
+    sizes: List[int]
+    group_pages: List[int]
+    q_lens: List[int]
+    starts: List[int]
+    requests: List[Hashable]
+    state_slots: List[int]
+    num_rows: int
+    max_ctx_len: int
+
+
+def build_arrays(entries: List[StepEntry], starts: List[int], rows: List[int], manager,
+                 pad_pages_to: int = 8, fixed_pages: int = 0) -> BatchArrays:
+    """The arrays of ``entries`` (already ordered: multi-token first) whose
     requests have ``starts[i]`` tokens cached and room for the new ones;
-    ``rows`` are the packed rows whose logits are wanted."""
+    ``rows`` are the packed rows whose logits are wanted.  ``fixed_pages`` sets
+    the width of every block table instead of deriving it from the contexts."""
     bs = manager.page_size
     S = len(entries)
     q_lens = [len(e.tokens) for e in entries]
@@ -81,10 +99,16 @@ def pack_batch(entries: List[StepEntry], starts: List[int], rows: List[int], man
 
     parts = [ids, pos, tok_seq, cu, ctx, np.asarray(slots_host, dtype=np.int32),
              np.asarray(rows, dtype=np.int32)]
-    group_shapes = []
+    group_pages = []
     for gi, g in enumerate(manager.page_groups):
         max_pages = max(manager.pages_for(int(c)) for c in ctx)
-        max_pages = -(-max_pages // pad_pages_to) * pad_pages_to
+        if not fixed_pages:
+            max_pages = -(-max_pages // pad_pages_to) * pad_pages_to
+        else:
+            if max_pages > fixed_pages:
+                raise ValueError(f"a context of {int(ctx.max())} tokens does not fit block tables "
+                                 f"of {fixed_pages} pages")
+            max_pages = fixed_pages
         tables = np.zeros((S, max_pages), dtype=np.int32)
         slots = np.empty(T, dtype=np.int32)
         for i, e in enumerate(entries):
@@ -97,27 +121,42 @@ def pack_batch(entries: List[StepEntry], starts: List[int], rows: List[int], man
                 raise AssertionError(f"request {e.request!r} writes into a released page")
             slots[cu[i]:cu[i + 1]] = page * bs + p % bs
         parts += [slots, tables.reshape(-1)]
-        group_shapes.append(max_pages)
+        group_pages.append(max_pages)
 
     sizes = [p.size for p in parts]
     offsets = np.concatenate([[0], np.cumsum([-(-s // 4) * 4 for s in sizes])])   # 16-byte aligned
-    host = torch.empty(int(offsets[-1]), dtype=torch.int32,
-                       pin_memory=(torch.device(device).type == "cuda"))
-    host_np = host.numpy()
+    flat = np.zeros(int(offsets[-1]), dtype=np.int32)
     for p, o in zip(parts, offsets[:-1]):
-        host_np[o:o + p.size] = p
-    dev = host.to(device, non_blocking=True)
-    views = [dev[int(o):int(o) + s] for o, s in zip(offsets[:-1], sizes)]
+        flat[o:o + p.size] = p
+    return BatchArrays(flat, [int(o) for o in offsets[:-1]], sizes, group_pages, q_lens,
+                       list(starts), [e.request for e in entries], slots_host, len(rows),
+                       int(ctx.max()))
 
+
+def batch_on_device(arr: BatchArrays, dev: torch.Tensor, max_ctx_len: int = 0) -> StepBatch:
+    """A StepBatch whose arrays are views into ``dev`` (the flat array on the
+    device)."""
+    views = [dev[o:o + s] for o, s in zip(arr.offsets, arr.sizes)]
+    S = len(arr.q_lens)
     groups = []
-    for gi, max_pages in enumerate(group_shapes):
+    for gi, max_pages in enumerate(arr.group_pages):
         groups.append(GroupMeta(views[7 + 2 * gi], views[8 + 2 * gi].view(S, max_pages), max_pages))
-    n_prefill = sum(1 for q in q_lens if q > 1)
+    n_prefill = sum(1 for q in arr.q_lens if q > 1)
     return StepBatch(
-        num_tokens=T, num_seqs=S, num_prefill_seqs=n_prefill,
-        num_prefill_tokens=int(cu[n_prefill]), num_logit_rows=len(rows),
-        max_q_len=max(q_lens), max_ctx_len=int(ctx.max()),
+        num_tokens=sum(arr.q_lens), num_seqs=S, num_prefill_seqs=n_prefill,
+        num_prefill_tokens=sum(q for q in arr.q_lens if q > 1), num_logit_rows=arr.num_rows,
+        max_q_len=max(arr.q_lens), max_ctx_len=max_ctx_len or arr.max_ctx_len,
         ids=views[0], positions=views[1], tok_seq=views[2], cu_q=views[3], ctx_len=views[4],
         state_slots=views[5], logit_rows=views[6], groups=groups,
-        q_lens=q_lens, starts=list(starts), requests=[e.request for e in entries],
-        host_state_slots=slots_host)
+        q_lens=arr.q_lens, starts=arr.starts, requests=arr.requests,
+        host_state_slots=arr.state_slots)
+
+
+def pack_batch(entries: List[StepEntry], starts: List[int], rows: List[int], manager, device,
+               pad_pages_to: int = 8) -> StepBatch:
+    """Build the arrays of a step and copy them to the device in one transfer."""
+    arr = build_arrays(entries, starts, rows, manager, pad_pages_to)
+    host = torch.from_numpy(arr.flat)
+    if torch.device(device).type == "cuda":
+        host = host.pin_memory()
+    return batch_on_device(arr, host.to(device, non_blocking=True))

@@ -14,7 +14,7 @@ import torch
 from ..cache import CacheManager, CachePool
 from ..parts.base import Runtime
 from ..parts.model import DecoderModel
-from .batch import StepBatch, StepEntry, pack_batch
+from .batch import StepBatch, StepEntry, batch_on_device, build_arrays, pack_batch
 
 
 class OutOfPages(RuntimeError):
@@ -22,8 +22,11 @@ class OutOfPages(RuntimeError):
 
 
 class ModelRunner:
+    GRAPH_MAX_SEQS = 64
+    GRAPH_MIN_CONTEXT = 512
+
     def __init__(self, model: DecoderModel, num_pages: int, page_size: int,
-                 max_num_seqs: int = 64):
+                 max_num_seqs: int = 64, use_graphs: bool = True):
         self.model = model
         self.rt: Runtime = model.rt
         self.manager = CacheManager(model.spec.stream_specs(), num_pages, page_size,
@@ -33,6 +36,10 @@ class ModelRunner:
         self.max_positions = model.spec.max_position_embeddings
         self.steps = 0
         self.tokens_run = 0
+        # decode steps of up to GRAPH_MAX_SEQS single tokens replay a captured HIP graph
+        self.use_graphs = (use_graphs and self.rt.device.type == "cuda" and model.spec.graph_safe)
+        self._graphs = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------ requests
     def open(self, request: Hashable) -> bool:
@@ -42,11 +49,12 @@ class ModelRunner:
         self.manager.close(request)
 
     # ---------------------------------------------------------------- step
-    def prepare(self, entries: List[StepEntry]):
-        """Reserve pages and build the device batch.  Returns (batch, order):
-        the entries are packed with multi-token ones first, ``order`` maps the
-        packed position back; wanted rows stay in the callers' order."""
+    def reserve(self, entries: List[StepEntry]):
+        """Open what is new, reserve pages for every entry, and order the step:
+        multi-token entries first.  Returns (packed entries, their cached
+        lengths, wanted rows in the callers' order of entries)."""
         m = self.manager
+        vocab = self.model.spec.vocab_size
         seen = set()
         for e in entries:
             if e.request in seen:
@@ -54,6 +62,8 @@ class ModelRunner:
             seen.add(e.request)
             if len(e.tokens) < 1:
                 raise ValueError(f"request {e.request!r} brings no tokens")
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:
+                raise ValueError(f"request {e.request!r}: token id outside the vocabulary of {vocab}")
             if not m.is_open(e.request) and not m.open(e.request):
                 raise OutOfPages(f"no state slot free for request {e.request!r}")
         for e in entries:
@@ -79,8 +89,65 @@ class ModelRunner:
                     raise ValueError(f"request {e.request!r}: wanted place {w} is outside its "
                                      f"{len(e.tokens)} tokens")
                 rows.append(offset_of[i] + int(w))
-        batch = pack_batch(packed, starts, rows, m, self.rt.device)
-        return batch, packed
+        return packed, starts, rows
+
+    def prepare(self, entries: List[StepEntry]):
+        """Reserve pages and build the device batch: (batch, packed entries)."""
+        packed, starts, rows = self.reserve(entries)
+        return pack_batch(packed, starts, rows, self.manager, self.rt.device), packed
+
+    # -------------------------------------------------------------- graphs
+    def _graph_key(self, packed, starts, rows):
+        """(sequences, context capacity) when the step is a pure decode step
+        that a captured graph can run, else None."""
+        B = len(packed)
+        if not self.use_graphs or B > self.GRAPH_MAX_SEQS or len(rows) != B:
+            return None
+        if any(len(e.tokens) != 1 for e in packed) or rows != list(range(B)):
+            return None
+        cap = self.GRAPH_MIN_CONTEXT
+        need = max(starts) + 1
+        while cap < need:
+            cap *= 2
+        return (B, cap)
+
+    def _step_graph(self, key, packed, starts, rows):
+        """Decode step through a HIP graph.  The first step of a shape runs
+        eagerly on a side stream (its result is returned) and is then captured;
+        later steps overwrite the graph's metadata buffer and replay it.
+        Everything a launch depends on besides device memory is fixed by the
+        key: the number of sequences and the context capacity, which sets the
+        width of the block tables and how the decode attention splits."""
+        B, cap = key
+        pages = cap // self.manager.page_size
+        arr = build_arrays(packed, starts, rows, self.manager, fixed_pages=pages)
+        host = torch.from_numpy(arr.flat)
+        entry = self._graphs.get(key)
+        if entry is not None:
+            graph, dev, staging, logits, copied = entry
+            copied.synchronize()              # the last copy out of the staging buffer is done
+            staging.copy_(host)
+            dev.copy_(staging, non_blocking=True)
+            copied.record()
+            graph.replay()
+            self.graph_replays += 1
+            return logits
+        staging = torch.empty_like(host).pin_memory()
+        staging.copy_(host)
+        dev = staging.to(self.rt.device, non_blocking=True)
+        batch = batch_on_device(arr, dev, max_ctx_len=cap)
+        side = torch.cuda.Stream(device=self.rt.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            eager = self.model.forward(batch, self.bindings)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(batch, self.bindings)
+        copied = torch.cuda.Event()
+        copied.record()
+        self._graphs[key] = (graph, dev, staging, logits, copied)
+        return eager
 
     @torch.no_grad()
     def step(self, entries: List[StepEntry]) -> torch.Tensor:
@@ -89,10 +156,15 @@ class ModelRunner:
         if not entries:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32,
                                device=self.rt.device)
-        batch, packed = self.prepare(entries)
-        logits = self.model.forward(batch, self.bindings)
-        for e, start, n in zip(packed, batch.starts, batch.q_lens):
-            self.manager.commit(e.request, start + n)
+        packed, starts, rows = self.reserve(entries)
+        key = self._graph_key(packed, starts, rows)
+        if key is not None:
+            logits = self._step_graph(key, packed, starts, rows)
+        else:
+            batch = pack_batch(packed, starts, rows, self.manager, self.rt.device)
+            logits = self.model.forward(batch, self.bindings)
+        for e, start in zip(packed, starts):
+            self.manager.commit(e.request, start + len(e.tokens))
         self.steps += 1
-        self.tokens_run += batch.num_tokens
+        self.tokens_run += sum(len(e.tokens) for e in packed)
         return logits

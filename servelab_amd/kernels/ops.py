@@ -30,7 +30,8 @@ def _p(t: Optional[torch.Tensor]):
 
 
 class HipOps:
-    ROWS_KERNEL_MAX_M = 16        # the few-rows GEMM takes up to this many rows per pass
+    ROWS_KERNEL_MAX_M = 16        # the wavefront-per-column GEMM is used up to this many rows
+    SKINNY_MAX_M = 64             # the matrix-core few-rows GEMM takes up to this many rows
 
     def __init__(self, act_dtype: torch.dtype, device="cuda:0"):
         if act_dtype not in (torch.bfloat16, torch.float32):
@@ -115,17 +116,25 @@ class HipOps:
         self._check(w, self.act_dtype, (N, K), "weight")
         if bias is not None:
             self._check(bias, torch.float32, (N,), "bias")
-        vec = 4 if self.act_dtype == torch.float32 else 8
-        rows_ok = K % vec == 0
-        if rows_ok and M <= self.ROWS_KERNEL_MAX_M:
-            return self.linear_rows(x, w, bias, out_f32)
         if self.act_dtype == torch.float32:
-            return self.linear_tiled(x, w, bias, out_f32)
-        if out_f32:
-            if rows_ok and M <= 4 * self.ROWS_KERNEL_MAX_M:
+            if K % 4 == 0 and M <= self.ROWS_KERNEL_MAX_M:
                 return self.linear_rows(x, w, bias, out_f32)
             return self.linear_tiled(x, w, bias, out_f32)
+        if M <= self.SKINNY_MAX_M and K % 32 == 0:
+            return self.linear_skinny(x, w, bias, out_f32)
+        if M <= self.ROWS_KERNEL_MAX_M and K % 8 == 0:
+            return self.linear_rows(x, w, bias, out_f32)
+        if out_f32:
+            return self.linear_tiled(x, w, bias, out_f32)
         return self.linear_library(x, w, bias)
+
+    def linear_skinny(self, x, w, bias, out_f32=False, nt=0):
+        M, K = x.shape
+        N = w.shape[0]
+        y = self._new((M, N), torch.float32 if out_f32 else None)
+        self._call("gemm", "sl_gemm_skinny", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32),
+                   int(nt))
+        return y
 
     def linear_rows(self, x, w, bias, out_f32=False):
         M, K = x.shape
@@ -260,7 +269,7 @@ class HipOps:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
                 blocks = min(blocks, -(-int(window) // 32) + 1)
-            nsplit = max(1, min(blocks // 2, -(-self.TARGET_WAVES // (n_dec * nkv))))
+            nsplit = max(1, min(64, blocks // 2, -(-self.TARGET_WAVES // (n_dec * nkv))))
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)

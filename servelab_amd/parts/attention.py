@@ -17,6 +17,8 @@ from .base import Mixer, PagedKVSpec, ParamSpec
 
 
 class PagedAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, position,
                  qkv_bias=True, window=None, scale=None):
         if num_heads % num_kv_heads:

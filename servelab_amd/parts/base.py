@@ -60,7 +60,13 @@ def prefixed(prefix: str, source: TensorSource) -> TensorSource:
 
 
 class Part:
-    """Base of all parts."""
+    """Base of all parts.  ``graph_safe`` says that the part's computation is a
+    fixed sequence of kernel launches that reads sizes only from the batch's
+    host fields and data only from device memory (no host synchronisation, no
+    library call that records memsets), so a decode step through it may be
+    captured into a HIP graph and replayed."""
+
+    graph_safe = False
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {}

@@ -14,6 +14,10 @@ class PreNormBlock(Block):
         self.norm1, self.mixer, self.norm2, self.feedforward = norm1, mixer, norm2, feedforward
         self.names = tuple(names)
 
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for _, part in self._children())
+
     def _children(self):
         return list(zip(self.names, (self.norm1, self.mixer, self.norm2, self.feedforward)))
 

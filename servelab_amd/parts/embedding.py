@@ -8,6 +8,8 @@ from .base import Part, ParamSpec
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
 
@@ -24,6 +26,8 @@ class TokenEmbedding(Part):
 
 
 class OutputHead(Part):
+    graph_safe = True
+
     """``tied_to`` is the embedding part whose table the head shares, or None."""
 
     def __init__(self, vocab_size: int, hidden_size: int, tied_to=None):

@@ -10,6 +10,8 @@ from .base import FeedForward, ParamSpec
 
 
 class GatedMLP(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         if activation != "silu":
             raise ValueError(f"GatedMLP: activation '{activation}' is not supported")

@@ -42,6 +42,10 @@ class ModelSpec:
     def children(self):
         return [self.embedding] + list(self.layers) + [self.final_norm, self.head]
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for _, part in self.children())
+
     def param_specs(self) -> Dict[str, ParamSpec]:
         """Every checkpoint tensor of the model, in a fixed order."""
         specs: Dict[str, ParamSpec] = {}

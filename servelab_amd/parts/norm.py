@@ -8,6 +8,8 @@ from .base import Norm, ParamSpec
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size = int(size)
         self.eps = float(eps)

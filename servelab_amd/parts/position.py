@@ -11,6 +11,8 @@ from .base import PositionEncoding
 
 
 class RotaryPosition(PositionEncoding):
+    graph_safe = True
+
     kind = "rotary"
 
     def __init__(self, head_dim: int, theta: float):
@@ -33,6 +35,8 @@ class RotaryPosition(PositionEncoding):
 
 
 class NoPosition(PositionEncoding):
+    graph_safe = True
+
     kind = "none"
 
     def tables(self, batch, shared):

@@ -1,0 +1,150 @@
+"""The whole engine on the GPU, in float32 and in bfloat16: greedy generation
+through the entry point, long decoding across graph captures, the first tokens
+of a sequence, preemption, sampling with a temperature."""
+import random
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+import replay_schedules as rs
+from replay_harness import compare, plain_logits, replay_in_process
+from servelab_amd import CacheConfig, LLMEngine, SamplingParams, SchedulerConfig, load_config
+from servelab_amd.engine import ModelRunner, StepEntry
+from servelab_amd.engine.session import load_model_on_device
+from tiny_configs import TINY, make_folder
+
+pytestmark = pytest.mark.gpu
+TOL = {"float32": 1e-4, "bfloat16": 3e-2}
+PROMPTS = [list(range(10, 40)), [5, 9, 200, 31], list(range(300, 377)), [7]]
+
+
+def make_engine(folder, dtype, num_blocks=64, max_batched=256, max_seqs=8):
+    return LLMEngine(load_config(folder), CacheConfig(num_blocks=num_blocks),
+                     SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched),
+                     dtype=dtype)
+
+
+def check_greedy(cfg, w, prompt, tokens, dtype):
+    """float32: the plain implementation's tokens exactly.  bfloat16: every
+    chosen token is, for the plain implementation fed the same tokens, within
+    the tolerance of the best logit (rounding may flip near ties)."""
+    if dtype == "float32":
+        assert tokens == plain.greedy_generate(cfg, w, prompt, len(tokens))
+        return
+    logits = plain.forward(cfg, w, list(prompt) + tokens)
+    for i, t in enumerate(tokens):
+        row = logits[len(prompt) - 1 + i]
+        assert row[t] >= row.max() - 2 * TOL[dtype], f"token {i}: {row[t]} vs best {row.max()}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(tmp_path, which, dtype):
+    folder = make_folder(tmp_path, which, seed=21)
+    cfg, w = plain.load_folder(folder)
+    vocab = TINY[which]["vocab_size"]
+    prompts = [[t % vocab for t in p] for p in PROMPTS]
+    outs = make_engine(folder, dtype).generate(prompts, SamplingParams.greedy(12))
+    for p, o in zip(prompts, outs):
+        assert o.finished and o.outputs[0].finish_reason == "length" and len(o.outputs[0].token_ids) == 12
+        check_greedy(cfg, w, p, o.outputs[0].token_ids, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cutting_and_preemption_do_not_change_the_tokens(tmp_path, dtype):
+    folder = make_folder(tmp_path, "B", seed=22)
+    cfg, w = plain.load_folder(folder)
+    base = [o.outputs[0].token_ids for o in
+            make_engine(folder, dtype).generate(PROMPTS, SamplingParams.greedy(12))]
+    for p, t in zip(PROMPTS, base):
+        check_greedy(cfg, w, p, t, dtype)
+    if dtype == "float32":
+        small = make_engine(folder, dtype, max_batched=8)
+        assert [o.outputs[0].token_ids for o in small.generate(PROMPTS, SamplingParams.greedy(12))] == base
+        tight = make_engine(folder, dtype, num_blocks=9, max_batched=64)
+        assert [o.outputs[0].token_ids for o in tight.generate(PROMPTS, SamplingParams.greedy(12))] == base
+        assert tight.stats()["num_preemptions_total"] > 0
+        tight.runner.manager.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_long_decoding_across_graph_captures(tmp_path, which, dtype, monkeypatch):
+    """A short prompt, then 200 tokens one by one: the context outgrows the
+    captured graphs' capacity several times (64 -> 128 -> 256), and two requests
+    decode side by side in one graph."""
+    monkeypatch.setattr(ModelRunner, "GRAPH_MIN_CONTEXT", 64)
+    folder = make_folder(tmp_path, which, seed=23)
+    vocab = TINY[which]["vocab_size"]
+    rng = random.Random(3)
+    requests = {r: [rng.randrange(vocab) for _ in range(n)] for r, n in (("x", 230), ("y", 215))}
+    reference = plain_logits(folder, requests)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": requests["x"][:20], "want": [19]},
+                                     {"id": "y", "tokens": requests["y"][:5], "want": [4]}], "end": []}]
+    for i in range(210):
+        steps.append({"step": i + 1, "entries": [
+            {"id": "x", "tokens": [requests["x"][20 + i]], "want": [0]},
+            {"id": "y", "tokens": [requests["y"][5 + i]], "want": [0]}],
+            "end": ["x", "y"] if i == 209 else []})
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, dtype, rs.max_tokens_needed(steps))
+    worst, where = compare(out, steps, reference, vocab)
+    assert worst < TOL[dtype], f"max abs err {worst} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager(tmp_path, dtype):
+    """The same decode steps with and without graphs; the graph is replayed
+    several times with the program's own eager work between the replays."""
+    folder = make_folder(tmp_path, "B", seed=24)
+    _, model = load_model_on_device(folder, dtype)
+    runs = {}
+    for use_graphs in (False, True):
+        runner = ModelRunner(model, 64, 16, use_graphs=use_graphs)
+        rows = []
+        runner.step([StepEntry("a", list(range(50)), []), StepEntry("b", list(range(7)), [])])
+        for i in range(12):
+            rows.append(runner.step([StepEntry("a", [100 + i], [0]), StepEntry("b", [200 + i], [0])]).clone())
+            if i % 4 == 3:            # an eager mixed step in between
+                rows.append(runner.step([StepEntry("c", [1, 2, 3 + i], [2])]).clone())
+                runner.close("c")
+        runs[use_graphs] = torch.cat(rows)
+        if use_graphs:
+            assert runner.graph_replays >= 10
+    if dtype == "float32":
+        assert torch.equal(runs[True], runs[False])
+    else:        # the captured decode attention splits the context differently: rounding only
+        assert (runs[True] - runs[False]).abs().max().item() < 1e-2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_first_tokens_of_a_sequence(tmp_path, which, dtype):
+    """Position 0 alone, then 1, 2, 3...: a prompt of one token, portions of one."""
+    folder = make_folder(tmp_path, which, seed=25)
+    vocab = TINY[which]["vocab_size"]
+    requests = {"s": [3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7, 9, 3, 2, 3, 8, 4]}
+    reference = plain_logits(folder, requests)
+    steps = [{"step": i, "entries": [{"id": "s", "tokens": [t], "want": [0]}],
+              "end": ["s"] if i == 19 else []} for i, t in enumerate(requests["s"])]
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, dtype, 64)
+    worst, where = compare(out, steps, reference, vocab)
+    assert worst < TOL[dtype], f"max abs err {worst} at {where}"
+
+
+def test_temperature_sampling_through_the_engine(tmp_path):
+    folder = make_folder(tmp_path, "A", seed=26)
+    eng = make_engine(folder, "float32")
+    sp = SamplingParams(temperature=0.8, max_tokens=8, seed=7, ignore_eos=True)
+    a = eng.generate([PROMPTS[0]], sp)[0].outputs[0].token_ids
+    b = eng.generate([PROMPTS[0], PROMPTS[1]], sp)[0].outputs[0].token_ids
+    assert a == b                                    # a seeded request does not depend on its batch
+    hot = SamplingParams(temperature=1.5, max_tokens=8, ignore_eos=True)
+    c = eng.generate([PROMPTS[0]], hot)[0].outputs[0].token_ids
+    d = eng.generate([PROMPTS[0]], hot)[0].outputs[0].token_ids
+    assert c != d                                    # unseeded requests draw from the engine's stream
+    k1 = SamplingParams(temperature=1.0, top_k=1, max_tokens=8, ignore_eos=True)
+    greedy = eng.generate([PROMPTS[0]], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    assert eng.generate([PROMPTS[0]], k1)[0].outputs[0].token_ids == greedy[0].outputs[0].token_ids

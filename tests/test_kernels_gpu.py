@@ -87,6 +87,20 @@ def test_linear(both, M, N, K, bias):
         assert rel_err(got, ref) < tol, (M, N, K, out_f32)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 50, 64), (7, 1000, 3584), (16, 17, 96), (33, 200, 352), (64, 130, 1024)])
+def test_linear_skinny(M, N, K):
+    """The matrix-core few-rows kernel alone (bfloat16): ragged M and N."""
+    from servelab_amd.kernels import HipOps
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    x = randn(M, K, dtype=torch.bfloat16, seed=4)
+    w = randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5)
+    b = randn(N, seed=6)
+    for bias in (None, b):
+        for out_f32 in (False, True):
+            got = ops.linear_skinny(x, w, bias, out_f32)
+            assert rel_err(got, emu.linear(x, w, bias, out_f32)) < (2e-5 if out_f32 else 2 ** -7)
+
+
 @pytest.mark.parametrize("M,N,K", [(5, 70, 24), (64, 64, 16), (65, 129, 37)])
 def test_linear_kernels_separately(both, M, N, K):
     """The tiled kernel takes any K; the few-rows kernel any K that fills
