@@ -29,9 +29,30 @@ def _p(t: Optional[torch.Tensor]):
     return None if t is None else _c_void_p(t.data_ptr())
 
 
+class LinearWeight:
+    """A weight matrix [N, K] as the products read it: row-major for products
+    with many rows, and (bfloat16, when memory allows) a second copy tiled for
+    the few-rows kernel that decode steps use."""
+    __slots__ = ("w", "tiled")
+
+    def __init__(self, w, tiled=None):
+        self.w, self.tiled = w, tiled
+
+    @property
+    def shape(self):
+        return self.w.shape
+
+
 class HipOps:
     ROWS_KERNEL_MAX_M = 16        # the wavefront-per-column GEMM is used up to this many rows
     SKINNY_MAX_M = 64             # the matrix-core few-rows GEMM takes up to this many rows
+
+    # Decode reads every weight once per step and is bound by how fast it
+    # streams; the tiled copy streams faster (see gemm.hip) at the price of
+    # holding the matrices twice.  It is made while the copies stay below this
+    # share of the device's memory; beyond it only the row-major matrix is kept
+    # and the few-rows kernel is not used.
+    TILED_COPY_MEMORY_SHARE = 0.30
 
     def __init__(self, act_dtype: torch.dtype, device="cuda:0"):
         if act_dtype not in (torch.bfloat16, torch.float32):
@@ -48,6 +69,11 @@ class HipOps:
         self._fn = {}
         self._bias_cache = {}
         self.use_mfma_attention = True
+        self.tiled_bytes = 0
+        self.tiled_budget = 0
+        if act_dtype == torch.bfloat16:
+            self.tiled_budget = int(torch.cuda.get_device_properties(self.device).total_memory
+                                    * self.TILED_COPY_MEMORY_SHARE)
 
     # ------------------------------------------------------------ plumbing
     def _call(self, stem, name, *args):
@@ -109,7 +135,24 @@ class HipOps:
         return out
 
     # --------------------------------------------------------------- linear
-    def linear(self, x, w, bias, out_f32=False):
+    def prepare_weight(self, w):
+        """Called once per matrix at load: returns what ``linear`` takes."""
+        N, K = w.shape
+        self._check(w, self.act_dtype, None, "weight")
+        nbytes = -(-N // 16) * 16 * K * 2
+        if (self.act_dtype != torch.bfloat16 or K % 32
+                or self.tiled_bytes + nbytes > self.tiled_budget):
+            return LinearWeight(w)
+        tiled = torch.empty(-(-N // 16) * 16 * K, dtype=torch.bfloat16, device=self.device)
+        self._call("gemm", "sl_tile_weight", _p(w), _p(tiled), N, K)
+        self.tiled_bytes += nbytes
+        return LinearWeight(w, tiled)
+
+    def linear(self, x, weight, bias, out_f32=False):
+        """y = x W^T (+ bias); ``weight`` is a LinearWeight or a plain [N, K] tensor."""
+        if not isinstance(weight, LinearWeight):
+            weight = LinearWeight(weight)
+        w = weight.w
         M, K = x.shape
         N = w.shape[0]
         self._check(x, self.act_dtype, None, "x")
@@ -120,20 +163,24 @@ class HipOps:
             if K % 4 == 0 and M <= self.ROWS_KERNEL_MAX_M:
                 return self.linear_rows(x, w, bias, out_f32)
             return self.linear_tiled(x, w, bias, out_f32)
-        if M <= self.SKINNY_MAX_M and K % 32 == 0:
-            return self.linear_skinny(x, w, bias, out_f32)
+        if M <= self.SKINNY_MAX_M and weight.tiled is not None:
+            return self.linear_skinny(x, weight, bias, out_f32)
         if M <= self.ROWS_KERNEL_MAX_M and K % 8 == 0:
             return self.linear_rows(x, w, bias, out_f32)
         if out_f32:
+            if M <= 4 * self.ROWS_KERNEL_MAX_M and K % 8 == 0:
+                return self.linear_rows(x, w, bias, out_f32)
             return self.linear_tiled(x, w, bias, out_f32)
         return self.linear_library(x, w, bias)
 
-    def linear_skinny(self, x, w, bias, out_f32=False, nt=0):
+    def linear_skinny(self, x, weight, bias, out_f32=False):
         M, K = x.shape
-        N = w.shape[0]
+        N = weight.w.shape[0]
+        if weight.tiled is None:
+            raise KernelError("linear_skinny needs the tiled copy of the weight")
         y = self._new((M, N), torch.float32 if out_f32 else None)
-        self._call("gemm", "sl_gemm_skinny", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32),
-                   int(nt))
+        self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
+                   int(out_f32))
         return y
 
     def linear_rows(self, x, w, bias, out_f32=False):

@@ -54,14 +54,14 @@ class PagedAttention(Mixer):
         self.rt = rt
         self.position.load(tensors, rt)
         # [Wq; Wk; Wv] -> one [(nh + 2 nkv) D, H] matrix, one GEMM
-        self.w_qkv = rt.matrix(torch.cat(
+        self.w_qkv = rt.linear_weight(torch.cat(
             [tensors("q_proj.weight"), tensors("k_proj.weight"), tensors("v_proj.weight")], 0))
         self.b_qkv = None
         if self.qkv_bias:
             self.b_qkv = rt.vector(torch.cat(
                 [tensors("q_proj.bias").float(), tensors("k_proj.bias").float(),
                  tensors("v_proj.bias").float()], 0))
-        self.w_o = rt.matrix(tensors("o_proj.weight"))
+        self.w_o = rt.linear_weight(tensors("o_proj.weight"))
 
     # ---- compute
     def forward(self, x, batch, cache, shared):

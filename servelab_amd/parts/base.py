@@ -47,6 +47,13 @@ class Runtime:
         """A matrix or table in the activation dtype, on the device."""
         return t.to(device=self.device, dtype=self.act_dtype).contiguous()
 
+    def linear_weight(self, t: torch.Tensor):
+        """A matrix that only ``ops.linear`` reads, in whatever form the kernel
+        table wants it."""
+        m = self.matrix(t)
+        prepare = getattr(self.ops, "prepare_weight", None)
+        return prepare(m) if prepare is not None else m
+
     def vector(self, t: torch.Tensor) -> torch.Tensor:
         """A gain or bias: always float32 on the device (they enter float32 math)."""
         return t.to(device=self.device, dtype=torch.float32).contiguous()

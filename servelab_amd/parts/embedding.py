@@ -41,8 +41,8 @@ class OutputHead(Part):
 
     def load(self, tensors, rt):
         self.rt = rt
-        self.weight = self.tied_to.weight if self.tied_to is not None \
-            else rt.matrix(tensors("weight"))
+        self.weight = rt.linear_weight(self.tied_to.weight if self.tied_to is not None
+                                       else tensors("weight"))
 
     def forward(self, rows):
         """normed rows [R, H] -> float32 logits [R, V]."""

@@ -26,9 +26,9 @@ class GatedMLP(FeedForward):
 
     def load(self, tensors, rt):
         self.rt = rt
-        self.w_gate_up = rt.matrix(torch.cat(
+        self.w_gate_up = rt.linear_weight(torch.cat(
             [tensors("gate_proj.weight"), tensors("up_proj.weight")], 0))
-        self.w_down = rt.matrix(tensors("down_proj.weight"))
+        self.w_down = rt.linear_weight(tensors("down_proj.weight"))
 
     def forward(self, x):
         ops = self.rt.ops

@@ -81,6 +81,9 @@ def test_linear(both, M, N, K, bias):
     b = randn(N, seed=3) if bias else None
     tol = 1e-5 if dt == torch.float32 else 2 ** -7
     for out_f32 in (False, True):
+        if dt == torch.bfloat16 and K % 32 == 0:
+            tiled = ops.linear(x, ops.prepare_weight(w), b, out_f32=out_f32)
+            assert rel_err(tiled, emu.linear(x, w, b, out_f32=out_f32)) < tol, (M, N, K, out_f32)
         got = ops.linear(x, w, b, out_f32=out_f32)
         ref = emu.linear(x, w, b, out_f32=out_f32)
         assert got.dtype == ref.dtype and got.shape == ref.shape
@@ -95,9 +98,12 @@ def test_linear_skinny(M, N, K):
     x = randn(M, K, dtype=torch.bfloat16, seed=4)
     w = randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5)
     b = randn(N, seed=6)
+    weight = ops.prepare_weight(w)
+    assert weight.tiled is not None and weight.tiled.numel() == -(-N // 16) * 16 * K
     for bias in (None, b):
         for out_f32 in (False, True):
-            got = ops.linear_skinny(x, w, bias, out_f32)
+            got = ops.linear_skinny(x, weight, bias, out_f32)
+            assert torch.equal(got, ops.linear(x, weight, bias, out_f32))
             assert rel_err(got, emu.linear(x, w, bias, out_f32)) < (2e-5 if out_f32 else 2 ** -7)
 
 
