@@ -23,27 +23,31 @@ extern "C" const char* sl_embed(const int* ids, const void* table, float* out, i
 }
 
 // ------------------------------------------------------------- silu * up
-// out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i], silu(z) = z * sigmoid(z)
-// (servelab/parallel/tp_model.py:68), float inside.
+// out[t, i] = silu(gate[t, i]) * up[t, i], silu(z) = z * sigmoid(z)
+// (servelab/parallel/tp_model.py:68), float inside.  A row of gate_up holds
+// gate and up interleaved in blocks: gate i sits at 2 * block * (i / block) +
+// i % block and up i one block further; block = I is plain [gate | up].
 __global__ void silu_mul_kernel(const act_t* __restrict__ gate_up, act_t* __restrict__ out,
-                                int I, size_t total) {
+                                int I, int block, size_t total) {
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / I;
     const int i = (int)(idx - t * I);
-    const float g = to_f(gate_up[t * 2 * I + i]);
-    const float u = to_f(gate_up[t * 2 * I + I + i]);
+    const size_t at = t * 2 * I + (size_t)2 * block * (i / block) + i % block;
+    const float g = to_f(gate_up[at]);
+    const float u = to_f(gate_up[at + block]);
     out[idx] = from_f<act_t>(g / (1.f + expf(-g)) * u);
   }
 }
 
-extern "C" const char* sl_silu_mul(const void* gate_up, void* out, int T, int I,
+extern "C" const char* sl_silu_mul(const void* gate_up, void* out, int T, int I, int block,
                                    hipStream_t stream) {
   SL_CHECK(T >= 0 && I > 0, "silu_mul: sizes must be positive");
+  SL_CHECK(block > 0 && I % block == 0, "silu_mul: the block must divide the width");
   if (T == 0) return nullptr;
   const size_t total = (size_t)T * I;
   const int blocks = (int)((total + 255) / 256 < 65535 * 4 ? (total + 255) / 256 : 65535 * 4);
-  silu_mul_kernel<<<blocks, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, I, total);
+  silu_mul_kernel<<<blocks, 256, 0, stream>>>((const act_t*)gate_up, (act_t*)out, I, block, total);
   return sl_launch_status();
 }
 

@@ -166,7 +166,11 @@ extern "C" const char* sl_gemm_tiled(const void* x, const void* w, const float* 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int MB>
+//
+// GATED: the 16 rows of a tile are 8 gate rows followed by the 8 up rows of the
+// same channels; the workgroup then writes silu(gate) * up, 8 columns of an
+// [M, N / 2] result, instead of 16 columns of y (servelab/parallel/tp_model.py:68).
+template <int MB, bool GATED>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int out_f32) {
@@ -211,6 +215,22 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
   for (int b = 0; b < MB; ++b) red[wave][b][lane] = acc[b];
   __syncthreads();
   // lane (m_local + 16 (n_local / 4)) holds y[m_local, n_local] in element n_local % 4
+  if (GATED) {
+    for (int idx = threadIdx.x; idx < MB * 128; idx += WAVES * 64) {
+      const int b = idx / 128, rem = idx % 128, m_local = rem / 8, j = rem % 8;
+      const int m = 16 * b + m_local, n = blockIdx.x * 8 + j;
+      if (m < M && n < N / 2) {
+        float gsum = 0.f, usum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; ++wv) {
+          gsum += red[wv][b][m_local + 16 * (j / 4)][j % 4];
+          usum += red[wv][b][m_local + 16 * (2 + j / 4)][j % 4];
+        }
+        ((__bf16*)y)[(size_t)m * (N / 2) + n] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
+      }
+    }
+    return;
+  }
   for (int idx = threadIdx.x; idx < MB * 256; idx += WAVES * 64) {
     const int b = idx / 256, rem = idx % 256, m_local = rem / 16, n_local = rem % 16;
     const int m = 16 * b + m_local, n = n0 + n_local;
@@ -227,8 +247,11 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
 
 // wt: W in the tiled layout, ceil(N / 16) * 16 rows (rows beyond N are zero).
 extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float* bias, void* y,
-                                      int M, int N, int K, int out_f32, hipStream_t stream) {
+                                      int M, int N, int K, int out_f32, int gated,
+                                      hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
+  SL_CHECK(!gated || (N % 16 == 0 && bias == nullptr && !out_f32),
+           "gemm_skinny: the gated form needs N % 16 == 0, no bias, activation output");
   SL_CHECK(M <= 64, "gemm_skinny: at most 64 rows");
   SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
@@ -237,9 +260,15 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
   const dim3 grid((N + 15) / 16);
   const __bf16* xx = (const __bf16*)x;
   const __bf16* ww = (const __bf16*)wt;
-  if (M <= 16) gemm_skinny_kernel<1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
-  else if (M <= 32) gemm_skinny_kernel<2><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
-  else gemm_skinny_kernel<4><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+  if (gated) {
+    if (M <= 16) gemm_skinny_kernel<1, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
+    else if (M <= 32) gemm_skinny_kernel<2, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
+    else gemm_skinny_kernel<4, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
+    return sl_launch_status();
+  }
+  if (M <= 16) gemm_skinny_kernel<1, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+  else if (M <= 32) gemm_skinny_kernel<2, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+  else gemm_skinny_kernel<4, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
   return sl_launch_status();
 }
 

@@ -180,8 +180,27 @@ class HipOps:
             raise KernelError("linear_skinny needs the tiled copy of the weight")
         y = self._new((M, N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
-                   int(out_f32))
+                   int(out_f32), 0)
         return y
+
+    GATE_BLOCK = 8                # gate and up rows alternate in blocks of 8 (half an MFMA tile)
+
+    def gated_linear(self, x, weight, block):
+        """silu(x Wg^T) * (x Wu^T) for a weight whose rows hold gate and up
+        interleaved in blocks of ``block`` rows (``block`` = I: plain [Wg; Wu]).
+        Few rows and a tiled weight with blocks of 8: one fused kernel."""
+        if not isinstance(weight, LinearWeight):
+            weight = LinearWeight(weight)
+        M, K = x.shape
+        N = weight.w.shape[0]
+        if (M <= self.SKINNY_MAX_M and weight.tiled is not None and block == self.GATE_BLOCK
+                and N % 16 == 0):
+            self._check(x, self.act_dtype, None, "x")
+            y = self._new((M, N // 2))
+            self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), None, _p(y), M, N, K,
+                       0, 1)
+            return y
+        return self.silu_mul(self.linear(x, weight, None), block)
 
     def linear_rows(self, x, w, bias, out_f32=False):
         M, K = x.shape
@@ -209,13 +228,17 @@ class HipOps:
             self._bias_cache[key] = b
         return torch.addmm(b, x, w.t())
 
-    def silu_mul(self, gate_up):
+    def silu_mul(self, gate_up, block=None):
         T, two_i = gate_up.shape
         if two_i % 2:
             raise KernelError("silu_mul: the row must hold gate and up of equal width")
+        inter = two_i // 2
+        block = inter if block is None else int(block)
+        if block < 1 or inter % block:
+            raise KernelError(f"silu_mul: block {block} does not divide the width {inter}")
         self._check(gate_up, self.act_dtype, None, "gate_up")
-        out = self._new((T, two_i // 2))
-        self._call("elementwise", "sl_silu_mul", _p(gate_up), _p(out), T, two_i // 2)
+        out = self._new((T, inter))
+        self._call("elementwise", "sl_silu_mul", _p(gate_up), _p(out), T, inter, block)
         return out
 
     # ----------------------------------------------------------------- rope

@@ -1,8 +1,10 @@
 """Gated feed-forward (SwiGLU): down(silu(gate(x)) * up(x)), no biases.
 
 Reference: servelab/parallel/tp_model.py:56-68 (two GEMMs, silu, multiply, one
-GEMM).  Here gate and up are one GEMM over [Wg; Wu] followed by one fused
-silu-multiply kernel.
+GEMM).  Here gate and up are one GEMM over a matrix that holds the rows of Wg
+and Wu interleaved in blocks of 8 (so that one output tile of the few-rows
+kernel has a channel's gate and up and can apply silu-multiply itself), then
+the down GEMM.
 """
 import torch
 
@@ -26,11 +28,16 @@ class GatedMLP(FeedForward):
 
     def load(self, tensors, rt):
         self.rt = rt
-        self.w_gate_up = rt.linear_weight(torch.cat(
-            [tensors("gate_proj.weight"), tensors("up_proj.weight")], 0))
+        gate, up = tensors("gate_proj.weight"), tensors("up_proj.weight")
+        i, h = self.intermediate_size, self.hidden_size
+        self.block = getattr(rt.ops, "GATE_BLOCK", i)
+        if i % self.block:
+            self.block = i                       # plain [Wg; Wu]
+        b = self.block
+        self.w_gate_up = rt.linear_weight(torch.stack(
+            [gate.reshape(i // b, b, h), up.reshape(i // b, b, h)], 1).reshape(2 * i, h))
         self.w_down = rt.linear_weight(tensors("down_proj.weight"))
 
     def forward(self, x):
         ops = self.rt.ops
-        gate_up = ops.linear(x, self.w_gate_up, None)
-        return ops.linear(ops.silu_mul(gate_up), self.w_down, None)
+        return ops.linear(ops.gated_linear(x, self.w_gate_up, self.block), self.w_down, None)

@@ -45,10 +45,16 @@ class EmulatedOps:
             y = y + bias
         return y if out_f32 else y.to(self.act_dtype)
 
-    def silu_mul(self, gate_up):
-        inter = gate_up.shape[1] // 2
-        g, u = _f(gate_up[:, :inter]), _f(gate_up[:, inter:])
+    def silu_mul(self, gate_up, block=None):
+        """gate and up interleaved in blocks of ``block`` columns (default: halves)."""
+        T, inter = gate_up.shape[0], gate_up.shape[1] // 2
+        block = inter if block is None else block
+        gu = _f(gate_up).view(T, inter // block, 2, block)
+        g, u = gu[:, :, 0].reshape(T, inter), gu[:, :, 1].reshape(T, inter)
         return (g * torch.sigmoid(g) * u).to(self.act_dtype)
+
+    def gated_linear(self, x, w, block):
+        return self.silu_mul(self.linear(x, w, None), block)
 
     # ----------------------------------------------------------------- rope
     def rope_tables(self, positions, inv_freq):

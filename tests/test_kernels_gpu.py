@@ -133,6 +133,24 @@ def test_silu_mul(both):
     assert ops.silu_mul(gu).abs().max().item() == 0
 
 
+@pytest.mark.parametrize("M,I,K", [(1, 352, 128), (9, 192, 64), (40, 1000, 96), (70, 24, 32), (3, 12, 64)])
+def test_gated_linear(both, M, I, K):
+    """gate/up GEMM + silu-multiply: the fused few-rows kernel (bfloat16, blocks
+    of 8) and the two-kernel path, against the plain product with separate halves."""
+    ops, emu, dt = both
+    x = randn(M, K, dtype=dt, seed=1)
+    gate, up = randn(I, K, dtype=dt, scale=0.2, seed=2), randn(I, K, dtype=dt, scale=0.2, seed=3)
+    ref = emu.silu_mul(emu.linear(x, torch.cat([gate, up]), None))
+    tol = 2e-5 if dt == torch.float32 else 2 ** -6
+    for block in (8, I):
+        if I % block:
+            continue
+        w = torch.stack([gate.reshape(I // block, block, K), up.reshape(I // block, block, K)], 1)
+        w = w.reshape(2 * I, K).contiguous()
+        assert rel_err(ops.gated_linear(x, ops.prepare_weight(w), block), ref) < tol
+        assert rel_err(ops.silu_mul(ops.linear(x, w, None), block), ref) < tol
+
+
 def test_rope_tables(both):
     ops, emu, dt = both
     D, theta = 48, 1e6
