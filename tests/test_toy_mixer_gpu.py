@@ -1,0 +1,166 @@
+"""A toy architecture defined here, in the test, is registered, written as a
+random model folder, loaded, and stepped by the engine without any change to
+the framework's files: a mixer with a fixed-size state of its own per request
+(a decaying sum of projected inputs), used in a model whose layers have
+different mixers and whose run list calls the recurrent layer twice with two
+state streams.  It is no model of anyone's; it only exercises the interfaces."""
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+from servelab_amd import LLMEngine, CacheConfig, SamplingParams, SchedulerConfig, load_config, \
+    register_architecture, write_random_model
+from servelab_amd.engine import ModelRunner, StepEntry
+from servelab_amd.engine.session import load_model_on_device
+from servelab_amd.parts import (GatedMLP, LayerCall, Mixer, ModelSpec, OutputHead, PagedAttention,
+                                ParamSpec, PreNormBlock, RMSNorm, RotaryPosition, StateSpec,
+                                TokenEmbedding)
+
+pytestmark = pytest.mark.gpu
+
+
+class DecayingSumMixer(Mixer):
+    """s_t = decay * s_{t-1} + W x_t ; y_t = s_t.  The state s (one vector per
+    request) lives in the state slot the cache manager gives the request."""
+
+    def __init__(self, hidden_size, decay):
+        self.hidden_size, self.decay = hidden_size, decay
+
+    def param_specs(self):
+        return {"in_proj.weight": ParamSpec((self.hidden_size, self.hidden_size))}
+
+    def cache_spec(self):
+        return StateSpec((self.hidden_size,), "float32")
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        self.w = tensors("in_proj.weight").to(rt.device, torch.float32)
+
+    def forward(self, x, batch, cache, shared):
+        u = x.float() @ self.w.T
+        out = torch.empty_like(u)
+        row = 0
+        for start, n, slot in zip(batch.starts, batch.q_lens, batch.host_state_slots):
+            s = torch.zeros(self.hidden_size, device=u.device) if start == 0 else cache.state[slot].clone()
+            for i in range(n):
+                s = self.decay * s + u[row + i]
+                out[row + i] = s
+            if cache.write:
+                cache.state[slot] = s
+            row += n
+        return out.to(x.dtype)
+
+
+@dataclass
+class ToyConfig:
+    hidden_size: int = 48
+    vocab_size: int = 211
+    decay: float = 0.8
+    dtype: str = "float32"
+    architecture: str = "ToyRecurrentForCausalLM"
+    path: str = ""
+
+    @classmethod
+    def from_hf(cls, raw, path=""):
+        return cls(raw["hidden_size"], raw["vocab_size"], raw["decay"], raw.get("torch_dtype", "float32"), path=path)
+
+    def to_hf(self):
+        return {"architectures": [self.architecture], "hidden_size": self.hidden_size,
+                "vocab_size": self.vocab_size, "decay": self.decay, "torch_dtype": self.dtype}
+
+
+def build_toy(cfg):
+    h = cfg.hidden_size
+    emb = TokenEmbedding(cfg.vocab_size, h)
+    recurrent = PreNormBlock(RMSNorm(h, 1e-6), DecayingSumMixer(h, cfg.decay), RMSNorm(h, 1e-6),
+                             GatedMLP(h, 80), names=("norm_a.", "mixer.", "norm_b.", "ffn."))
+    attention = PreNormBlock(RMSNorm(h, 1e-6), PagedAttention(h, 3, 1, 16, RotaryPosition(16, 1e4), qkv_bias=False),
+                             RMSNorm(h, 1e-6), GatedMLP(h, 80))
+    return ModelSpec(("tok.", emb), [("layers.0.", recurrent), ("layers.1.", attention)],
+                     [LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2)],
+                     ("final_norm.", RMSNorm(h, 1e-6)), ("out.", OutputHead(cfg.vocab_size, h)),
+                     cfg.vocab_size, h, eos_token_id=-1, max_position_embeddings=4096)
+
+
+def plain_toy(cfg, w, toks):
+    """The same model, whole sequence, plain torch on the CPU."""
+    import math
+    import plain_qwen2 as plain
+    T, h = len(toks), cfg.hidden_size
+    pos = torch.arange(T)
+    x = w["tok.weight"][toks]
+
+    def recurrent(x):
+        u = plain.rms_norm(x, w["layers.0.norm_a.weight"], 1e-6) @ w["layers.0.mixer.in_proj.weight"].T
+        s, ys = torch.zeros(h), []
+        for t in range(T):
+            s = cfg.decay * s + u[t]
+            ys.append(s)
+        x = x + torch.stack(ys)
+        return x + plain.swiglu(plain.rms_norm(x, w["layers.0.norm_b.weight"], 1e-6), w["layers.0.ffn.gate_proj.weight"],
+                                w["layers.0.ffn.up_proj.weight"], w["layers.0.ffn.down_proj.weight"])
+    x = recurrent(x)
+    p = "layers.1."
+    n = plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-6)
+    inv = plain.rope_inv_freq(1e4, 16)
+    q = plain.apply_rope((n @ w[p + "self_attn.q_proj.weight"].T).view(T, 3, 16), pos, inv)
+    k = plain.apply_rope((n @ w[p + "self_attn.k_proj.weight"].T).view(T, 1, 16), pos, inv)
+    v = (n @ w[p + "self_attn.v_proj.weight"].T).view(T, 1, 16)
+    x = x + plain.attention(q, k, v, 1 / math.sqrt(16), pos, pos).reshape(T, 48) @ w[p + "self_attn.o_proj.weight"].T
+    x = x + plain.swiglu(plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-6), w[p + "mlp.gate_proj.weight"],
+                         w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    x = recurrent(x)
+    return plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["out.weight"].T
+
+
+def test_toy_architecture_registers_builds_and_steps(tmp_path):
+    register_architecture("ToyRecurrentForCausalLM", ToyConfig.from_hf, build_toy)
+    folder = write_random_model(ToyConfig(), str(tmp_path / "toy"), seed=3, std=0.1)
+    cfg = load_config(folder)
+    assert isinstance(cfg, ToyConfig)
+    _, model = load_model_on_device(folder, "float32")
+    runner = ModelRunner(model, num_pages=16, page_size=16, max_num_seqs=2)
+    m = runner.manager
+    assert len(m.state_groups) == 1 and m.state_groups[0].streams == [0, 2] and len(m.page_groups) == 1
+    assert not runner.use_graphs                       # the toy mixer loops on the host
+    from safetensors.torch import load_file
+    w = {k: v.float() for k, v in load_file(folder + "/model.safetensors").items()}
+    gen = torch.Generator().manual_seed(0)
+    seqs = {r: torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for r, n in (("a", 40), ("b", 23), ("c", 31))}
+    ref = {r: plain_toy(cfg, w, t) for r, t in seqs.items()}
+    # a and b side by side in uneven portions; c starts when a has ended and takes its slot
+    plan = [[("a", 0, 13), ("b", 0, 1)], [("a", 13, 14), ("b", 1, 9)], [("b", 9, 10)], [("a", 14, 40), ("b", 10, 23)]]
+    worst = 0.0
+    for step in plan:
+        out = runner.step([StepEntry(r, seqs[r][a:b], list(range(b - a))) for r, a, b in step])
+        row = 0
+        for r, a, b in step:
+            worst = max(worst, (out[row:row + b - a].cpu() - ref[r][a:b]).abs().max().item())
+            row += b - a
+    slot_a = m.state_slot("a")
+    runner.close("a")
+    out = runner.step([StepEntry("c", seqs["c"][:30], list(range(30)))])
+    assert m.state_slot("c") == slot_a                 # the freed slot is used again, state restarted
+    worst = max(worst, (out.cpu() - ref["c"][:30]).abs().max().item())
+    out = runner.step([StepEntry("c", seqs["c"][30:], [0])])
+    worst = max(worst, (out.cpu() - ref["c"][30:]).abs().max().item())
+    assert worst < 1e-4, worst
+    m.check()
+
+
+def test_toy_architecture_generates_through_the_engine(tmp_path):
+    register_architecture("ToyRecurrentForCausalLM", ToyConfig.from_hf, build_toy)
+    folder = write_random_model(ToyConfig(), str(tmp_path / "toy"), seed=4, std=0.1)
+    cfg = load_config(folder)
+    from safetensors.torch import load_file
+    w = {k: v.float() for k, v in load_file(folder + "/model.safetensors").items()}
+    eng = LLMEngine(cfg, CacheConfig(num_blocks=8), SchedulerConfig(max_num_seqs=2, max_num_batched_tokens=16),
+                    dtype="float32")
+    prompts = [[5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24], [100, 3]]
+    outs = eng.generate(prompts, SamplingParams.greedy(6))
+    for p, o in zip(prompts, outs):
+        toks = list(p)
+        for t in o.outputs[0].token_ids:
+            assert t == int(torch.argmax(plain_toy(cfg, w, toks)[-1]))
+            toks.append(t)
