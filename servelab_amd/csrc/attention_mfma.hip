@@ -44,6 +44,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// 2^x by the hardware instruction; arguments here are <= 0 and tiny results may flush to 0
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 constexpr int D = SL_HEAD_DIM;
 constexpr int KK = D / 32;       // k-steps of the score product
 constexpr int DD = D / 16;       // row tiles of the output product
@@ -95,7 +98,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const AttnParams P) 
     if (!valid) c = ncols - 1;
     tok[b] = c / g;
     head[b] = kvh * g + c % g;
-    pos_c[b] = valid ? pos0 + tok[b] : -1;         // -1: every key is masked
+    pos_c[b] = valid ? pos0 + tok[b] : -1;         // padding: computed like its neighbour, never stored
     lo_c[b] = (P.window > 0 && pos_c[b] - P.window + 1 > 0) ? pos_c[b] - P.window + 1 : 0;
     const __bf16* q = P.qkv + (size_t)(q0 + tok[b]) * P.row_stride + (size_t)head[b] * D + 8 * gq;
 #pragma unroll
@@ -126,8 +129,18 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const AttnParams P) 
     for (int dd = 0; dd < DD; ++dd) o[b][dd] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
+  // blocks every column of this wavefront sees whole need no mask
+  const int full_end = (pos0 + tok_first + 1) / 32;             // blocks below: keys <= first position
+  int full_begin = 0;
+  if (P.window > 0) {
+    const int lo_last = pos0 + c_last / g - P.window + 1;
+    full_begin = lo_last > 0 ? (lo_last + 31) / 32 : 0;
+  }
+  const float scale_log2 = P.scale * 1.4426950408889634f;
+
   for (int kb = kb_begin; kb < kb_end; ++kb) {
     const int kbase = kb * 32;
+    const bool edge = kb >= full_end || kb < full_begin;
     // K: row i of tile m is key kbase + 8 (i / 4) + 4 m + i % 4
     bf16x8 kf[2][KK];
 #pragma unroll
@@ -155,36 +168,43 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const AttnParams P) 
         s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kk], qf[b][kk], s0, 0, 0, 0);
         s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kk], qf[b][kk], s1, 0, 0, 0);
       }
-      // this lane: column n, keys kbase + 8 gq + j, j = 0..7
+      // this lane: column n, keys kbase + 8 gq + j, j = 0..7; scores in units of log 2
       float s[8];
-      float mx = -INFINITY;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = kbase + 8 * gq + j;
-        const float v = (j < 4 ? s0[j] : s1[j - 4]) * P.scale;
-        s[j] = (key <= pos_c[b] && key >= lo_c[b]) ? v : -INFINITY;
-        mx = fmaxf(mx, s[j]);
+      for (int j = 0; j < 8; ++j) s[j] = (j < 4 ? s0[j] : s1[j - 4]) * scale_log2;
+      if (edge) {                                  // a block some column does not see whole
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = kbase + 8 * gq + j;
+          if (key > pos_c[b] || key < lo_c[b]) s[j] = -INFINITY;
+        }
       }
+      float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                       fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run[b], mx);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __expf(m_run[b] - m_safe);
-      m_run[b] = m_new;
+      const bool grew = m_new != m_run[b];
       float psum = 0.f;
       bf16x8 pb;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float p = __expf(s[j] - m_safe);
+        const float p = fast_exp2(s[j] - m_safe);
         psum += p;
         pb[j] = (__bf16)p;
       }
-      l_run[b] = l_run[b] * alpha + psum;
+      if (__any(grew)) {                           // rescale only when some column's maximum grew
+        const float alpha = fast_exp2(m_run[b] - m_safe);
+        m_run[b] = m_new;
+        l_run[b] *= alpha;
 #pragma unroll
-      for (int dd = 0; dd < DD; ++dd) {
-        o[b][dd] *= alpha;
-        o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb, o[b][dd], 0, 0, 0);
+        for (int dd = 0; dd < DD; ++dd) o[b][dd] *= alpha;
       }
+      l_run[b] += psum;
+#pragma unroll
+      for (int dd = 0; dd < DD; ++dd)
+        o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb, o[b][dd], 0, 0, 0);
     }
   }
 
@@ -235,7 +255,7 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
     l = part_ml[(base + lane) * 2 + 1];
   }
   const float mx = wave_max(m);
-  const float w = m == -INFINITY ? 0.f : __expf(m - mx);
+  const float w = m == -INFINITY ? 0.f : fast_exp2(m - mx);     // maxima are in units of log 2
   const float denom = wave_sum(w * l);
   ws[lane] = w;
   __syncthreads();
