@@ -71,6 +71,7 @@ class HipOps:
         self.use_mfma_attention = True
         self.tiled_bytes = 0
         self.tiled_budget = 0
+
         if act_dtype == torch.bfloat16:
             self.tiled_budget = int(torch.cuda.get_device_properties(self.device).total_memory
                                     * self.TILED_COPY_MEMORY_SHARE)
@@ -173,11 +174,25 @@ class HipOps:
             return self.linear_tiled(x, w, bias, out_f32)
         return self.linear_library(x, w, bias)
 
+    WIDE_MIN_M = 17               # from this many rows on, two tiles of W share one read of x
+
+    def linear_wide(self, x, weight, bias, out_f32=False, gated=False):
+        M, K = x.shape
+        N = weight.w.shape[0]
+        if weight.tiled is None:
+            raise KernelError("linear_wide needs the tiled copy of the weight")
+        y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
+        self._call("gemm", "sl_gemm_wide", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
+                   int(out_f32), int(gated))
+        return y
+
     def linear_skinny(self, x, weight, bias, out_f32=False):
         M, K = x.shape
         N = weight.w.shape[0]
         if weight.tiled is None:
             raise KernelError("linear_skinny needs the tiled copy of the weight")
+        if M >= self.WIDE_MIN_M:
+            return self.linear_wide(x, weight, bias, out_f32)
         y = self._new((M, N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                    int(out_f32), 0)
@@ -196,6 +211,8 @@ class HipOps:
         if (M <= self.SKINNY_MAX_M and weight.tiled is not None and block == self.GATE_BLOCK
                 and N % 16 == 0):
             self._check(x, self.act_dtype, None, "x")
+            if M >= self.WIDE_MIN_M:
+                return self.linear_wide(x, weight, None, gated=True)
             y = self._new((M, N // 2))
             self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), None, _p(y), M, N, K,
                        0, 1)

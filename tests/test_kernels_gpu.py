@@ -107,6 +107,19 @@ def test_linear_skinny(M, N, K):
             assert rel_err(got, emu.linear(x, w, bias, out_f32)) < (2e-5 if out_f32 else 2 ** -7)
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048)])
+def test_linear_wide(M, N, K):
+    """The 17..64-row kernel alone: ragged M and N, an odd number of tiles."""
+    from servelab_amd.kernels import HipOps
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    x = randn(M, K, dtype=torch.bfloat16, seed=4)
+    weight = ops.prepare_weight(randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5))
+    b = randn(N, seed=6)
+    assert rel_err(ops.linear_wide(x, weight, b, out_f32=True), emu.linear(x, weight.w, b, True)) < 2e-5
+    assert rel_err(ops.linear_wide(x, weight, None), emu.linear(x, weight.w, None)) < 2 ** -7
+    assert torch.equal(ops.linear(x, weight, b), ops.linear_wide(x, weight, b))
+
+
 @pytest.mark.parametrize("M,N,K", [(5, 70, 24), (64, 64, 16), (65, 129, 37)])
 def test_linear_kernels_separately(both, M, N, K):
     """The tiled kernel takes any K; the few-rows kernel any K that fills
