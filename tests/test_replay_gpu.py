@@ -9,15 +9,10 @@ import pytest
 import torch
 
 import replay_schedules as rs
-from replay_harness import compare, plain_logits, replay_in_process, replay_program
+from replay_harness import compare, plain_logits, replay_in_process, replay_program, tolerance
 from tiny_configs import TINY, make_folder
 
 pytestmark = pytest.mark.gpu
-
-# float32: the bar of the reference's own cross-checks (tests/test_parallel.py:103-104).
-# bfloat16: weights, activations and cache rounded to 8 bits of mantissa; logits
-# of these models are O(0.5), see the measured errors in each assertion message.
-TOL = {"float32": 1e-4, "bfloat16": 3e-2}
 
 
 def make_requests(vocab, lengths, seed):
@@ -51,7 +46,7 @@ def test_replay_matches_plain(tmp_path, which, schedule, dtype):
     replay_in_process(folder, steps, out, dtype, rs.max_tokens_needed(steps))
     worst, where = compare(out, steps, reference, vocab)
     print(f"{which} {schedule} {dtype}: max abs err {worst:.3e} at {where}")
-    assert worst < TOL[dtype], f"max abs err {worst} at {where}"
+    assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -65,4 +60,4 @@ def test_trace_run_program(tmp_path, dtype):
     out = str(tmp_path / "out")
     replay_program(folder, steps, out, dtype, rs.max_tokens_needed(steps))
     worst, where = compare(out, steps, reference, vocab)
-    assert worst < TOL[dtype], f"max abs err {worst} at {where}"
+    assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
