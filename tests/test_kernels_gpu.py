@@ -254,27 +254,34 @@ def test_paged_attention(both, nh, nkv, D, page, window):
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
-def test_attention_finds_a_far_key(both):
-    """One key among hundreds carries all the weight: scale one query and that
-    key so its score stands out; the output must be that key's value."""
+@pytest.mark.parametrize("D,page", [(16, 16), (32, 16), (128, 32)])
+@pytest.mark.parametrize("q_len", [1, 5])
+def test_attention_finds_one_key_at_edges(both, D, page, q_len):
+    """One key among hundreds carries all the weight (its score stands out by
+    construction), placed at a page's last and first slot, at the first and the
+    last visible position, and just inside and just outside a window: the
+    output must be that key's value, or must not be."""
     ops, emu, dt = both
-    nh, nkv, D, page = 4, 2, 32, 16
-    seqs = [(400, 1)]
-    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=3)
-    target = 37
-    pg, off = int(tables[0, target // page]), target % page
-    q = torch.zeros(D)
-    q[0] = 30.0
-    qkv[0, :nh * D] = q.repeat(nh).to(dt)
-    kc[:, :, :, 0] = 0
-    kc[pg, :, off, 0] = 30.0
-    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, None)
-    for h in range(nh):
-        want = vc[pg, h // 2, :, off].float()
-        assert (got[0, h * D:(h + 1) * D].float() - want).abs().max().item() < 2e-2
-    # with a window that ends before the target the key is invisible
-    got_w = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, 100)
-    assert (got_w.float() - got.float()).abs().max().item() > 0.1
+    nh, nkv, ctx, W = 4, 2, 300, 48
+    p_last = ctx - 1                                   # position of the last query
+    targets = [0, page - 1, page, 2 * page - 1, 5 * page, p_last - W + 1, p_last - W, p_last]
+    for window in (None, W):
+        for target in targets:
+            qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, [(ctx, q_len)], seed=3)
+            qkv[:, :nh * D] = 0
+            qkv[:, 0:nh * D:D] = 30.0                  # every head's query: 30 on channel 0
+            kc[:, :, :, 0] = 0
+            pg, off = int(tables[0, target // page]), target % page
+            kc[pg, :, off, 0] = 30.0                   # score 900 for the target, 0 elsewhere
+            got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, window)
+            last = got[-1].float().view(nh, D)         # the query at position ctx - 1
+            visible = window is None or target > p_last - window
+            for h in range(nh):
+                hit = (last[h] - vc[pg, h // 2, :, off].float()).abs().max().item() < 2e-2
+                assert hit == visible, (window, target, h)
+            if q_len > 1 and target == p_last:         # earlier queries of the portion do not see it
+                first = got[0].float().view(nh, D)
+                assert (first[0] - vc[pg, 0, :, off].float()).abs().max().item() > 0.1
 
 
 def test_argmax_and_sampling():
