@@ -120,6 +120,45 @@ __global__ __launch_bounds__(1024) void sample_kernel(
   if (threadIdx.x == 0) out[r] = g.i;
 }
 
+// Greedy rows of a wide vocabulary: CHUNKS workgroups per row each find the
+// best of a slice, a second small kernel picks among them (ties: first index).
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, int V,
+                                                             int chunks, Best* __restrict__ part) {
+  __shared__ Best sb[16];
+  const int r = blockIdx.y, c = blockIdx.x;
+  const float* x = logits + (size_t)r * V;
+  const int per = (V + chunks - 1) / chunks;
+  const int lo = c * per, hi = lo + per < V ? lo + per : V;
+  Best b = {-INFINITY, 0x7fffffff};
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) b = better(b, Best{x[i], i});
+  b = block_best(b, sb);
+  if (threadIdx.x == 0) part[(size_t)r * chunks + c] = b;
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const Best* __restrict__ part, int chunks,
+                                                          int* __restrict__ out) {
+  __shared__ Best sb[16];
+  const int r = blockIdx.x;
+  Best b = {-INFINITY, 0x7fffffff};
+  for (int i = threadIdx.x; i < chunks; i += blockDim.x) b = better(b, part[(size_t)r * chunks + i]);
+  b = block_best(b, sb);
+  if (threadIdx.x == 0) out[r] = b.i;
+}
+
+// part: chunks * R pairs of (float, int) = 8 * chunks * R bytes of scratch.
+extern "C" const char* sl_argmax(const float* logits, int R, int V, int chunks, void* part,
+                                 int* out, hipStream_t stream) {
+  SL_CHECK(R >= 0 && V > 0, "argmax: sizes must be positive");
+  SL_CHECK(chunks >= 1 && chunks <= 1024 && part != nullptr, "argmax: 1..1024 chunks and scratch");
+  SL_CHECK(R <= 65535, "argmax: more than 65535 rows");
+  if (R == 0) return nullptr;
+  argmax_partial_kernel<<<dim3(chunks, R), 256, 0, stream>>>(logits, V, chunks, (Best*)part);
+  const char* e = sl_launch_status();
+  if (e) return e;
+  argmax_final_kernel<<<R, 64, 0, stream>>>((const Best*)part, chunks, out);
+  return sl_launch_status();
+}
+
 extern "C" const char* sl_sample(const float* logits, int R, int V, const float* temperature,
                                  const int* top_k, const float* top_p, const int64_t* seeds,
                                  const int64_t* draws, int* out, hipStream_t stream) {

@@ -369,8 +369,9 @@ class HipOps:
         R, V = logits.shape
         self._check(logits, torch.float32, None, "logits")
         out = self._new((R,), torch.int32)
-        self._call("sampling", "sl_sample", _p(logits), R, V, None, None, None, None, None,
-                   _p(out))
+        chunks = max(1, min(64, V // 2048))
+        part = self._new((R, chunks, 2), torch.float32)
+        self._call("sampling", "sl_argmax", _p(logits), R, V, chunks, _p(part), _p(out))
         return out
 
     def sample(self, logits, temperature, top_k, top_p, seeds, draws):
