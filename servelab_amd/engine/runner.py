@@ -40,6 +40,7 @@ class ModelRunner:
         self.use_graphs = (use_graphs and self.rt.device.type == "cuda" and model.spec.graph_safe)
         self._graphs = {}
         self.graph_replays = 0
+        self._decoding = None         # the last graph step, for the next one to continue from
 
     # ------------------------------------------------------------ requests
     def open(self, request: Hashable) -> bool:
@@ -131,6 +132,7 @@ class ModelRunner:
             copied.record()
             graph.replay()
             self.graph_replays += 1
+            self._decoding = (key, arr)
             return logits
         staging = torch.empty_like(host).pin_memory()
         staging.copy_(host)
@@ -147,7 +149,62 @@ class ModelRunner:
         copied = torch.cuda.Event()
         copied.record()
         self._graphs[key] = (graph, dev, staging, logits, copied)
+        self._decoding = (key, arr)
         return eager
+
+    def _continue_decoding(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+        """The common decode step — the same requests as the last graph step,
+        one more token each — without rebuilding the step's arrays: ids are
+        replaced, positions and contexts advance by one, slots follow the block
+        tables, and a table gains an entry when a request enters a new page.
+        Returns None when the step is anything else."""
+        if self._decoding is None:
+            return None
+        key, arr = self._decoding
+        B, cap = key
+        if len(entries) != B:
+            return None
+        m = self.manager
+        lengths = m.lengths
+        vocab = self.model.spec.vocab_size
+        for e, request, start in zip(entries, arr.requests, arr.starts):
+            if (e.request != request or len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0
+                    or lengths.get(request) != start + 1):
+                return None
+        if max(arr.starts) + 2 > min(cap, self.max_positions):
+            return None
+        for e in entries:
+            if not 0 <= e.tokens[0] < vocab:
+                raise ValueError(f"request {e.request!r}: token id outside the vocabulary of {vocab}")
+            if not m.grow(e.request, lengths[e.request] + 1):
+                raise OutOfPages(
+                    f"request {e.request!r} needs a page, {m.num_free_pages()} free")
+        flat, off, bs = arr.flat, arr.offsets, m.page_size
+        starts = [s + 1 for s in arr.starts]
+        flat[off[0]:off[0] + B] = [e.tokens[0] for e in entries]
+        flat[off[1]:off[1] + B] += 1                      # positions
+        flat[off[4]:off[4] + B] += 1                      # contexts
+        for gi, g in enumerate(m.page_groups):
+            pages = arr.group_pages[gi]
+            slots_at, tables_at = off[7 + 2 * gi], off[8 + 2 * gi]
+            for i, (request, p) in enumerate(zip(arr.requests, starts)):
+                page = g.tables[request][p // bs]
+                flat[slots_at + i] = page * bs + p % bs
+                if p % bs == 0:
+                    flat[tables_at + i * pages + p // bs] = page
+        arr.starts = starts
+        graph, dev, staging, logits, copied = self._graphs[key]
+        copied.synchronize()
+        staging.copy_(torch.from_numpy(flat))
+        dev.copy_(staging, non_blocking=True)
+        copied.record()
+        graph.replay()
+        self.graph_replays += 1
+        for request, p in zip(arr.requests, starts):
+            m.commit(request, p + 1)
+        self.steps += 1
+        self.tokens_run += B
+        return logits
 
     @torch.no_grad()
     def step(self, entries: List[StepEntry]) -> torch.Tensor:
@@ -156,6 +213,10 @@ class ModelRunner:
         if not entries:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32,
                                device=self.rt.device)
+        logits = self._continue_decoding(entries)
+        if logits is not None:
+            return logits
+        self._decoding = None
         packed, starts, rows = self.reserve(entries)
         key = self._graph_key(packed, starts, rows)
         if key is not None:
