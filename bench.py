@@ -37,6 +37,15 @@ QWEN25_7B = dict(
     torch_dtype="bfloat16", eos_token_id=151645)
 
 
+# the other shapes of the same architecture that the engine is sized for
+QWEN25_32B = dict(QWEN25_7B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
+                  num_key_value_heads=8, intermediate_size=27648)
+QWEN25_72B = dict(QWEN25_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                  num_key_value_heads=8, intermediate_size=29568)
+SHAPES = {"7b": ("Qwen2.5-7B shape", QWEN25_7B), "32b": ("Qwen2.5-32B shape", QWEN25_32B),
+          "72b": ("Qwen2.5-72B shape", QWEN25_72B)}
+
+
 class RandomCheckpoint:
     """Seeded random tensors made on the device when a part asks for them, so
     that a 15 GB model needs no file: N(0, 0.02), norm gains 1 + N(0, 0.05)."""
@@ -65,7 +74,7 @@ def build(args):
     from servelab_amd.engine.session import make_runtime, resolve_dtype
     from servelab_amd.parts import DecoderModel, build_model_spec
 
-    raw = dict(QWEN25_7B)
+    raw = dict(SHAPES[args.shape][1])
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -192,6 +201,7 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--prefill-chunk", type=int, default=2048)
+    ap.add_argument("--shape", default="7b", choices=sorted(SHAPES))
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--block-size", type=int, default=16)
@@ -221,13 +231,14 @@ def main():
         "data": "synthetic: seeded random weights, uniform random token ids, cache filled with "
                 "random keys and values up to the context",
         "config": {
-            "model": "Qwen2.5-7B shape", "global_batch": args.batch, "seq_len": args.context,
+            "model": SHAPES[args.shape][0], "global_batch": args.batch, "seq_len": args.context,
             "parallelism": "none", "layers": cfg.num_layers, "layers_of_shape": full_layers,
             "hidden_size": cfg.hidden_size, "num_heads": cfg.num_heads,
             "num_kv_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
             "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "page_size": page, "prefill_tokens": args.prefill_tokens,
             "decode_mean_context": round(mean_ctx, 1), "sampling": "greedy",
+            "weight_layout": model.rt.ops.weight_layout,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},

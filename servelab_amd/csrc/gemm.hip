@@ -427,4 +427,29 @@ extern "C" const char* sl_tile_weight(const void* w, void* wt, int N, int K, hip
       (const __bf16*)w, (__bf16*)wt, N, K, total_vec);
   return sl_launch_status();
 }
+// Tiled -> row-major [N, K] (the inverse), for products with many rows when only
+// the tiled copy is kept.
+__global__ void untile_weight_kernel(const __bf16* __restrict__ wt, __bf16* __restrict__ w, int N,
+                                     int K, size_t total_vec) {
+  const int KT = K / 32;
+  for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec;
+       v += (size_t)gridDim.x * blockDim.x) {
+    // v enumerates the row-major matrix in 16-byte vectors, so the stores are contiguous
+    const size_t n = v / (K / 8);
+    const int k8 = (int)(v % (K / 8));
+    const int ks = k8 / 4, gq = k8 % 4;
+    const size_t src = (((n / 16) * KT + ks) * 64 + 16 * gq + (n % 16)) * 8;
+    *(bf16x8*)(w + v * 8) = *(const bf16x8*)(wt + src);
+  }
+}
+
+extern "C" const char* sl_untile_weight(const void* wt, void* w, int N, int K, hipStream_t stream) {
+  SL_CHECK(N > 0 && K > 0 && K % 32 == 0, "untile_weight: K must be a positive multiple of 32");
+  SL_CHECK(((uintptr_t)w % 16) == 0 && ((uintptr_t)wt % 16) == 0, "untile_weight: 16-byte alignment");
+  const size_t total_vec = (size_t)N * (K / 8);
+  const size_t blocks = (total_vec + 255) / 256;
+  untile_weight_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>(
+      (const __bf16*)wt, (__bf16*)w, N, K, total_vec);
+  return sl_launch_status();
+}
 #endif

@@ -30,17 +30,14 @@ def _p(t: Optional[torch.Tensor]):
 
 
 class LinearWeight:
-    """A weight matrix [N, K] as the products read it: row-major for products
-    with many rows, and (bfloat16, when memory allows) a second copy tiled for
-    the few-rows kernel that decode steps use."""
-    __slots__ = ("w", "tiled")
+    """A weight matrix [N, K] as the products read it: row-major (``w``) for
+    products with many rows, tiled (``tiled``, bfloat16 only) for the few-rows
+    kernels that decode steps use.  Both, or one of them."""
+    __slots__ = ("w", "tiled", "shape")
 
-    def __init__(self, w, tiled=None):
+    def __init__(self, w, tiled=None, shape=None):
         self.w, self.tiled = w, tiled
-
-    @property
-    def shape(self):
-        return self.w.shape
+        self.shape = tuple(w.shape) if w is not None else tuple(shape)
 
 
 class HipOps:
@@ -48,11 +45,16 @@ class HipOps:
     SKINNY_MAX_M = 64             # the matrix-core few-rows GEMM takes up to this many rows
 
     # Decode reads every weight once per step and is bound by how fast it
-    # streams; the tiled copy streams faster (see gemm.hip) at the price of
-    # holding the matrices twice.  It is made while the copies stay below this
-    # share of the device's memory; beyond it only the row-major matrix is kept
-    # and the few-rows kernel is not used.
-    TILED_COPY_MEMORY_SHARE = 0.30
+    # streams; the tiled layout streams faster (see gemm.hip).  Layouts:
+    #   "dual"   row-major and tiled (twice the memory): library GEMM for many
+    #            rows, few-rows kernels for decode;
+    #   "tiled"  tiled only: a product with many rows first writes the matrix
+    #            row-major into a scratch buffer (one extra pass over the matrix
+    #            per product, only while prompts are being processed);
+    #   "rows"   row-major only: decode uses the slower row-major kernels.
+    # ``plan_weights(total_bytes)`` picks "dual" while two copies stay below
+    # DUAL_MEMORY_SHARE of the device's memory, else "tiled".
+    DUAL_MEMORY_SHARE = 0.45
 
     def __init__(self, act_dtype: torch.dtype, device="cuda:0"):
         if act_dtype not in (torch.bfloat16, torch.float32):
@@ -69,12 +71,8 @@ class HipOps:
         self._fn = {}
         self._bias_cache = {}
         self.use_mfma_attention = True
-        self.tiled_bytes = 0
-        self.tiled_budget = 0
-
-        if act_dtype == torch.bfloat16:
-            self.tiled_budget = int(torch.cuda.get_device_properties(self.device).total_memory
-                                    * self.TILED_COPY_MEMORY_SHARE)
+        self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
+        self._untiled = None          # scratch for "tiled": the row-major form of one matrix
 
     # ------------------------------------------------------------ plumbing
     def _call(self, stem, name, *args):
@@ -136,36 +134,61 @@ class HipOps:
         return out
 
     # --------------------------------------------------------------- linear
-    def prepare_weight(self, w):
-        """Called once per matrix at load: returns what ``linear`` takes."""
+    def plan_weights(self, total_bytes: int) -> str:
+        """Choose the layout for a model whose matrices take ``total_bytes``
+        (called before the matrices are loaded)."""
+        if self.act_dtype == torch.bfloat16:
+            total = torch.cuda.get_device_properties(self.device).total_memory
+            self.weight_layout = "dual" if 2 * total_bytes <= self.DUAL_MEMORY_SHARE * total else "tiled"
+        return self.weight_layout
+
+    def prepare_weight(self, w, keep_rows=False):
+        """Called once per matrix at load: returns what ``linear`` takes.
+        ``keep_rows``: the caller holds the row-major tensor anyway (a tied
+        embedding table), so keeping it costs nothing."""
         N, K = w.shape
         self._check(w, self.act_dtype, None, "weight")
-        nbytes = -(-N // 16) * 16 * K * 2
-        if (self.act_dtype != torch.bfloat16 or K % 32
-                or self.tiled_bytes + nbytes > self.tiled_budget):
+        if self.act_dtype != torch.bfloat16 or K % 32 or self.weight_layout == "rows":
             return LinearWeight(w)
         tiled = torch.empty(-(-N // 16) * 16 * K, dtype=torch.bfloat16, device=self.device)
         self._call("gemm", "sl_tile_weight", _p(w), _p(tiled), N, K)
-        self.tiled_bytes += nbytes
+        if self.weight_layout == "tiled" and not keep_rows:
+            return LinearWeight(None, tiled, (N, K))
         return LinearWeight(w, tiled)
+
+    def rows_of(self, weight):
+        """The row-major matrix of a weight; for a tiled-only weight it is
+        written into the scratch buffer (valid until the next call)."""
+        if weight.w is not None:
+            return weight.w
+        N, K = weight.shape
+        if self._untiled is None or self._untiled.numel() < N * K:
+            self._untiled = None
+            self._untiled = torch.empty(N * K, dtype=torch.bfloat16, device=self.device)
+        out = self._untiled[:N * K].view(N, K)
+        self._call("gemm", "sl_untile_weight", _p(weight.tiled), _p(out), N, K)
+        return out
 
     def linear(self, x, weight, bias, out_f32=False):
         """y = x W^T (+ bias); ``weight`` is a LinearWeight or a plain [N, K] tensor."""
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
-        w = weight.w
         M, K = x.shape
-        N = w.shape[0]
+        N = weight.shape[0]
         self._check(x, self.act_dtype, None, "x")
-        self._check(w, self.act_dtype, (N, K), "weight")
+        if weight.shape != (N, K):
+            raise KernelError(f"weight has shape {list(weight.shape)}, x has {K} columns")
+        if weight.w is not None:
+            self._check(weight.w, self.act_dtype, (N, K), "weight")
         if bias is not None:
             self._check(bias, torch.float32, (N,), "bias")
         if self.act_dtype == torch.float32:
             if K % 4 == 0 and M <= self.ROWS_KERNEL_MAX_M:
-                return self.linear_rows(x, w, bias, out_f32)
-            return self.linear_tiled(x, w, bias, out_f32)
+                return self.linear_rows(x, weight.w, bias, out_f32)
+            return self.linear_tiled(x, weight.w, bias, out_f32)
         if M <= self.SKINNY_MAX_M and weight.tiled is not None:
             return self.linear_skinny(x, weight, bias, out_f32)
+        w = self.rows_of(weight)
         if M <= self.ROWS_KERNEL_MAX_M and K % 8 == 0:
             return self.linear_rows(x, w, bias, out_f32)
         if out_f32:
@@ -178,7 +201,7 @@ class HipOps:
 
     def linear_wide(self, x, weight, bias, out_f32=False, gated=False):
         M, K = x.shape
-        N = weight.w.shape[0]
+        N = weight.shape[0]
         if weight.tiled is None:
             raise KernelError("linear_wide needs the tiled copy of the weight")
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
@@ -188,7 +211,7 @@ class HipOps:
 
     def linear_skinny(self, x, weight, bias, out_f32=False):
         M, K = x.shape
-        N = weight.w.shape[0]
+        N = weight.shape[0]
         if weight.tiled is None:
             raise KernelError("linear_skinny needs the tiled copy of the weight")
         if M >= self.WIDE_MIN_M:
@@ -207,7 +230,7 @@ class HipOps:
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
         M, K = x.shape
-        N = weight.w.shape[0]
+        N = weight.shape[0]
         if (M <= self.SKINNY_MAX_M and weight.tiled is not None and block == self.GATE_BLOCK
                 and N % 16 == 0):
             self._check(x, self.act_dtype, None, "x")

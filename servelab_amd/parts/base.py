@@ -47,12 +47,12 @@ class Runtime:
         """A matrix or table in the activation dtype, on the device."""
         return t.to(device=self.device, dtype=self.act_dtype).contiguous()
 
-    def linear_weight(self, t: torch.Tensor):
+    def linear_weight(self, t: torch.Tensor, shared: bool = False):
         """A matrix that only ``ops.linear`` reads, in whatever form the kernel
-        table wants it."""
+        table wants it.  ``shared``: another part keeps ``t`` itself as well."""
         m = self.matrix(t)
         prepare = getattr(self.ops, "prepare_weight", None)
-        return prepare(m) if prepare is not None else m
+        return prepare(m, keep_rows=shared) if prepare is not None else m
 
     def vector(self, t: torch.Tensor) -> torch.Tensor:
         """A gain or bias: always float32 on the device (they enter float32 math)."""

@@ -41,8 +41,10 @@ class OutputHead(Part):
 
     def load(self, tensors, rt):
         self.rt = rt
-        self.weight = rt.linear_weight(self.tied_to.weight if self.tied_to is not None
-                                       else tensors("weight"))
+        if self.tied_to is not None:
+            self.weight = rt.linear_weight(self.tied_to.weight, shared=True)
+        else:
+            self.weight = rt.linear_weight(tensors("weight"))
 
     def forward(self, rows):
         """normed rows [R, H] -> float32 logits [R, V]."""

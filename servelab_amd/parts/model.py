@@ -100,6 +100,14 @@ class DecoderModel:
             get = checkpoint.get
         check_tensors({n: s.shape for n, s in specs.items()}, found,
                       optional=self.spec.optional_tensors)
+        plan = getattr(self.rt.ops, "plan_weights", None)
+        if plan is not None:          # let the kernel table choose its weight layout for this size
+            itemsize = torch.empty((), dtype=self.rt.act_dtype).element_size()
+            total = 0
+            for s in specs.values():
+                if len(s.shape) == 2:
+                    total += s.shape[0] * s.shape[1] * itemsize
+            plan(total)
         for prefix, part in self.spec.children():
             part.load(prefixed(prefix, get), self.rt)
         self.loaded = True

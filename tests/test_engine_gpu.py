@@ -148,3 +148,22 @@ def test_temperature_sampling_through_the_engine(tmp_path):
     k1 = SamplingParams(temperature=1.0, top_k=1, max_tokens=8, ignore_eos=True)
     greedy = eng.generate([PROMPTS[0]], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
     assert eng.generate([PROMPTS[0]], k1)[0].outputs[0].token_ids == greedy[0].outputs[0].token_ids
+
+
+def test_tiled_only_weight_layout_runs_the_whole_model(tmp_path, monkeypatch):
+    """A model too large for two copies of its matrices keeps only the tiled
+    one: prompts go through the row-major scratch, decode straight to the matrix
+    cores; logits equal those with both copies."""
+    from servelab_amd.kernels import HipOps
+    folder = make_folder(tmp_path, "B", seed=27)
+    toks = list(range(100, 180))
+    rows = {}
+    for share in (0.45, 0.0):
+        monkeypatch.setattr(HipOps, "DUAL_MEMORY_SHARE", share)
+        _, model = load_model_on_device(folder, "bfloat16")
+        assert model.rt.ops.weight_layout == ("dual" if share else "tiled")
+        runner = ModelRunner(model, 16, 16)
+        out = [runner.step([StepEntry("a", toks[:70], [0, 69])])]
+        out += [runner.step([StepEntry("a", [t], [0])]).clone() for t in toks[70:]]
+        rows[share] = torch.cat(out)
+    assert torch.equal(rows[0.45], rows[0.0])

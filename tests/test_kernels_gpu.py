@@ -108,6 +108,31 @@ def test_linear_skinny(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048)])
+def test_tiled_only_weights(M, N, K):
+    """Only the tiled copy kept: few rows go straight to the matrix cores, many
+    rows through the row-major scratch and the library; same results as with
+    both copies."""
+    from servelab_amd.kernels import HipOps
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    w = randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5)
+    b = randn(N, seed=6)
+    both_copies = ops.prepare_weight(w)
+    ops.weight_layout = "tiled"
+    tiled_only = ops.prepare_weight(w.clone())
+    assert tiled_only.w is None and tiled_only.shape == (N, K)
+    assert torch.equal(ops.rows_of(tiled_only), w)
+    for rows in (M, 100):
+        x = randn(rows, K, dtype=torch.bfloat16, seed=rows)
+        assert torch.equal(ops.linear(x, tiled_only, b), ops.linear(x, both_copies, b))
+    kept = ops.prepare_weight(w, keep_rows=True)
+    assert kept.w is w and kept.tiled is not None
+    ops.weight_layout = "rows"
+    assert ops.prepare_weight(w).tiled is None
+    assert rel_err(ops.linear(randn(3, K, dtype=torch.bfloat16), ops.prepare_weight(w), b),
+                   emu.linear(randn(3, K, dtype=torch.bfloat16), w, b)) < 2 ** -7
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048)])
 def test_linear_wide(M, N, K):
     """The 17..64-row kernel alone: ragged M and N, an odd number of tiles."""
     from servelab_amd.kernels import HipOps
