@@ -400,6 +400,184 @@ extern "C" const char* sl_gemm_wide(const void* x, const void* wt, const float* 
   return sl_launch_status();
 }
 
+// ------------------------------------- 17 to 64 rows, x staged through LDS
+// The kernel above reads x from L2 once per 32 rows of W.  Here a workgroup of
+// 4 wavefronts owns 128 rows of W (each wavefront two tiles over the
+// workgroup's whole share of K, so nothing is reduced across wavefronts) and
+// stages x through LDS in chunks of 128 values of k, already in the order of
+// the mfma B operand and double-buffered: x leaves L2 once per 128 rows of W.
+// The next chunk of x and of W is loaded while the current one is multiplied.
+// When N is small, K is split over `KS` workgroups (grid.y) that write float
+// partials [KS, M, N]; `splitk_reduce_kernel` adds them, the bias, and rounds.
+template <int MB, int NT, int KC>
+__global__ __launch_bounds__(256) void gemm_mid_kernel(
+    const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
+    void* __restrict__ y, int M, int N, int K, int out_f32, int gated, int KS) {
+  constexpr int WAVES = 4;
+  __shared__ bf16x8 xs[2][KC][MB][64];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
+  const int ntiles = (N + 15) / 16;
+  const int tile0 = (blockIdx.x * WAVES + wave) * NT;
+  const int KT = K / 32;
+  const int kbeg = (int)((long long)KT * blockIdx.y / KS), kend = (int)((long long)KT * (blockIdx.y + 1) / KS);
+  const int nchunks = (kend - kbeg + KC - 1) / KC;
+  const __bf16* wp[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int tile = tile0 + t < ntiles ? tile0 + t : ntiles - 1;
+    wp[t] = wt + ((size_t)tile * KT * 64 + lane) * 8;
+  }
+  // this thread's share of a chunk of x: XF fragments (ks, mb, lane) = (idx / (MB * 64), idx / 64 % MB, idx % 64)
+  constexpr int XF = MB * KC / 4;
+  const __bf16* xsrc[XF];
+  int xks[XF];
+#pragma unroll
+  for (int j = 0; j < XF; ++j) {
+    const int idx = threadIdx.x + 256 * j;
+    const int fl = idx % 64, mb = idx / 64 % MB;
+    xks[j] = idx / (MB * 64);
+    const int m = 16 * mb + (fl & 15) < M ? 16 * mb + (fl & 15) : M - 1;
+    xsrc[j] = x + (size_t)m * K + 8 * (fl >> 4);
+  }
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto load_x = [&](int c, bf16x8 (&xr)[XF]) {
+#pragma unroll
+    for (int j = 0; j < XF; ++j) {
+      const int ks = kbeg + c * KC + xks[j];
+      xr[j] = ks < kend ? *(const bf16x8*)(xsrc[j] + 32 * (size_t)ks) : zero;
+    }
+  };
+  auto store_x = [&](int buf, const bf16x8 (&xr)[XF]) {
+#pragma unroll
+    for (int j = 0; j < XF; ++j) {
+      const int idx = threadIdx.x + 256 * j;
+      xs[buf][idx / (MB * 64)][idx / 64 % MB][idx % 64] = xr[j];
+    }
+  };
+  auto load_w = [&](int c, bf16x8 (&a)[NT][KC]) {
+#pragma unroll
+    for (int u = 0; u < KC; ++u) {
+      int ks = kbeg + c * KC + u;
+      if (ks >= kend) ks = kend - 1;               // its x is zero
+#pragma unroll
+      for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)ks);
+    }
+  };
+  f32x4 acc[NT][MB];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[t][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 a[NT][KC], a_next[NT][KC], xr[XF];
+  load_x(0, xr);
+  load_w(0, a);
+  store_x(0, xr);
+  for (int c = 0; c < nchunks; ++c) {
+    __syncthreads();
+    const bool more = c + 1 < nchunks;
+    if (more) {
+      load_x(c + 1, xr);
+      load_w(c + 1, a_next);
+    }
+#pragma unroll
+    for (int u = 0; u < KC; ++u)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const bf16x8 bv = xs[c & 1][u][b][lane];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv, acc[t][b], 0, 0, 0);
+      }
+    if (more) {
+      store_x((c + 1) & 1, xr);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int u = 0; u < KC; ++u) a[t][u] = a_next[t][u];
+    }
+  }
+  // lane: column m = 16 b + i of x, rows n = 16 tile + 4 gq + r of W
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (tile0 + t >= ntiles) continue;
+    const int n = (tile0 + t) * 16 + 4 * gq;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const int m = 16 * b + i;
+      if (gated) {
+        // rows 0..7 of a tile are gates, 8..15 their ups: lanes gq < 2 fetch the ups from gq + 2
+        f32x4 up;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) up[r] = __shfl(acc[t][b][r], lane + 32, 64);
+        if (gq < 2 && m < M) {
+          __bf16* o = (__bf16*)y + (size_t)m * (N / 2) + (tile0 + t) * 8 + 4 * gq;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float g = acc[t][b][r];
+            o[r] = (__bf16)(g / (1.f + expf(-g)) * up[r]);
+          }
+        }
+        continue;
+      }
+      if (m >= M) continue;
+      if (KS > 1) {
+        float* o = (float*)y + ((size_t)blockIdx.y * M + m) * N + n;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) o[r] = acc[t][b][r];
+        continue;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (n + r >= N) continue;
+        const float v = acc[t][b][r] + (bias != nullptr ? bias[n + r] : 0.f);
+        if (out_f32) ((float*)y)[(size_t)m * N + n + r] = v;
+        else ((__bf16*)y)[(size_t)m * N + n + r] = (__bf16)v;
+      }
+    }
+  }
+}
+
+__global__ void splitk_reduce_kernel(const float* __restrict__ part, const float* __restrict__ bias,
+                                     void* __restrict__ y, int M, int N, int KS, int out_f32) {
+  const size_t total = (size_t)M * N;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    float v = bias != nullptr ? bias[idx % N] : 0.f;
+    for (int j = 0; j < KS; ++j) v += part[(size_t)j * total + idx];
+    if (out_f32) ((float*)y)[idx] = v;
+    else ((__bf16*)y)[idx] = (__bf16)v;
+  }
+}
+
+// ks > 1: `part` holds ks * M * N floats.
+extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* bias, void* y,
+                                   int M, int N, int K, int out_f32, int gated, int ks,
+                                   float* part, hipStream_t stream) {
+  SL_CHECK(M > 0 && N > 0 && K > 0, "gemm_mid: sizes must be positive");
+  SL_CHECK(M <= 64, "gemm_mid: at most 64 rows");
+  SL_CHECK(K % 32 == 0, "gemm_mid: K must be a multiple of 32");
+  SL_CHECK(ks >= 1 && ks <= 16 && ks <= K / 32, "gemm_mid: ks must be in 1..16 and <= K / 32");
+  SL_CHECK(ks == 1 || part != nullptr, "gemm_mid: a split of K needs the partial buffer");
+  SL_CHECK(!gated || (ks == 1 && N % 16 == 0 && bias == nullptr && !out_f32),
+           "gemm_mid: the gated form needs ks == 1, N % 16 == 0, no bias, activation output");
+  SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
+           "gemm_mid: x and W must be 16-byte aligned");
+  const int ntiles = (N + 15) / 16;
+  const __bf16* xx = (const __bf16*)x;
+  const __bf16* ww = (const __bf16*)wt;
+  void* dst = ks > 1 ? (void*)part : y;
+  // two tiles per wavefront and chunks of four k-steps measured fastest (against 1 and 4 tiles, 8 k-steps)
+  const dim3 grid((ntiles + 7) / 8, ks);
+  if (M <= 32) gemm_mid_kernel<2, 2, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+  else gemm_mid_kernel<4, 2, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+  const char* e = sl_launch_status();
+  if (e || ks == 1) return e;
+  const size_t total = (size_t)M * N;
+  splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(part, bias, y, M, N, ks, out_f32);
+  return sl_launch_status();
+}
+
 // Row-major W [N, K] -> tiled [ceil(N / 16)][K / 32][64][8]; rows beyond N are zero.
 __global__ void tile_weight_kernel(const __bf16* __restrict__ w, __bf16* __restrict__ wt, int N,
                                    int K, size_t total_vec) {

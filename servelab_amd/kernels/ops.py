@@ -209,12 +209,33 @@ class HipOps:
                    int(out_f32), int(gated))
         return y
 
+    MID_TARGET_WORKGROUPS = 448
+    MID_MIN_ELEMENTS = 48 << 20   # matrices from this size on take the LDS-staged kernel at 17..64 rows
+
+    def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None):
+        """17..64 rows with x staged through LDS; K split over workgroups when
+        N alone gives too few of them."""
+        M, K = x.shape
+        N = weight.shape[0]
+        if weight.tiled is None:
+            raise KernelError("linear_mid needs the tiled copy of the weight")
+        wgs = -(-(-(-N // 16)) // 8)
+        if ks is None:
+            ks = 1 if gated else max(1, min(16, K // 32 // 4, -(-self.MID_TARGET_WORKGROUPS // wgs)))
+        part = self._new((ks, M, N), torch.float32) if ks > 1 else None
+        y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
+        self._call("gemm", "sl_gemm_mid", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
+                   int(out_f32), int(gated), int(ks), _p(part))
+        return y
+
     def linear_skinny(self, x, weight, bias, out_f32=False):
         M, K = x.shape
         N = weight.shape[0]
         if weight.tiled is None:
             raise KernelError("linear_skinny needs the tiled copy of the weight")
         if M >= self.WIDE_MIN_M:
+            if N * K >= self.MID_MIN_ELEMENTS:
+                return self.linear_mid(x, weight, bias, out_f32)
             return self.linear_wide(x, weight, bias, out_f32)
         y = self._new((M, N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
@@ -235,6 +256,8 @@ class HipOps:
                 and N % 16 == 0):
             self._check(x, self.act_dtype, None, "x")
             if M >= self.WIDE_MIN_M:
+                if N * K >= self.MID_MIN_ELEMENTS:
+                    return self.linear_mid(x, weight, None, gated=True)
                 return self.linear_wide(x, weight, None, gated=True)
             y = self._new((M, N // 2))
             self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), None, _p(y), M, N, K,

@@ -108,6 +108,27 @@ def test_linear_skinny(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048)])
+def test_linear_mid(M, N, K):
+    """The LDS-staged 17..64-row kernel alone: whole K and K split over up to
+    16 workgroups with the separate reduction, plain and gated."""
+    from servelab_amd.kernels import HipOps
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    x = randn(M, K, dtype=torch.bfloat16, seed=4)
+    w = randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5)
+    weight = ops.prepare_weight(w)
+    b = randn(N, seed=6)
+    ref = emu.linear(x, w, b, True)
+    for ks in (1, 2, 5, 16, None):
+        if ks and ks > K // 32:
+            continue
+        assert rel_err(ops.linear_mid(x, weight, b, out_f32=True, ks=ks), ref) < 2e-5, ks
+        assert rel_err(ops.linear_mid(x, weight, None, ks=ks), emu.linear(x, w, None)) < 2 ** -7, ks
+    if N % 16 == 0:
+        gated = ops.linear_mid(x, weight, None, gated=True)
+        assert rel_err(gated, emu.silu_mul(emu.linear(x, w, None), 8)) < 2 ** -6
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 144, 352), (64, 80, 2048)])
 def test_tiled_only_weights(M, N, K):
     """Only the tiled copy kept: few rows go straight to the matrix cores, many
     rows through the row-major scratch and the library; same results as with
