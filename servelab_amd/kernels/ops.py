@@ -284,12 +284,11 @@ class HipOps:
             raise KernelError("the library GEMM is for the bfloat16 table only")
         if bias is None:
             return torch.mm(x, w.t())
-        key = bias.data_ptr()
-        b = self._bias_cache.get(key)
-        if b is None or b.shape != bias.shape:
-            b = bias.to(torch.bfloat16)
-            self._bias_cache[key] = b
-        return torch.addmm(b, x, w.t())
+        entry = self._bias_cache.get(id(bias))       # (the float bias itself, its bfloat16 copy)
+        if entry is None or entry[0] is not bias:
+            entry = (bias, bias.to(torch.bfloat16))
+            self._bias_cache[id(bias)] = entry
+        return torch.addmm(entry[1], x, w.t())
 
     def silu_mul(self, gate_up, block=None):
         T, two_i = gate_up.shape
