@@ -170,75 +170,141 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // GATED: the 16 rows of a tile are 8 gate rows followed by the 8 up rows of the
 // same channels; the workgroup then writes silu(gate) * up, 8 columns of an
 // [M, N / 2] result, instead of 16 columns of y (servelab/parallel/tp_model.py:68).
-template <int MB, bool GATED>
+//
+// Residual add and RMSNorm fused into the products around them (decode steps
+// are bound by the number of kernels as much as by bytes):
+//   PRODUCER  the product's result is a delta of the residual stream.  The
+//             workgroup adds it to its 16 columns of the float stream, writes
+//             the stream times the next norm's gain in bfloat16 ("un-normalised
+//             rows": everything of y = x * rsqrt(mean x^2 + eps) * w but the
+//             rsqrt), and the sum of squares of its 16 columns per row into
+//             parts[workgroup][16].
+//   CONSUMER  x are such un-normalised rows; the workgroup first adds up the
+//             parts in a fixed order (so the result does not depend on timing),
+//             and scales row m of the result by rsqrt(sum / K + eps) before
+//             the bias.  `rows` optionally picks which rows of x are multiplied.
+#define SL_MAX_PARTS_PER_THREAD 16      // 32 * 16 parts of 16 columns: rows of up to 8192 values
+                                        // (8 per thread, and fewer registers, for rows of up to 4096)
+
+struct NormFusion {
+  const float* in_parts;     // CONSUMER: [in_nparts][16] sums of squares by row
+  int in_nparts;
+  float eps;
+  const int* rows;           // CONSUMER: result row m reads row rows[m] of x, or nullptr
+  float* resid;              // PRODUCER: float stream [M, N], updated in place
+  const float* next_w;       // PRODUCER: gain of the norm that reads the stream next [N]
+  float* out_parts;          // PRODUCER: [gridDim.x][16]
+};
+
+template <bool GATED, bool CONSUMER, bool PRODUCER, int PARTS>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
-    void* __restrict__ y, int M, int N, int K, int out_f32) {
+    void* __restrict__ y, int M, int N, int K, int out_f32, const NormFusion F) {
   constexpr int WAVES = 8, U = 8;
-  __shared__ f32x4 red[WAVES][MB][64];
+  __shared__ f32x4 red[WAVES][64];
+  __shared__ float wsum[WAVES][16];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const int KT = K / 32;
   const int ks0 = (int)((long long)KT * wave / WAVES), ks1 = (int)((long long)KT * (wave + 1) / WAVES);
   const __bf16* wp = wt + ((size_t)blockIdx.x * KT * 64 + lane) * 8;
-  const __bf16* xp[MB];
+  int xrow = i < M ? i : M - 1;
+  if (CONSUMER && F.rows != nullptr) xrow = F.rows[xrow];
+  const __bf16* xp = x + (size_t)xrow * K + 8 * gq;
+  // Loads that only the epilogue needs are issued here, before W streams, so
+  // that their latency is hidden: the consumer's share of the sums of squares
+  // (thread t takes parts t / 16, t / 16 + 32, ... of row t % 16) and the
+  // producer's elements of the stream and of the next gain.
+  float pv[PARTS];
+  if (CONSUMER) {
 #pragma unroll
-  for (int b = 0; b < MB; ++b) {
-    const int m = 16 * b + i < M ? 16 * b + i : M - 1;
-    xp[b] = x + (size_t)m * K + 8 * gq;
+    for (int j = 0; j < PARTS; ++j) {
+      const int p = threadIdx.x / 16 + 32 * j;
+      pv[j] = p < F.in_nparts ? F.in_parts[p * 16 + i] : 0.f;
+    }
   }
-  f32x4 acc[MB];
-#pragma unroll
-  for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int em = threadIdx.x / 16, en = n0 + threadIdx.x % 16;       // epilogue element of threads < 256
+  float r_old = 0.f, g_next = 0.f;
+  if (PRODUCER && threadIdx.x < 256 && em < M && en < N) {
+    r_old = F.resid[(size_t)em * N + en];
+    g_next = F.next_w[en];
+  }
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   int ks = ks0;
   for (; ks + U <= ks1; ks += U) {
     bf16x8 a[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) a[u] = *(const bf16x8*)(wp + 512 * (size_t)(ks + u));
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int b = 0; b < MB; ++b) {
-        const bf16x8 bv = *(const bf16x8*)(xp[b] + 32 * (size_t)(ks + u));
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[b], 0, 0, 0);
-      }
+    for (int u = 0; u < U; ++u) {
+      const bf16x8 bv = *(const bf16x8*)(xp + 32 * (size_t)(ks + u));
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc, 0, 0, 0);
+    }
   }
   for (; ks < ks1; ++ks) {
     const bf16x8 a = *(const bf16x8*)(wp + 512 * (size_t)ks);
-#pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const bf16x8 bv = *(const bf16x8*)(xp[b] + 32 * (size_t)ks);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bv, acc[b], 0, 0, 0);
-    }
+    const bf16x8 bv = *(const bf16x8*)(xp + 32 * (size_t)ks);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bv, acc, 0, 0, 0);
   }
+  red[wave][lane] = acc;
+  if (CONSUMER) {            // this wavefront's share of the sums of squares, by row
+    float sacc = 0.f;
 #pragma unroll
-  for (int b = 0; b < MB; ++b) red[wave][b][lane] = acc[b];
+    for (int j = 0; j < PARTS; ++j) sacc += pv[j];
+    sacc += __shfl_xor(sacc, 16, 64);
+    sacc += __shfl_xor(sacc, 32, 64);
+    if (lane < 16) wsum[wave][lane] = sacc;
+  }
   __syncthreads();
-  // lane (m_local + 16 (n_local / 4)) holds y[m_local, n_local] in element n_local % 4
+  auto inv_of = [&](int m) {   // rsqrt(mean x^2 + eps) of the row of x behind result row m
+    const int tok = F.rows != nullptr ? F.rows[m] : m;
+    float ss = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) ss += wsum[wv][tok];
+    return rsqrtf(ss / (float)K + F.eps);
+  };
+  // lane (m + 16 (n_local / 4)) holds y[m, n_local] in element n_local % 4
   if (GATED) {
-    for (int idx = threadIdx.x; idx < MB * 128; idx += WAVES * 64) {
-      const int b = idx / 128, rem = idx % 128, m_local = rem / 8, j = rem % 8;
-      const int m = 16 * b + m_local, n = blockIdx.x * 8 + j;
+    if (threadIdx.x < 128) {
+      const int m = threadIdx.x / 8, j = threadIdx.x % 8;
+      const int n = blockIdx.x * 8 + j;
       if (m < M && n < N / 2) {
         float gsum = 0.f, usum = 0.f;
 #pragma unroll
         for (int wv = 0; wv < WAVES; ++wv) {
-          gsum += red[wv][b][m_local + 16 * (j / 4)][j % 4];
-          usum += red[wv][b][m_local + 16 * (2 + j / 4)][j % 4];
+          gsum += red[wv][m + 16 * (j / 4)][j % 4];
+          usum += red[wv][m + 16 * (2 + j / 4)][j % 4];
+        }
+        if (CONSUMER) {
+          const float inv = inv_of(m);
+          gsum *= inv;
+          usum *= inv;
         }
         ((__bf16*)y)[(size_t)m * (N / 2) + n] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
       }
     }
     return;
   }
-  for (int idx = threadIdx.x; idx < MB * 256; idx += WAVES * 64) {
-    const int b = idx / 256, rem = idx % 256, m_local = rem / 16, n_local = rem % 16;
-    const int m = 16 * b + m_local, n = n0 + n_local;
-    if (m < M && n < N) {
-      float s = 0.f;
+  if (threadIdx.x < 256) {
+    const int m = em, n_local = threadIdx.x % 16, n = en;
+    const bool live = m < M && n < N;
+    float s = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < WAVES; ++wv) s += red[wv][b][m_local + 16 * (n_local / 4)][n_local % 4];
-      if (bias != nullptr) s += bias[n];
+    for (int wv = 0; wv < WAVES; ++wv) s += red[wv][m + 16 * (n_local / 4)][n_local % 4];
+    if (CONSUMER && live) s *= inv_of(m);
+    if (live && bias != nullptr) s += bias[n];
+    if (PRODUCER) {
+      float sq = 0.f;
+      if (live) {
+        const float r = r_old + s;
+        F.resid[(size_t)m * N + n] = r;
+        ((__bf16*)y)[(size_t)m * N + n] = (__bf16)(r * g_next);
+        sq = r * r;
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);     // over the 16 columns of row m
+      if (n_local == 0) F.out_parts[(size_t)blockIdx.x * 16 + m] = sq;
+    } else if (live) {
       if (out_f32) ((float*)y)[(size_t)m * N + n] = s;
       else ((__bf16*)y)[(size_t)m * N + n] = (__bf16)s;
     }
@@ -246,29 +312,41 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
 }
 
 // wt: W in the tiled layout, ceil(N / 16) * 16 rows (rows beyond N are zero).
+// At most 16 rows.  Fusion: in_parts != nullptr makes x un-normalised rows
+// (consumer), resid != nullptr makes the result a delta of the stream (producer).
 extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float* bias, void* y,
                                       int M, int N, int K, int out_f32, int gated,
-                                      hipStream_t stream) {
+                                      const float* in_parts, int in_nparts, float eps,
+                                      const int* rows, float* resid, const float* next_w,
+                                      float* out_parts, hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
+  SL_CHECK(M <= 16, "gemm_skinny: at most 16 rows");
+  SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
   SL_CHECK(!gated || (N % 16 == 0 && bias == nullptr && !out_f32),
            "gemm_skinny: the gated form needs N % 16 == 0, no bias, activation output");
-  SL_CHECK(M <= 64, "gemm_skinny: at most 64 rows");
-  SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
            "gemm_skinny: x and W must be 16-byte aligned");
+  const bool consumer = in_parts != nullptr, producer = resid != nullptr;
+  SL_CHECK(!(consumer && producer), "gemm_skinny: a product is a consumer or a producer, not both");
+  SL_CHECK(!consumer || (in_nparts > 0 && eps > 0.f), "gemm_skinny: a consumer needs parts and eps");
+  SL_CHECK(!consumer || in_nparts <= 32 * SL_MAX_PARTS_PER_THREAD,
+           "gemm_skinny: un-normalised rows of more than 8192 values");
+  SL_CHECK(rows == nullptr || consumer, "gemm_skinny: a row gather belongs to a consumer");
+  SL_CHECK(!producer || (next_w != nullptr && out_parts != nullptr && !gated && !out_f32),
+           "gemm_skinny: a producer needs the next gain and a parts buffer, and is neither gated nor float");
   if (M == 0) return nullptr;
   const dim3 grid((N + 15) / 16);
   const __bf16* xx = (const __bf16*)x;
   const __bf16* ww = (const __bf16*)wt;
-  if (gated) {
-    if (M <= 16) gemm_skinny_kernel<1, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
-    else if (M <= 32) gemm_skinny_kernel<2, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
-    else gemm_skinny_kernel<4, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0);
-    return sl_launch_status();
-  }
-  if (M <= 16) gemm_skinny_kernel<1, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
-  else if (M <= 32) gemm_skinny_kernel<2, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
-  else gemm_skinny_kernel<4, false><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+  const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts};
+  const bool few = in_nparts <= 32 * 8;
+  if (producer) gemm_skinny_kernel<false, false, true, 1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);
+  else if (consumer && gated && few) gemm_skinny_kernel<true, true, false, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);
+  else if (consumer && gated) gemm_skinny_kernel<true, true, false, 16><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);
+  else if (consumer && few) gemm_skinny_kernel<false, true, false, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F);
+  else if (consumer) gemm_skinny_kernel<false, true, false, 16><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F);
+  else if (gated) gemm_skinny_kernel<true, false, false, 1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);
+  else gemm_skinny_kernel<false, false, false, 1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F);
   return sl_launch_status();
 }
 

@@ -40,6 +40,32 @@ class LinearWeight:
         self.shape = tuple(w.shape) if w is not None else tuple(shape)
 
 
+class Deferred:
+    """A product whose result is only ever added to the residual stream; the
+    norm that takes it as its delta runs it, fused with the add and the norm
+    (``HipOps.add_rmsnorm(..., fuse=True)``) or plainly (``materialize``)."""
+    __slots__ = ("x", "weight", "bias")
+
+    def __init__(self, x, weight, bias):
+        self.x, self.weight, self.bias = x, weight, bias
+
+
+class ScaledRows:
+    """Rows [T, H] that are normalised but for the factor rsqrt(mean x^2 + eps):
+    ``x`` holds stream * gain in the activation dtype, ``parts`` [nparts, 16] the
+    sums of squares of the stream by row.  Only ``linear`` and ``gated_linear``
+    read them: they scale their result rows instead.  ``rows`` optionally
+    selects which rows take part."""
+    __slots__ = ("x", "parts", "eps", "rows")
+
+    def __init__(self, x, parts, eps, rows=None):
+        self.x, self.parts, self.eps, self.rows = x, parts, eps, rows
+
+    @property
+    def shape(self):
+        return (self.rows.shape[0] if self.rows is not None else self.x.shape[0], self.x.shape[1])
+
+
 class HipOps:
     ROWS_KERNEL_MAX_M = 16        # the wavefront-per-column GEMM is used up to this many rows
     SKINNY_MAX_M = 64             # the matrix-core few-rows GEMM takes up to this many rows
@@ -71,6 +97,7 @@ class HipOps:
         self._fn = {}
         self._bias_cache = {}
         self.use_mfma_attention = True
+        self.fuse_norms = act_dtype == torch.bfloat16
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
         self._untiled = None          # scratch for "tiled": the row-major form of one matrix
 
@@ -109,10 +136,17 @@ class HipOps:
         return out
 
     # ---------------------------------------------------------------- norms
-    def add_rmsnorm(self, resid, delta, weight, eps):
+    def add_rmsnorm(self, resid, delta, weight, eps, fuse=False):
+        """resid += delta (in place, float32); returns the normed rows.  A
+        ``Deferred`` delta is run here; with ``fuse`` (the reader takes
+        ``ScaledRows``) the product, the add and the norm are one kernel."""
         T, H = resid.shape
         self._check(resid, torch.float32, None, "residual stream")
         self._check(weight, torch.float32, (H,), "norm weight")
+        if isinstance(delta, Deferred):
+            if fuse:
+                return self._produce_scaled_rows(resid, delta, weight, eps)
+            delta = self.materialize(delta)
         if delta is not None:
             self._check(delta, self.act_dtype, (T, H), "delta")
         out = self._new((T, H))
@@ -120,18 +154,47 @@ class HipOps:
                    T, H, _c_float(eps))
         return out
 
-    def rows_add_rmsnorm(self, resid, delta, rows, weight, eps):
+    def rows_add_rmsnorm(self, resid, delta, rows, weight, eps, fuse=False):
+        """The normed rows ``rows`` of resid + delta.  The stream is left as it
+        is, except that a fused ``Deferred`` delta is added into it."""
         T, H = resid.shape
         R = rows.shape[0]
         self._check(resid, torch.float32, None, "residual stream")
         self._check(weight, torch.float32, (H,), "norm weight")
         self._check(rows, torch.int32, (R,), "rows")
+        if isinstance(delta, Deferred):
+            if fuse and R <= 16:
+                scaled = self._produce_scaled_rows(resid, delta, weight, eps)
+                scaled.rows = rows
+                return scaled
+            delta = self.materialize(delta)
         if delta is not None:
             self._check(delta, self.act_dtype, (T, H), "delta")
         out = self._new((R, H))
         self._call("norm", "sl_add_rmsnorm", _p(resid), _p(delta), _p(rows), _p(weight), _p(out),
                    R, H, _c_float(eps))
         return out
+
+    def materialize(self, value):
+        """The plain tensor of a ``Deferred`` product (anything else is returned as it is)."""
+        if isinstance(value, Deferred):
+            return self.linear(value.x, value.weight, value.bias)
+        return value
+
+    def _produce_scaled_rows(self, resid, d, gain, eps):
+        x, weight = d.x, d.weight
+        M, K = x.shape
+        N = weight.shape[0]
+        if tuple(resid.shape) != (M, N):
+            raise KernelError(f"a delta of shape {[M, N]} does not fit the stream {list(resid.shape)}")
+        self._check(x, self.act_dtype, None, "x")
+        if d.bias is not None:
+            self._check(d.bias, torch.float32, (N,), "bias")
+        out = self._new((M, N))
+        parts = self._new((-(-N // 16), 16), torch.float32)
+        self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(d.bias), _p(out), M, N, K,
+                   0, 0, None, 0, _c_float(0.0), None, _p(resid), _p(gain), _p(parts))
+        return ScaledRows(out, parts, eps)
 
     # --------------------------------------------------------------- linear
     def plan_weights(self, total_bytes: int) -> str:
@@ -169,12 +232,21 @@ class HipOps:
         self._call("gemm", "sl_untile_weight", _p(weight.tiled), _p(out), N, K)
         return out
 
-    def linear(self, x, weight, bias, out_f32=False):
-        """y = x W^T (+ bias); ``weight`` is a LinearWeight or a plain [N, K] tensor."""
+    FUSED_NORM_MAX_M = 16         # the fused add + norm lives in the kernel for up to 16 rows
+
+    def linear(self, x, weight, bias, out_f32=False, defer=False):
+        """y = x W^T (+ bias); ``weight`` is a LinearWeight or a plain [N, K] tensor.
+        ``defer``: y will only be added to the residual stream, so the product
+        may be left to the norm that adds it (a ``Deferred`` comes back then)."""
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
+        if isinstance(x, ScaledRows):
+            return self._linear_scaled(x, weight, bias, out_f32, False)
         M, K = x.shape
         N = weight.shape[0]
+        if (defer and self.fuse_norms and not out_f32 and 0 < M <= self.FUSED_NORM_MAX_M
+                and weight.tiled is not None and weight.shape == (N, K) and N <= 8192):
+            return Deferred(x, weight, bias)
         self._check(x, self.act_dtype, None, "x")
         if weight.shape != (N, K):
             raise KernelError(f"weight has shape {list(weight.shape)}, x has {K} columns")
@@ -239,7 +311,22 @@ class HipOps:
             return self.linear_wide(x, weight, bias, out_f32)
         y = self._new((M, N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
-                   int(out_f32), 0)
+                   int(out_f32), 0, None, 0, _c_float(0.0), None, None, None, None)
+        return y
+
+    def _linear_scaled(self, xs, weight, bias, out_f32, gated):
+        """The consumer of un-normalised rows: one few-rows product that scales
+        its result rows by rsqrt(mean x^2 + eps)."""
+        M, K = xs.shape
+        N = weight.shape[0]
+        if weight.tiled is None or weight.shape != (N, K) or M > self.FUSED_NORM_MAX_M:
+            raise KernelError("un-normalised rows need a tiled weight and at most 16 rows")
+        if bias is not None:
+            self._check(bias, torch.float32, (N,), "bias")
+        y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
+        self._call("gemm", "sl_gemm_skinny", _p(xs.x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
+                   int(out_f32), int(gated), _p(xs.parts), xs.parts.shape[0], _c_float(xs.eps),
+                   _p(xs.rows), None, None, None)
         return y
 
     GATE_BLOCK = 8                # gate and up rows alternate in blocks of 8 (half an MFMA tile)
@@ -250,6 +337,10 @@ class HipOps:
         Few rows and a tiled weight with blocks of 8: one fused kernel."""
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
+        if isinstance(x, ScaledRows):
+            if block != self.GATE_BLOCK or weight.shape[0] % 16:
+                raise KernelError("un-normalised rows need gate and up in blocks of 8")
+            return self._linear_scaled(x, weight, None, False, True)
         M, K = x.shape
         N = weight.shape[0]
         if (M <= self.SKINNY_MAX_M and weight.tiled is not None and block == self.GATE_BLOCK
@@ -261,7 +352,7 @@ class HipOps:
                 return self.linear_wide(x, weight, None, gated=True)
             y = self._new((M, N // 2))
             self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), None, _p(y), M, N, K,
-                       0, 1)
+                       0, 1, None, 0, _c_float(0.0), None, None, None, None)
             return y
         return self.silu_mul(self.linear(x, weight, None), block)
 

@@ -18,6 +18,7 @@ from .base import Mixer, PagedKVSpec, ParamSpec
 
 class PagedAttention(Mixer):
     graph_safe = True
+    takes_scaled_rows = True
 
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, position,
                  qkv_bias=True, window=None, scale=None):
@@ -77,4 +78,4 @@ class PagedAttention(Mixer):
         attn = ops.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
             cache.page_size, group.block_tables, batch, self.scale, self.window)
-        return ops.linear(attn, self.w_o, None)
+        return ops.linear(attn, self.w_o, None, defer=True)

@@ -86,13 +86,19 @@ class Part:
 class Norm(Part):
     """forward(resid, delta) adds ``delta`` (or nothing) into the float32
     residual stream in place and returns the normed rows in the activation
-    dtype; forward_rows does the same for selected rows without changing the
-    stream."""
+    dtype; forward_rows returns the normed selected rows.
 
-    def forward(self, resid, delta):
+    ``delta`` is what the part before returned: a tensor, or a product the
+    kernel table deferred (``ops.linear(..., defer=True)``), which the norm's
+    kernel call runs.  ``fuse`` says that the reader of the normed rows passes
+    them only to ``ops.linear`` / ``ops.gated_linear`` (it has
+    ``takes_scaled_rows``); the kernel table may then hand it rows whose
+    normalisation the reader's product completes."""
+
+    def forward(self, resid, delta, fuse=False):
         raise NotImplementedError
 
-    def forward_rows(self, resid, delta, rows):
+    def forward_rows(self, resid, delta, rows, fuse=False):
         raise NotImplementedError
 
 
@@ -106,12 +112,15 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    """Sequence mixer.  ``cache_spec`` declares its per-request cache need
+    """Sequence mixer.  ``takes_scaled_rows``: forward hands ``x`` to nothing but
+    ``ops.linear`` / ``ops.gated_linear`` (same flag on FeedForward and the head).  ``cache_spec`` declares its per-request cache need
     (PagedKVSpec, StateSpec or None); ``forward(x, batch, cache, shared)`` maps
     normed rows [T, H] to rows [T, H].  ``cache`` is the binding the cache
     manager made for the layer call: pages plus block tables, or state plus
     slot ids; ``cache.write`` is False when the call reads another call's
     cache."""
+
+    takes_scaled_rows = False
 
     def cache_spec(self):
         return None
@@ -121,7 +130,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """forward(x [T, H]) -> [T, H]."""
+    """forward(x [T, H]) -> [T, H] (or a deferred product of that shape)."""
+
+    takes_scaled_rows = False
 
     def forward(self, x):
         raise NotImplementedError

@@ -34,7 +34,7 @@ class PreNormBlock(Block):
             part.load(prefixed(prefix, tensors), rt)
 
     def forward(self, resid, delta, batch, cache, shared):
-        x = self.norm1.forward(resid, delta)
+        x = self.norm1.forward(resid, delta, fuse=self.mixer.takes_scaled_rows)
         a = self.mixer.forward(x, batch, cache, shared)
-        x2 = self.norm2.forward(resid, a)
+        x2 = self.norm2.forward(resid, a, fuse=self.feedforward.takes_scaled_rows)
         return self.feedforward.forward(x2)

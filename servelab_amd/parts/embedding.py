@@ -27,6 +27,7 @@ class TokenEmbedding(Part):
 
 class OutputHead(Part):
     graph_safe = True
+    takes_scaled_rows = True
 
     """``tied_to`` is the embedding part whose table the head shares, or None."""
 

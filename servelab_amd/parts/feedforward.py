@@ -13,6 +13,7 @@ from .base import FeedForward, ParamSpec
 
 class GatedMLP(FeedForward):
     graph_safe = True
+    takes_scaled_rows = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         if activation != "silu":
@@ -40,4 +41,5 @@ class GatedMLP(FeedForward):
 
     def forward(self, x):
         ops = self.rt.ops
-        return ops.linear(ops.gated_linear(x, self.w_gate_up, self.block), self.w_down, None)
+        return ops.linear(ops.gated_linear(x, self.w_gate_up, self.block), self.w_down, None,
+                          defer=True)

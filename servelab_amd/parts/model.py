@@ -125,5 +125,6 @@ class DecoderModel:
         if batch.num_logit_rows == 0:
             # the last block's output is never read; nothing to add
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.rt.device)
-        rows = spec.final_norm[1].forward_rows(resid, delta, batch.logit_rows)
+        rows = spec.final_norm[1].forward_rows(resid, delta, batch.logit_rows,
+                                               fuse=getattr(spec.head[1], "takes_scaled_rows", False))
         return spec.head[1].forward(rows)

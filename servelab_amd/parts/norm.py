@@ -21,8 +21,8 @@ class RMSNorm(Norm):
         self.rt = rt
         self.weight = rt.vector(tensors("weight"))
 
-    def forward(self, resid, delta):
-        return self.rt.ops.add_rmsnorm(resid, delta, self.weight, self.eps)
+    def forward(self, resid, delta, fuse=False):
+        return self.rt.ops.add_rmsnorm(resid, delta, self.weight, self.eps, fuse=fuse)
 
-    def forward_rows(self, resid, delta, rows):
-        return self.rt.ops.rows_add_rmsnorm(resid, delta, rows, self.weight, self.eps)
+    def forward_rows(self, resid, delta, rows, fuse=False):
+        return self.rt.ops.rows_add_rmsnorm(resid, delta, rows, self.weight, self.eps, fuse=fuse)

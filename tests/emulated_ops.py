@@ -25,13 +25,13 @@ class EmulatedOps:
         return _f(table[ids.long()])
 
     # ---------------------------------------------------------------- norms
-    def add_rmsnorm(self, resid, delta, weight, eps):
+    def add_rmsnorm(self, resid, delta, weight, eps, fuse=False):
         if delta is not None:
             resid += _f(delta)
         var = resid.pow(2).mean(-1, keepdim=True)
         return (resid * torch.rsqrt(var + eps) * weight).to(self.act_dtype)
 
-    def rows_add_rmsnorm(self, resid, delta, rows, weight, eps):
+    def rows_add_rmsnorm(self, resid, delta, rows, weight, eps, fuse=False):
         x = resid[rows.long()]
         if delta is not None:
             x = x + _f(delta[rows.long()])
@@ -39,7 +39,7 @@ class EmulatedOps:
         return (x * torch.rsqrt(var + eps) * weight).to(self.act_dtype)
 
     # --------------------------------------------------------------- linear
-    def linear(self, x, w, bias, out_f32=False):
+    def linear(self, x, w, bias, out_f32=False, defer=False):
         y = _f(x) @ _f(w).T
         if bias is not None:
             y = y + bias

@@ -210,6 +210,53 @@ def test_gated_linear(both, M, I, K):
         assert rel_err(ops.silu_mul(ops.linear(x, w, None), block), ref) < tol
 
 
+@pytest.mark.parametrize("M,H,N2", [(1, 64, 96), (8, 3584, 4608), (16, 200 * 32, 48), (5, 96, 1000)])
+def test_fused_add_norm_around_few_rows_products(M, H, N2):
+    """A deferred product run by the norm that adds it (stream += x W1^T, rows
+    left un-normalised, sums of squares by workgroup) and the products that
+    read such rows (plain with bias, gated, float output with a row gather):
+    same results as product, add, norm and product one after the other."""
+    from servelab_amd.kernels import HipOps
+    from servelab_amd.kernels.ops import Deferred, ScaledRows
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    K1 = 128
+    x = randn(M, K1, dtype=torch.bfloat16, seed=1)
+    w1 = ops.prepare_weight(randn(H, K1, dtype=torch.bfloat16, scale=0.1, seed=2))
+    gain = 1 + 0.1 * randn(H, seed=3)
+    resid0 = randn(M, H, seed=4)
+    eps = 1e-5
+    # reference: the unfused sequence in float32 with the same roundings of inputs
+    delta = x.float() @ w1.w.float().T
+    stream = resid0 + delta
+    normed = stream * torch.rsqrt(stream.pow(2).mean(-1, keepdim=True) + eps) * gain
+    resid = resid0.clone()
+    deferred = ops.linear(x, w1, None, defer=True)
+    assert isinstance(deferred, Deferred)
+    scaled = ops.add_rmsnorm(resid, deferred, gain, eps, fuse=True)
+    assert isinstance(scaled, ScaledRows) and scaled.shape == (M, H)
+    assert rel_err(resid, stream) < 1e-5
+    w2 = ops.prepare_weight(randn(N2, H, dtype=torch.bfloat16, scale=0.05, seed=5))
+    b2 = randn(N2, seed=6)
+    ref = normed @ w2.w.float().T + b2
+    assert rel_err(ops.linear(scaled, w2, b2), ref) < 2 ** -6
+    assert rel_err(ops.linear(scaled, w2, b2, out_f32=True), ref) < 2 ** -7
+    if N2 % 16 == 0:
+        got = ops.gated_linear(scaled, w2, 8)
+        assert rel_err(got, emu.silu_mul((normed @ w2.w.float().T).to(torch.bfloat16), 8)) < 2 ** -5
+    # the same deferred product without a reader of scaled rows, and row-gathered for a head
+    resid = resid0.clone()
+    plain_rows = ops.add_rmsnorm(resid, ops.linear(x, w1, None, defer=True), gain, eps)
+    assert torch.is_tensor(plain_rows) and rel_err(plain_rows, normed) < 2 ** -6
+    rows = torch.tensor([M - 1, 0][:min(2, M)], dtype=torch.int32).cuda()
+    resid = resid0.clone()
+    picked = ops.rows_add_rmsnorm(resid, ops.linear(x, w1, None, defer=True), rows, gain, eps, fuse=True)
+    assert isinstance(picked, ScaledRows) and picked.shape == (rows.shape[0], H)
+    assert rel_err(ops.linear(picked, w2, None, out_f32=True), normed[rows.long()] @ w2.w.float().T) < 2 ** -7
+    # more rows than the fused kernels take: the product is simply done
+    big = randn(17, K1, dtype=torch.bfloat16, seed=7)
+    assert torch.is_tensor(ops.linear(big, w1, None, defer=True))
+
+
 def test_rope_tables(both):
     ops, emu, dt = both
     D, theta = 48, 1e6

@@ -79,7 +79,7 @@ def test_gated_mlp_part(rt):
     for rows in (3, 70):
         x = rand(rows, 96, seed=4).to(runtime.act_dtype)
         ref = plain.swiglu(x.float(), t["gate_proj.weight"], t["up_proj.weight"], t["down_proj.weight"])
-        assert rel(ffn.forward(x.cuda()), ref) < TOL[name]
+        assert rel(runtime.ops.materialize(ffn.forward(x.cuda())), ref) < TOL[name]
     with pytest.raises(ValueError):
         GatedMLP(96, 200, activation="gelu")
 
@@ -146,7 +146,8 @@ def test_attention_part_in_portions(rt, nh, nkv, D, bias, theta, window):
     for n in (20, 1, 33, 2, 19):
         manager.grow("r", start + n)
         batch = pack_batch([StepEntry("r", [0] * n, [])], [start], [], manager, runtime.device)
-        got.append(mixer.forward(x[start:start + n].cuda().contiguous(), batch, binding, {}))
+        got.append(runtime.ops.materialize(
+            mixer.forward(x[start:start + n].cuda().contiguous(), batch, binding, {})))
         manager.commit("r", start + n)
         start += n
     assert rel(torch.cat(got), ref) < TOL[name]
@@ -171,7 +172,7 @@ def test_block_part(rt):
     h = rand(T, H, seed=20)
     pending = rand(T, H, scale=0.1, seed=21).to(runtime.act_dtype)
     resid = h.cuda()
-    delta = block.forward(resid, pending.cuda(), batch, pool.binding(0, True), {})
+    delta = runtime.ops.materialize(block.forward(resid, pending.cuda(), batch, pool.binding(0, True), {}))
     h0 = h + pending.float()
     att = {n[len("self_attn."):]: v for n, v in t.items() if n.startswith("self_attn.")}
     h1 = h0 + plain_attention_layer(plain.rms_norm(h0, t["input_layernorm.weight"], 1e-6), att,
