@@ -123,10 +123,16 @@ extern "C" const char* sl_rope_tables(const int* pos, const float* inv_freq, flo
 // rotated k and the v of each token go to its cache row (:129,
 // servelab/kv_cache/pool.py:68-78): K pages [page, nkv, page_size, D], V pages
 // [page, nkv, D, page_size].  One block per (token, head).
+//
+// pairs8: the channels of every q and k head come in the order the fused
+// few-rows product wants them (gemm.hip): blocks of 16 that hold channels
+// 8b..8b+7 followed by their partners D/2+8b..D/2+8b+7, so that pair j sits at
+// 16 (j / 8) + j % 8 and 8 further.  Scores do not depend on the order of the
+// channels as long as q and the cached k agree; v keeps its order.
 __global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restrict__ cosv,
                                   const float* __restrict__ sinv, const int* __restrict__ slots,
                                   act_t* __restrict__ kc, act_t* __restrict__ vc, int nh, int nkv,
-                                  int D, int page) {
+                                  int D, int page, int pairs8) {
   const int t = blockIdx.x, hd = blockIdx.y;
   const int half = D / 2;
   act_t* x = qkv + ((size_t)t * (nh + 2 * nkv) + hd) * D;
@@ -137,18 +143,20 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restri
       dst = kc + (((size_t)(slot / page) * nkv + (hd - nh)) * page + slot % page) * D;
     }
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
-      float x1 = to_f(x[j]), x2 = to_f(x[j + half]);
+      const int p1 = pairs8 ? 16 * (j / 8) + j % 8 : j;
+      const int p2 = pairs8 ? p1 + 8 : j + half;
+      float x1 = to_f(x[p1]), x2 = to_f(x[p2]);
       if (cosv != nullptr) {
         const float c = cosv[(size_t)t * half + j], s = sinv[(size_t)t * half + j];
         const float r1 = x1 * c - x2 * s, r2 = x2 * c + x1 * s;
         x1 = r1;
         x2 = r2;
-        x[j] = from_f<act_t>(x1);
-        x[j + half] = from_f<act_t>(x2);
+        x[p1] = from_f<act_t>(x1);
+        x[p2] = from_f<act_t>(x2);
       }
       if (dst != nullptr) {
-        dst[j] = from_f<act_t>(x1);
-        dst[j + half] = from_f<act_t>(x2);
+        dst[p1] = from_f<act_t>(x1);
+        dst[p2] = from_f<act_t>(x2);
       }
     }
   } else if (vc != nullptr) {
@@ -160,16 +168,17 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restri
 
 extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* sinv,
                                      const int* slots, void* kc, void* vc, int T, int nh, int nkv,
-                                     int D, int page, hipStream_t stream) {
+                                     int D, int page, int pairs8, hipStream_t stream) {
   SL_CHECK(T >= 0 && nh > 0 && nkv > 0, "rope_store: sizes must be positive");
   SL_CHECK(D > 0 && D % 2 == 0, "rope_store: head_dim must be even");
+  SL_CHECK(!pairs8 || D % 16 == 0, "rope_store: the blocked pair order needs head_dim % 16 == 0");
   SL_CHECK((cosv == nullptr) == (sinv == nullptr), "rope_store: cos and sin go together");
   SL_CHECK((kc == nullptr) == (vc == nullptr), "rope_store: k and v pages go together");
   SL_CHECK(kc == nullptr || (slots != nullptr && page > 0), "rope_store: pages need slots");
   if (T == 0) return nullptr;
   const int heads = kc != nullptr ? nh + 2 * nkv : nh + nkv;
   if (cosv == nullptr && kc == nullptr) return nullptr;
-  rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, cosv, sinv, slots,
-                                                       (act_t*)kc, (act_t*)vc, nh, nkv, D, page);
+  rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, cosv, sinv, slots, (act_t*)kc,
+                                                       (act_t*)vc, nh, nkv, D, page, pairs8);
   return sl_launch_status();
 }

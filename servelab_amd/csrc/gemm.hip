@@ -196,10 +196,27 @@ struct NormFusion {
   float* out_parts;          // PRODUCER: [gridDim.x][16]
 };
 
-template <bool GATED, bool CONSUMER, bool PRODUCER, int PARTS>
+// Rotary embedding and the write to the cache pages fused into the q/k/v
+// product (ROPE): the rows of W are ordered so that a tile of 16 result columns
+// of a q or k head holds channels 8b..8b+7 and their partners D/2+8b..D/2+8b+7;
+// the epilogue rotates each pair, writes q into the result buffer and the
+// rotated k and the v of token m into the cache row slots[m]
+// (servelab/parallel/tp_model.py:128-129).  q and the cached k keep that
+// channel order (scores do not depend on it); v is in its own order.
+struct RopeStore {
+  const float* cosv;         // [M, D / 2] or nullptr (no rotation)
+  const float* sinv;
+  const int* slots;          // [M] cache rows, or nullptr (nothing is written)
+  __bf16* kc;                // [pages, nkv, page, D]
+  __bf16* vc;                // [pages, nkv, D, page]
+  int nh, nkv, D, page;
+};
+
+template <bool GATED, bool CONSUMER, bool PRODUCER, int PARTS, bool ROPE = false>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
-    void* __restrict__ y, int M, int N, int K, int out_f32, const NormFusion F) {
+    void* __restrict__ y, int M, int N, int K, int out_f32, const NormFusion F,
+    const RopeStore R = RopeStore{}) {
   constexpr int WAVES = 8, U = 8;
   __shared__ f32x4 red[WAVES][64];
   __shared__ float wsum[WAVES][16];
@@ -293,6 +310,29 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     for (int wv = 0; wv < WAVES; ++wv) s += red[wv][m + 16 * (n_local / 4)][n_local % 4];
     if (CONSUMER && live) s *= inv_of(m);
     if (live && bias != nullptr) s += bias[n];
+    if (ROPE) {
+      const float partner = __shfl_xor(s, 8, 64);      // the other half of the pair, same row
+      if (!live) return;
+      const int hd = n / R.D, p = n % R.D;
+      if (hd < R.nh + R.nkv) {
+        float val = s;
+        if (R.cosv != nullptr) {
+          const int j = 8 * (p / 16) + p % 8, half = R.D / 2;
+          const float c = R.cosv[(size_t)m * half + j], sn = R.sinv[(size_t)m * half + j];
+          val = p % 16 < 8 ? s * c - partner * sn : s * c + partner * sn;
+        }
+        if (hd < R.nh) {
+          ((__bf16*)y)[(size_t)m * N + n] = (__bf16)val;
+        } else if (R.slots != nullptr) {
+          const int slot = R.slots[m];
+          R.kc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh)) * R.page + slot % R.page) * R.D + p] = (__bf16)val;
+        }
+      } else if (R.slots != nullptr) {
+        const int slot = R.slots[m];
+        R.vc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh - R.nkv)) * R.D + p) * R.page + slot % R.page] = (__bf16)s;
+      }
+      return;
+    }
     if (PRODUCER) {
       float sq = 0.f;
       if (live) {
@@ -318,7 +358,8 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
                                       int M, int N, int K, int out_f32, int gated,
                                       const float* in_parts, int in_nparts, float eps,
                                       const int* rows, float* resid, const float* next_w,
-                                      float* out_parts, hipStream_t stream) {
+                                      float* out_parts, const RopeStore* rope,
+                                      hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
   SL_CHECK(M <= 16, "gemm_skinny: at most 16 rows");
   SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
@@ -340,6 +381,19 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
   const __bf16* ww = (const __bf16*)wt;
   const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts};
   const bool few = in_nparts <= 32 * 8;
+  if (rope != nullptr) {
+    const RopeStore R = *rope;
+    SL_CHECK(!gated && !producer && !out_f32, "gemm_skinny: q/k/v with rotary is a plain or a consumer product");
+    SL_CHECK(R.D % 16 == 0 && R.nh > 0 && R.nkv > 0 && N == (R.nh + 2 * R.nkv) * R.D,
+             "gemm_skinny: q/k/v columns must be (heads + 2 kv heads) * head_dim, head_dim % 16 == 0");
+    SL_CHECK((R.cosv == nullptr) == (R.sinv == nullptr), "gemm_skinny: cos and sin go together");
+    SL_CHECK(R.slots == nullptr || (R.kc != nullptr && R.vc != nullptr && R.page > 0),
+             "gemm_skinny: cache rows need the pages");
+    if (!consumer) gemm_skinny_kernel<false, false, false, 1, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+    else if (few) gemm_skinny_kernel<false, true, false, 8, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+    else gemm_skinny_kernel<false, true, false, 16, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+    return sl_launch_status();
+  }
   if (producer) gemm_skinny_kernel<false, false, true, 1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);
   else if (consumer && gated && few) gemm_skinny_kernel<true, true, false, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);
   else if (consumer && gated) gemm_skinny_kernel<true, true, false, 16><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);

@@ -29,6 +29,16 @@ def _p(t: Optional[torch.Tensor]):
     return None if t is None else _c_void_p(t.data_ptr())
 
 
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+class _RopeStore(ctypes.Structure):
+    """``RopeStore`` of gemm.hip."""
+    _fields_ = [("cosv", _c_void_p), ("sinv", _c_void_p), ("slots", _c_void_p), ("kc", _c_void_p),
+                ("vc", _c_void_p), ("nh", _c_int), ("nkv", _c_int), ("D", _c_int), ("page", _c_int)]
+
+
 class LinearWeight:
     """A weight matrix [N, K] as the products read it: row-major (``w``) for
     products with many rows, tiled (``tiled``, bfloat16 only) for the few-rows
@@ -98,6 +108,7 @@ class HipOps:
         self._bias_cache = {}
         self.use_mfma_attention = True
         self.fuse_norms = act_dtype == torch.bfloat16
+        self.fuse_rope = act_dtype == torch.bfloat16
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
         self._untiled = None          # scratch for "tiled": the row-major form of one matrix
 
@@ -124,6 +135,16 @@ class HipOps:
 
     def _new(self, shape, dtype=None):
         return torch.empty(shape, dtype=dtype or self.act_dtype, device=self.device)
+
+    def _skinny(self, x, weight, bias, y, M, N, K, out_f32=False, gated=False, scaled=None,
+                resid=None, next_gain=None, out_parts=None, rope=None):
+        """One call of the few-rows kernel (at most 16 rows) in any of its forms."""
+        parts = scaled.parts if scaled is not None else None
+        self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
+                   int(out_f32), int(gated), _p(parts), parts.shape[0] if parts is not None else 0,
+                   _c_float(scaled.eps if scaled is not None else 0.0),
+                   _p(scaled.rows) if scaled is not None else None, _p(resid), _p(next_gain),
+                   _p(out_parts), ctypes.byref(rope) if rope is not None else None)
 
     # ------------------------------------------------------------ embedding
     def embed(self, ids, table):
@@ -192,8 +213,7 @@ class HipOps:
             self._check(d.bias, torch.float32, (N,), "bias")
         out = self._new((M, N))
         parts = self._new((-(-N // 16), 16), torch.float32)
-        self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(d.bias), _p(out), M, N, K,
-                   0, 0, None, 0, _c_float(0.0), None, _p(resid), _p(gain), _p(parts))
+        self._skinny(x, weight, d.bias, out, M, N, K, resid=resid, next_gain=gain, out_parts=parts)
         return ScaledRows(out, parts, eps)
 
     # --------------------------------------------------------------- linear
@@ -310,8 +330,7 @@ class HipOps:
                 return self.linear_mid(x, weight, bias, out_f32)
             return self.linear_wide(x, weight, bias, out_f32)
         y = self._new((M, N), torch.float32 if out_f32 else None)
-        self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
-                   int(out_f32), 0, None, 0, _c_float(0.0), None, None, None, None)
+        self._skinny(x, weight, bias, y, M, N, K, out_f32)
         return y
 
     def _linear_scaled(self, xs, weight, bias, out_f32, gated):
@@ -324,9 +343,7 @@ class HipOps:
         if bias is not None:
             self._check(bias, torch.float32, (N,), "bias")
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
-        self._call("gemm", "sl_gemm_skinny", _p(xs.x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
-                   int(out_f32), int(gated), _p(xs.parts), xs.parts.shape[0], _c_float(xs.eps),
-                   _p(xs.rows), None, None, None)
+        self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs)
         return y
 
     GATE_BLOCK = 8                # gate and up rows alternate in blocks of 8 (half an MFMA tile)
@@ -351,8 +368,7 @@ class HipOps:
                     return self.linear_mid(x, weight, None, gated=True)
                 return self.linear_wide(x, weight, None, gated=True)
             y = self._new((M, N // 2))
-            self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), None, _p(y), M, N, K,
-                       0, 1, None, 0, _c_float(0.0), None, None, None, None)
+            self._skinny(x, weight, None, y, M, N, K, gated=True)
             return y
         return self.silu_mul(self.linear(x, weight, None), block)
 
@@ -411,7 +427,12 @@ class HipOps:
         self._check(v_cache, self.act_dtype, (pages, nkv, D, page_size), "V pages")
         return pages
 
-    def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size):
+    def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                   pairs8=False):
+        """Rotate q and k of ``qkv`` in place (``cos`` None: no rotation) and write
+        k and v to their cache rows (``k_cache`` None: no write).  ``pairs8``:
+        the channels of q and k heads come in blocks of 8 channels and their 8
+        partners (the order ``qkv_rope_store`` uses), else first and second half."""
         T = qkv.shape[0]
         self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
         if cos is not None:
@@ -421,7 +442,44 @@ class HipOps:
             self._check_pages(k_cache, v_cache, nkv, D, page_size)
             self._check(slots, torch.int32, (T,), "slots")
         self._call("elementwise", "sl_rope_store", _p(qkv), _p(cos), _p(sin), _p(slots),
-                   _p(k_cache), _p(v_cache), T, nh, nkv, D, page_size)
+                   _p(k_cache), _p(v_cache), T, nh, nkv, D, page_size, int(pairs8))
+
+    def qkv_rope_store(self, x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
+                       page_size):
+        """q/k/v product, rotation and cache write.  The rows of ``weight`` (and
+        ``bias``) hold every q and k head in the blocked pair order (``pairs8``
+        above).  Returns the [T, (nh + 2 nkv) D] buffer whose q columns the
+        attention reads.  For at most 16 rows and a tiled weight all of it is
+        one kernel; k and v columns of the buffer are then not written."""
+        if not isinstance(weight, LinearWeight):
+            weight = LinearWeight(weight)
+        M, K = x.shape
+        N = weight.shape[0]
+        if N != (nh + 2 * nkv) * D or D % 16:
+            raise KernelError("qkv_rope_store: weight rows must be (nh + 2 nkv) * D with D % 16 == 0")
+        fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
+                 and weight.tiled is not None and weight.shape == (N, K))
+        if not fused:
+            qkv = self.linear(x, weight, bias)
+            self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True)
+            return qkv
+        scaled = x if isinstance(x, ScaledRows) else None
+        if scaled is None:
+            self._check(x, self.act_dtype, None, "x")
+        if bias is not None:
+            self._check(bias, torch.float32, (N,), "bias")
+        if cos is not None:
+            self._check(cos, torch.float32, (M, D // 2), "cos")
+            self._check(sin, torch.float32, (M, D // 2), "sin")
+        if k_cache is not None:
+            self._check_pages(k_cache, v_cache, nkv, D, page_size)
+            self._check(slots, torch.int32, (M,), "slots")
+        rope = _RopeStore(_ptr(cos), _ptr(sin), _ptr(slots if k_cache is not None else None),
+                          _ptr(k_cache), _ptr(v_cache), nh, nkv, D, page_size)
+        qkv = self._new((M, N))
+        self._skinny(scaled.x if scaled is not None else x, weight, bias, qkv, M, N, K,
+                     scaled=scaled, rope=rope)
+        return qkv
 
     # ------------------------------------------------------------ attention
     def paged_attention(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,

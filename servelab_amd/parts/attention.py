@@ -54,27 +54,44 @@ class PagedAttention(Mixer):
     def load(self, tensors, rt):
         self.rt = rt
         self.position.load(tensors, rt)
-        # [Wq; Wk; Wv] -> one [(nh + 2 nkv) D, H] matrix, one GEMM
+        # [Wq; Wk; Wv] -> one [(nh + 2 nkv) D, H] matrix, one GEMM.  When the head
+        # size allows, the channels of every q and k head are reordered into
+        # blocks of 8 channels followed by their 8 rotation partners (what the
+        # fused product + rotation + cache write of the kernel table wants);
+        # q . k does not depend on the order, v keeps its own.
+        self.pairs8 = self.head_dim % 16 == 0 and hasattr(rt.ops, "qkv_rope_store")
+        d, half = self.head_dim, self.head_dim // 2
+
+        def reorder(t, heads):
+            if not self.pairs8:
+                return t
+            blocks = t.reshape(heads, 2, half // 8, 8, *t.shape[1:])      # [head, half, block, 8, ...]
+            return blocks.transpose(1, 2).reshape(t.shape)               # [head, block, half, 8, ...]
         self.w_qkv = rt.linear_weight(torch.cat(
-            [tensors("q_proj.weight"), tensors("k_proj.weight"), tensors("v_proj.weight")], 0))
+            [reorder(tensors("q_proj.weight"), self.num_heads),
+             reorder(tensors("k_proj.weight"), self.num_kv_heads), tensors("v_proj.weight")], 0))
         self.b_qkv = None
         if self.qkv_bias:
             self.b_qkv = rt.vector(torch.cat(
-                [tensors("q_proj.bias").float(), tensors("k_proj.bias").float(),
+                [reorder(tensors("q_proj.bias").float(), self.num_heads),
+                 reorder(tensors("k_proj.bias").float(), self.num_kv_heads),
                  tensors("v_proj.bias").float()], 0))
         self.w_o = rt.linear_weight(tensors("o_proj.weight"))
 
     # ---- compute
     def forward(self, x, batch, cache, shared):
         ops = self.rt.ops
-        qkv = ops.linear(x, self.w_qkv, self.b_qkv)
         tables = self.position.tables(batch, shared)
         cos, sin = tables if tables is not None else (None, None)
         group = batch.groups[cache.group]
-        ops.rope_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, cos, sin,
-                       group.slots if cache.write else None,
-                       cache.k if cache.write else None,
-                       cache.v if cache.write else None, cache.page_size)
+        slots, kc, vc = (group.slots, cache.k, cache.v) if cache.write else (None, None, None)
+        if self.pairs8:
+            qkv = ops.qkv_rope_store(x, self.w_qkv, self.b_qkv, self.num_heads, self.num_kv_heads,
+                                     self.head_dim, cos, sin, slots, kc, vc, cache.page_size)
+        else:
+            qkv = ops.linear(x, self.w_qkv, self.b_qkv)
+            ops.rope_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, cos, sin,
+                           slots, kc, vc, cache.page_size)
         attn = ops.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
             cache.page_size, group.block_tables, batch, self.scale, self.window)

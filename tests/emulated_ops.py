@@ -61,15 +61,25 @@ class EmulatedOps:
         ang = positions.float()[:, None] * inv_freq[None, :]
         return torch.cos(ang), torch.sin(ang)
 
-    def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size):
-        """Rotate q and k of ``qkv`` in place; write k and v to their pages."""
+    def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                   pairs8=False):
+        """Rotate q and k of ``qkv`` in place; write k and v to their pages.
+        ``pairs8``: q and k heads hold blocks of 8 channels and their 8 partners
+        (channel order [block][half][8]) instead of first half, second half."""
         T = qkv.shape[0]
         half = D // 2
         qk = qkv[:, :(nh + nkv) * D].view(T, nh + nkv, D)
         if cos is not None:
-            x1, x2 = _f(qk[..., :half]), _f(qk[..., half:])
+            if pairs8:
+                std = qk.reshape(T, nh + nkv, half // 8, 2, 8).transpose(2, 3).reshape(T, nh + nkv, D)
+            else:
+                std = qk
+            x1, x2 = _f(std[..., :half]), _f(std[..., half:])
             c, s = cos[:, None, :], sin[:, None, :]
-            qk.copy_(torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], -1).to(qkv.dtype))
+            rot = torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], -1).to(qkv.dtype)
+            if pairs8:
+                rot = rot.reshape(T, nh + nkv, 2, half // 8, 8).transpose(2, 3).reshape(T, nh + nkv, D)
+            qk.copy_(rot)
         if k_cache is None:
             return
         k = qkv[:, nh * D:(nh + nkv) * D].view(T, nkv, D)
@@ -77,6 +87,11 @@ class EmulatedOps:
         page, off = (slots // page_size).long(), (slots % page_size).long()
         k_cache[page, :, off, :] = k
         v_cache[page, :, :, off] = v
+
+    def qkv_rope_store(self, x, w, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size):
+        qkv = self.linear(x, w, bias)
+        self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True)
+        return qkv
 
     # ------------------------------------------------------------ attention
     def paged_attention(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,

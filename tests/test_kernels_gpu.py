@@ -269,8 +269,9 @@ def test_rope_tables(both):
     assert (sin.double() - torch.sin(ang)).abs().max().item() < 2e-7
 
 
+@pytest.mark.parametrize("pairs8", [False, True])
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (6, 1, 48, 32), (7, 7, 128, 64)])
-def test_rope_store(both, nh, nkv, D, page):
+def test_rope_store(both, nh, nkv, D, page, pairs8):
     ops, emu, dt = both
     T, pages = 37, 9
     qkv = randn(T, (nh + 2 * nkv) * D, dtype=dt, seed=1)
@@ -281,8 +282,8 @@ def test_rope_store(both, nh, nkv, D, page):
     kc = [randn(pages, nkv, page, D, dtype=dt, seed=7) for _ in range(2)]
     vc = [randn(pages, nkv, D, page, dtype=dt, seed=8) for _ in range(2)]
     q1, q2 = qkv.clone(), qkv.clone()
-    ops.rope_store(q1, nh, nkv, D, cos, sin, slots, kc[0], vc[0], page)
-    emu.rope_store(q2, nh, nkv, D, cos, sin, slots, kc[1], vc[1], page)
+    ops.rope_store(q1, nh, nkv, D, cos, sin, slots, kc[0], vc[0], page, pairs8)
+    emu.rope_store(q2, nh, nkv, D, cos, sin, slots, kc[1], vc[1], page, pairs8)
     assert rel_err(q1, q2) < ELEM_TOL[dt] * 2
     assert rel_err(kc[0], kc[1]) < ELEM_TOL[dt] * 2
     assert torch.equal(vc[0], vc[1])
@@ -293,6 +294,50 @@ def test_rope_store(both, nh, nkv, D, page):
     k_before = kc[0].clone()
     ops.rope_store(qkv.clone(), nh, nkv, D, cos, sin, None, None, None, page)
     assert torch.equal(kc[0], k_before)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 40])
+@pytest.mark.parametrize("nh,nkv,D,page,H", [(4, 2, 16, 16, 64), (28, 4, 128, 16, 256), (5, 1, 48, 32, 96)])
+def test_qkv_rope_store(M, nh, nkv, D, page, H):
+    """Product + rotation + cache write: the one fused kernel (at most 16 rows)
+    and the product followed by rope_store give the same q, K pages and V
+    pages; also with un-normalised input rows and with no rotation or no write."""
+    from servelab_amd.kernels import HipOps
+    from servelab_amd.kernels.ops import ScaledRows
+    dt = torch.bfloat16
+    ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+    N = (nh + 2 * nkv) * D
+    x = randn(M, H, dtype=dt, seed=1)
+    w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.1, seed=2))
+    bias = randn(N, scale=0.1, seed=3)
+    inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
+    cos, sin = emu.rope_tables(torch.arange(7, 7 + M, dtype=torch.int32).cuda(), inv)
+    pages = 8
+    slots = torch.randperm(pages * page)[:M].to(torch.int32).cuda()
+
+    def run(o, xin, cos, sin, write):
+        kc = randn(pages, nkv, page, D, dtype=dt, seed=7)
+        vc = randn(pages, nkv, D, page, dtype=dt, seed=8)
+        qkv = o.qkv_rope_store(xin, w if o is ops else w.w, bias, nh, nkv, D, cos, sin,
+                               slots if write else None, kc if write else None,
+                               vc if write else None, page)
+        return qkv[:, :nh * D].float(), kc.float(), vc.float()
+    for c, s_, write in ((cos, sin, True), (None, None, True), (cos, sin, False)):
+        got, want = run(ops, x, c, s_, write), run(emu, x, c, s_, write)
+        for g, r in zip(got, want):
+            assert rel_err(g, r) < 2 ** -6
+    if M <= 16:
+        # un-normalised rows: x * gain with the sums of squares in parts
+        stream = randn(M, H, seed=9)
+        gain = 1 + 0.1 * randn(H, seed=10)
+        parts = torch.zeros(-(-H // 16), 16, device="cuda")
+        sq = stream.pow(2).view(M, -1, 16).sum(-1)                  # [M, H / 16]
+        parts[:, :M] = sq.T
+        scaled = ScaledRows((stream * gain).to(dt), parts, 1e-5)
+        normed = (stream * torch.rsqrt(stream.pow(2).mean(-1, keepdim=True) + 1e-5) * gain).to(dt)
+        got, want = run(ops, scaled, cos, sin, True), run(emu, normed, cos, sin, True)
+        for g, r in zip(got, want):
+            assert rel_err(g, r) < 2 ** -5
 
 
 def make_attention_case(dt, nh, nkv, D, page, seqs, seed=0):
