@@ -23,11 +23,20 @@
 // operand of the second product, and the matching A operand is one 16-byte
 // load from the V pages, which are stored channel-major ([page, nkv, D, page_size]).
 // K pages are key-major ([page, nkv, page_size, D]): its A operand is one
-// 16-byte load as well.  Nothing goes through LDS.
+// 16-byte load as well.
 //
-// Decode (one token per sequence, g columns) splits the context over several
-// wavefronts; each writes an unnormalised partial (o, max, sum) and
-// attention_combine_kernel merges them.
+// Three launches share that inner block (struct Columns):
+//   - decode (one token per sequence, g columns): the context is split over
+//     several wavefronts; each writes an unnormalised partial (o, reference,
+//     sum) and attention_combine_kernel merges them;
+//   - prompt portions, one wavefront per 32 columns, operands straight from
+//     the pages, two wavefronts per SIMD so that one computes while the other
+//     waits for its loads;
+//   - prompt portions, four wavefronts per workgroup that share each block of
+//     keys and values through LDS (attention_mfma_shared_kernel), for launches
+//     large enough that L2 traffic, not latency, is the limit.
+// The softmax keeps a reference point per column instead of the exact running
+// maximum (see LAZY) and folds the scale into the exponent's multiply-add.
 #include "common.h"
 
 #if defined(SL_F32)
@@ -47,9 +56,27 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // 2^x by the hardware instruction; arguments here are <= 0 and tiny results may flush to 0
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Maximum / sum over the four lanes n, n + 16, n + 32, n + 48 that share a
+// column, by the row-swap instructions of gfx950 (register to register, no
+// trip through LDS): after a swap of x with itself one result holds the lower
+// partner and the other the upper one, in every lane.
+__device__ __forceinline__ float column_max(float x) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float column_sum(float x) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 constexpr int D = SL_HEAD_DIM;
 constexpr int KK = D / 32;       // k-steps of the score product
 constexpr int DD = D / 16;       // row tiles of the output product
+constexpr float LAZY = 8.f;      // growth of a column's maximum (log 2 units) that moves its reference point
 
 struct AttnParams {
   const __bf16* qkv;             // [T, row_stride], q heads first
@@ -61,7 +88,7 @@ struct AttnParams {
   const int* cu_q;               // [S + 1]
   const int* positions;          // [T]
   int seq_begin;                 // first sequence of this launch
-  int nh, nkv, page;
+  int nh, nkv, page;             // page: 16, 32 or 64 keys
   float scale;
   int window;                    // 0 = none
   int nsplit;
@@ -71,8 +98,146 @@ struct AttnParams {
   int part_row0;                 // token index of partial row 0
 };
 
+// The columns of one wavefront: queries, running maxima and sums, outputs.
+template <int NB>
+struct Columns {
+  int tok[NB], head[NB], pos_c[NB], lo_c[NB];
+  bf16x8 qf[NB][KK];
+  float m_run[NB], l_run[NB];
+  f32x4 o[NB][DD];
+  int kb_begin, kb_end;          // key blocks (of 32) some column sees
+  int full_begin, full_end;      // blocks in [full_begin, full_end) are seen whole by every column
+  float scale_log2;
+
+  __device__ __forceinline__ void init(const AttnParams& P, int q0, int ncols, int c0, int pos0,
+                                       int kvh, int g, int n, int gq) {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      int c = c0 + 16 * b + n;
+      const bool valid = c < ncols;
+      if (!valid) c = ncols - 1;
+      tok[b] = c / g;
+      head[b] = kvh * g + c % g;
+      pos_c[b] = valid ? pos0 + tok[b] : -1;       // padding: computed like its neighbour, never stored
+      lo_c[b] = (P.window > 0 && pos_c[b] - P.window + 1 > 0) ? pos_c[b] - P.window + 1 : 0;
+      const __bf16* q = P.qkv + (size_t)(q0 + tok[b]) * P.row_stride + (size_t)head[b] * D + 8 * gq;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) qf[b][kk] = *(const bf16x8*)(q + 32 * kk);
+      m_run[b] = -INFINITY;
+      l_run[b] = 0.f;
+#pragma unroll
+      for (int dd = 0; dd < DD; ++dd) o[b][dd] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int tok_first = c0 / g;
+    const int c_last = c0 + 16 * NB - 1 < ncols - 1 ? c0 + 16 * NB - 1 : ncols - 1;
+    const int kmax = pos0 + c_last / g;
+    int kmin = 0;
+    if (P.window > 0 && pos0 + tok_first - P.window + 1 > 0) kmin = pos0 + tok_first - P.window + 1;
+    kb_begin = kmin / 32;
+    kb_end = kmax / 32 + 1;
+    full_end = (pos0 + tok_first + 1) / 32;        // blocks below: keys <= first position
+    full_begin = 0;
+    if (P.window > 0) {
+      const int lo_last = pos0 + c_last / g - P.window + 1;
+      full_begin = lo_last > 0 ? (lo_last + 31) / 32 : 0;
+    }
+    scale_log2 = P.scale * 1.4426950408889634f;
+  }
+
+  // One block of 32 keys.  kf: row i of tile m is key kbase + 8 (i / 4) + 4 m + i % 4;
+  // vf: row d of V^T, keys kbase + 8 gq .. + 7.
+  __device__ __forceinline__ void block(int kb, const bf16x8 (&kf)[2][KK], const bf16x8 (&vf)[DD],
+                                        int gq) {
+    const int kbase = kb * 32;
+    const bool edge = kb >= full_end || kb < full_begin;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kk], qf[b][kk], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kk], qf[b][kk], s1, 0, 0, 0);
+      }
+      // this lane: column n, keys kbase + 8 gq + j, j = 0..7
+      float s[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s[j] = j < 4 ? s0[j] : s1[j - 4];
+      if (edge) {                                  // a block some column does not see whole
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = kbase + 8 * gq + j;
+          if (key > pos_c[b] || key < lo_c[b]) s[j] = -INFINITY;
+        }
+      }
+      float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                       fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+      mx = column_max(mx);
+      // m_run is a reference point, not the exact maximum: it moves only when
+      // the maximum has grown by more than LAZY (in units of log 2), so that
+      // the outputs are rescaled rarely; until then probabilities reach 2^LAZY
+      // at most, far from any overflow, with the same relative rounding.
+      const float mxs = mx * scale_log2;
+      if (__builtin_expect(__any(mxs > m_run[b] + LAZY), 0)) {
+        const float m_new = fmaxf(m_run[b], mxs);
+        const float alpha = fast_exp2(m_run[b] - (m_new == -INFINITY ? 0.f : m_new));
+        m_run[b] = m_new;
+        l_run[b] *= alpha;
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) o[b][dd] *= alpha;
+      }
+      const float neg_m = m_run[b] == -INFINITY ? 0.f : -m_run[b];
+      float psum = 0.f;
+      bf16x8 pb;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float p = fast_exp2(fmaf(s[j], scale_log2, neg_m));
+        psum += p;
+        pb[j] = (__bf16)p;
+      }
+      l_run[b] += psum;
+#pragma unroll
+      for (int dd = 0; dd < DD; ++dd)
+        o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb, o[b][dd], 0, 0, 0);
+    }
+  }
+
+  // lane holds column n, channels 16 dd + 4 gq + r
+  template <bool SPLIT>
+  __device__ __forceinline__ void store(const AttnParams& P, int q0, int split, int gq) {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const float l = column_sum(l_run[b]);
+      if (pos_c[b] < 0) continue;
+      const size_t row = (size_t)(q0 + tok[b]);
+      if (SPLIT) {
+        const size_t pr = ((row - P.part_row0) * P.nh + head[b]) * P.nsplit + split;
+        float* po = P.part_o + pr * D + 4 * gq;
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) *(f32x4*)(po + 16 * dd) = o[b][dd];
+        if (gq == 0) {
+          P.part_ml[pr * 2] = m_run[b];
+          P.part_ml[pr * 2 + 1] = l;
+        }
+      } else {
+        const float inv = 1.f / l;
+        __bf16* po = P.out + (row * P.nh + head[b]) * D + 4 * gq;
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) {
+          bf16x4 r;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) r[j] = (__bf16)(o[b][dd][j] * inv);
+          *(bf16x4*)(po + 16 * dd) = r;
+        }
+      }
+    }
+  }
+};
+
+// One wavefront per workgroup; operands straight from the pages.  Used for
+// decode tokens (SPLIT: the wavefront takes one share of the key blocks) and
+// for short prompt portions.
 template <int NB, bool SPLIT>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(const AttnParams P) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 256 ? 2 : 1))) void attention_mfma_kernel(const AttnParams P) {
   const int lane = threadIdx.x, n = lane & 15, gq = lane >> 4;
   const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
   const int g = P.nh / P.nkv;
@@ -83,35 +248,13 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const AttnParams P) 
   const int tile_rev = blockIdx.x / P.nsplit, split = blockIdx.x % P.nsplit;
   if (tile_rev >= ntiles) return;
   const int tile = ntiles - 1 - tile_rev;          // long (late) tiles first
-  const int c0 = tile * 16 * NB;
   const int pos0 = P.positions[q0];
   const int* table = P.block_tables + (size_t)seq * P.max_pages;
-  const int page = P.page;
+  const int page = P.page, page_shift = 31 - __builtin_clz(page);
 
-  // ---- columns of this lane
-  int tok[NB], head[NB], pos_c[NB], lo_c[NB];
-  bf16x8 qf[NB][KK];
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    int c = c0 + 16 * b + n;
-    const bool valid = c < ncols;
-    if (!valid) c = ncols - 1;
-    tok[b] = c / g;
-    head[b] = kvh * g + c % g;
-    pos_c[b] = valid ? pos0 + tok[b] : -1;         // padding: computed like its neighbour, never stored
-    lo_c[b] = (P.window > 0 && pos_c[b] - P.window + 1 > 0) ? pos_c[b] - P.window + 1 : 0;
-    const __bf16* q = P.qkv + (size_t)(q0 + tok[b]) * P.row_stride + (size_t)head[b] * D + 8 * gq;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qf[b][kk] = *(const bf16x8*)(q + 32 * kk);
-  }
-
-  // ---- key blocks of this wavefront
-  const int tok_first = c0 / g;
-  const int c_last = c0 + 16 * NB - 1 < ncols - 1 ? c0 + 16 * NB - 1 : ncols - 1;
-  const int kmax = pos0 + c_last / g;
-  int kmin = 0;
-  if (P.window > 0 && pos0 + tok_first - P.window + 1 > 0) kmin = pos0 + tok_first - P.window + 1;
-  int kb_begin = kmin / 32, kb_end = kmax / 32 + 1;
+  Columns<NB> C;
+  C.init(P, q0, ncols, tile * 16 * NB, pos0, kvh, g, n, gq);
+  int kb_begin = C.kb_begin, kb_end = C.kb_end;
   if (SPLIT) {
     const int nblk = kb_end - kb_begin;
     const int first = kb_begin + (int)((long long)nblk * split / P.nsplit);
@@ -119,124 +262,185 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const AttnParams P) 
     kb_begin = first;
   }
 
-  float m_run[NB], l_run[NB];
-  f32x4 o[NB][DD];
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    m_run[b] = -INFINITY;
-    l_run[b] = 0.f;
-#pragma unroll
-    for (int dd = 0; dd < DD; ++dd) o[b][dd] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-
-  // blocks every column of this wavefront sees whole need no mask
-  const int full_end = (pos0 + tok_first + 1) / 32;             // blocks below: keys <= first position
-  int full_begin = 0;
-  if (P.window > 0) {
-    const int lo_last = pos0 + c_last / g - P.window + 1;
-    full_begin = lo_last > 0 ? (lo_last + 31) / 32 : 0;
-  }
-  const float scale_log2 = P.scale * 1.4426950408889634f;
-
-  for (int kb = kb_begin; kb < kb_end; ++kb) {
+  // The two table entries a block of 32 keys can touch are the same for every
+  // lane, so they come through the scalar path, one block ahead of the keys.
+  auto load_pages = [&](int kb, int (&pg)[2]) {
     const int kbase = kb * 32;
-    const bool edge = kb >= full_end || kb < full_begin;
-    // K: row i of tile m is key kbase + 8 (i / 4) + 4 m + i % 4
-    bf16x8 kf[2][KK];
+    pg[0] = table[kbase >> page_shift];
+    pg[1] = table[(kbase + 16) >> page_shift];
+  };
+  auto load_block = [&](int kb, const int (&pg)[2], bf16x8 (&kf)[2][KK], bf16x8 (&vf)[DD]) {
+    const int kbase = kb * 32;
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
-      const int key = kbase + 8 * (n >> 2) + 4 * m + (n & 3);
-      const int pg = table[key / page];
-      const __bf16* kr = P.kc + (((size_t)pg * P.nkv + kvh) * page + key % page) * D + 8 * gq;
+      const int ko = 8 * (n >> 2) + 4 * m + (n & 3);
+      const int p = ko < 16 ? pg[0] : pg[1];
+      const __bf16* kr = P.kc + (((size_t)p * P.nkv + kvh) * page + ((kbase + ko) & (page - 1))) * D + 8 * gq;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) kf[m][kk] = *(const bf16x8*)(kr + 32 * kk);
     }
-    // V^T: row d, keys kbase + 8 gq .. + 7
-    bf16x8 vf[DD];
-    {
-      const int key0 = kbase + 8 * gq;
-      const int pg = table[key0 / page];
-      const __bf16* vr = P.vc + ((size_t)pg * P.nkv + kvh) * D * page + key0 % page;
+    const int p = gq < 2 ? pg[0] : pg[1];
+    const __bf16* vr = P.vc + ((size_t)p * P.nkv + kvh) * D * page + ((kbase + 8 * gq) & (page - 1));
 #pragma unroll
-      for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)(vr + (size_t)(16 * dd + n) * page);
-    }
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kk], qf[b][kk], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kk], qf[b][kk], s1, 0, 0, 0);
-      }
-      // this lane: column n, keys kbase + 8 gq + j, j = 0..7; scores in units of log 2
-      float s[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) s[j] = (j < 4 ? s0[j] : s1[j - 4]) * scale_log2;
-      if (edge) {                                  // a block some column does not see whole
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int key = kbase + 8 * gq + j;
-          if (key > pos_c[b] || key < lo_c[b]) s[j] = -INFINITY;
-        }
-      }
-      float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
-                       fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run[b], mx);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const bool grew = m_new != m_run[b];
-      float psum = 0.f;
-      bf16x8 pb;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float p = fast_exp2(s[j] - m_safe);
-        psum += p;
-        pb[j] = (__bf16)p;
-      }
-      if (__any(grew)) {                           // rescale only when some column's maximum grew
-        const float alpha = fast_exp2(m_run[b] - m_safe);
-        m_run[b] = m_new;
-        l_run[b] *= alpha;
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) o[b][dd] *= alpha;
-      }
-      l_run[b] += psum;
-#pragma unroll
-      for (int dd = 0; dd < DD; ++dd)
-        o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb, o[b][dd], 0, 0, 0);
-    }
-  }
+    for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)(vr + (size_t)(16 * dd + n) * page);
+  };
 
-  // ---- write: lane holds column n, channels 16 dd + 4 gq + r
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    float l = l_run[b];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    if (pos_c[b] < 0) continue;
-    const size_t row = (size_t)(q0 + tok[b]);
-    if (SPLIT) {
-      const size_t pr = ((row - P.part_row0) * P.nh + head[b]) * P.nsplit + split;
-      float* po = P.part_o + pr * D + 4 * gq;
-#pragma unroll
-      for (int dd = 0; dd < DD; ++dd) *(f32x4*)(po + 16 * dd) = o[b][dd];
-      if (gq == 0) {
-        P.part_ml[pr * 2] = m_run[b];
-        P.part_ml[pr * 2 + 1] = l;
+  // With 32 columns only one wavefront fits a SIMD (the accumulators fill the
+  // registers) and nothing else hides the latency of the loads: the keys and
+  // values of the next block are requested into a second set of registers
+  // before this block is computed, and the loop is unrolled over the two sets
+  // so that no copy waits for them.
+  constexpr bool AHEAD = false;
+  if (AHEAD && kb_begin < kb_end) {
+    bf16x8 kf_a[2][KK], vf_a[DD], kf_b[2][KK], vf_b[DD];
+    int pg[2];
+    const int last = kb_end - 1;
+    load_pages(kb_begin, pg);
+    load_block(kb_begin, pg, kf_a, vf_a);
+    load_pages(kb_begin + 1 < last ? kb_begin + 1 : last, pg);
+    for (int kb = kb_begin; kb < kb_end; kb += 2) {
+      if (kb + 1 < kb_end) {
+        load_block(kb + 1, pg, kf_b, vf_b);
+        load_pages(kb + 2 < last ? kb + 2 : last, pg);
       }
-    } else {
-      const float inv = 1.f / l;
-      __bf16* po = P.out + (row * P.nh + head[b]) * D + 4 * gq;
-#pragma unroll
-      for (int dd = 0; dd < DD; ++dd) {
-        bf16x4 r;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) r[j] = (__bf16)(o[b][dd][j] * inv);
-        *(bf16x4*)(po + 16 * dd) = r;
+      C.block(kb, kf_a, vf_a, gq);
+      if (kb + 1 < kb_end) {
+        if (kb + 2 < kb_end) {
+          load_block(kb + 2, pg, kf_a, vf_a);
+          load_pages(kb + 3 < last ? kb + 3 : last, pg);
+        }
+        C.block(kb + 1, kf_b, vf_b, gq);
       }
     }
   }
+  if (!AHEAD) {
+    for (int kb = kb_begin; kb < kb_end; ++kb) {
+      bf16x8 kf[2][KK], vf[DD];
+      int pg[2];
+      load_pages(kb, pg);
+      load_block(kb, pg, kf, vf);
+      C.block(kb, kf, vf, gq);
+    }
+  }
+  C.template store<SPLIT>(P, q0, split, gq);
+}
+
+// Prompt portions: four wavefronts, one per SIMD, take 32 columns each and
+// share every block of keys and values through LDS, so a block leaves the
+// cache hierarchy once per 128 columns instead of once per 32 (measured on
+// MI355X: with one wavefront per workgroup the kernel ran at the rate at which
+// L2 delivers the operands, 32 flop a byte, not at the rate of the matrix
+// cores).  Two buffers: the next block travels pages -> registers while this
+// one is computed, registers -> LDS afterwards, one barrier a block.
+//
+// LDS rows are padded by 16 bytes, which makes the row stride an odd number
+// of 16-byte units: the 16 lanes that read one operand column of a tile
+// (rows r..r+15, same offset) then fall into 16 different bank groups.  K rows
+// are stored in the order the product wants them (tile m, row i), not in key
+// order.
+constexpr int SHARED_WAVES = 4;
+constexpr int KS = D + 8;                          // K row stride in LDS, elements
+constexpr int VS = 32 + 8;                         // V^T row stride
+constexpr int STAGE = (4 * D + 64 * SHARED_WAVES - 1) / (64 * SHARED_WAVES);   // 16-byte units a thread carries, K and V each
+constexpr bool SHARED_FITS = 2 * (32 * KS + D * VS) * 2 <= 65536;
+
+__global__ __launch_bounds__(64 * SHARED_WAVES) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1)))
+void attention_mfma_shared_kernel(const AttnParams P) {
+  constexpr int NB = 2, THREADS = 64 * SHARED_WAVES, COLS = 16 * NB * SHARED_WAVES;
+  __shared__ __attribute__((aligned(16))) __bf16 k_lds[2][SHARED_FITS ? 32 * KS : 8];
+  __shared__ __attribute__((aligned(16))) __bf16 v_lds[2][SHARED_FITS ? D * VS : 8];
+  const int t = threadIdx.x, wave = t >> 6, lane = t & 63, n = lane & 15, gq = lane >> 4;
+  const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
+  const int g = P.nh / P.nkv;
+  const int q0 = P.cu_q[seq];
+  const int qlen = P.cu_q[seq + 1] - q0;
+  const int ncols = qlen * g;
+  const int ntiles = (ncols + COLS - 1) / COLS;
+  if ((int)blockIdx.x >= ntiles) return;           // the whole workgroup leaves together
+  const int tile = ntiles - 1 - blockIdx.x;        // long (late) tiles first
+  const int pos0 = P.positions[q0];
+  const int* table = P.block_tables + (size_t)seq * P.max_pages;
+  const int page = P.page, page_shift = 31 - __builtin_clz(page);
+
+  const int wg_c0 = tile * COLS;
+  const int c0 = wg_c0 + 16 * NB * wave;
+  const bool active = c0 < ncols;                  // a wavefront past the last column only helps loading
+  Columns<NB> C;
+  C.init(P, q0, ncols, active ? c0 : wg_c0, pos0, kvh, g, n, gq);
+
+  // key blocks of the workgroup: from the first block its first wavefront
+  // needs to the last block its last active wavefront needs
+  const int wg_tok_first = wg_c0 / g;
+  const int wg_c_last = wg_c0 + COLS - 1 < ncols - 1 ? wg_c0 + COLS - 1 : ncols - 1;
+  int kmin = 0;
+  if (P.window > 0 && pos0 + wg_tok_first - P.window + 1 > 0) kmin = pos0 + wg_tok_first - P.window + 1;
+  const int wg_begin = kmin / 32, wg_end = (pos0 + wg_c_last / g) / 32 + 1;
+
+  bf16x8 k_stage[STAGE], v_stage[STAGE];
+  int pg[2];
+  auto load_pages = [&](int kb) {
+    const int kbase = kb * 32;
+    pg[0] = table[kbase >> page_shift];
+    pg[1] = table[(kbase + 16) >> page_shift];
+  };
+  // 16-byte unit id of K: key id / (D/8), channels 8 (id % (D/8));  of V^T: row id / 4, keys 8 (id % 4)
+  auto stage_load = [&](int kb) {
+    const int kbase = kb * 32;
+#pragma unroll
+    for (int i = 0; i < STAGE; ++i) {
+      const int id = t + THREADS * i;
+      if (id < 4 * D) {
+        const int ko = id / (D / 8), c = id % (D / 8);
+        const int p = ko < 16 ? pg[0] : pg[1];
+        k_stage[i] = *(const bf16x8*)(P.kc + (((size_t)p * P.nkv + kvh) * page + ((kbase + ko) & (page - 1))) * D + 8 * c);
+        const int d = id >> 2, q = id & 3;
+        const int pv = q < 2 ? pg[0] : pg[1];
+        v_stage[i] = *(const bf16x8*)(P.vc + (((size_t)pv * P.nkv + kvh) * D + d) * page + ((kbase + 8 * q) & (page - 1)));
+      }
+    }
+  };
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < STAGE; ++i) {
+      const int id = t + THREADS * i;
+      if (id < 4 * D) {
+        const int ko = id / (D / 8), c = id % (D / 8);
+        const int row = 16 * ((ko >> 2) & 1) + 4 * (ko >> 3) + (ko & 3);   // key ko is row i = 4 (ko / 8) + ko % 4 of tile (ko / 4) % 2
+        *(bf16x8*)&k_lds[buf][row * KS + 8 * c] = k_stage[i];
+        const int d = id >> 2, q = id & 3;
+        *(bf16x8*)&v_lds[buf][d * VS + 8 * q] = v_stage[i];
+      }
+    }
+  };
+
+  const int last = wg_end - 1;
+  load_pages(wg_begin);
+  stage_load(wg_begin);
+  load_pages(wg_begin + 1 < last ? wg_begin + 1 : last);
+  stage_store(0);
+  __syncthreads();
+  for (int kb = wg_begin; kb < wg_end; ++kb) {
+    const int buf = (kb - wg_begin) & 1;
+    const bool more = kb + 1 < wg_end;
+    if (more) {
+      stage_load(kb + 1);
+      load_pages(kb + 2 < last ? kb + 2 : last);
+    }
+    if (active && kb >= C.kb_begin && kb < C.kb_end) {
+      bf16x8 kf[2][KK], vf[DD];
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+          kf[m][kk] = *(const bf16x8*)&k_lds[buf][(16 * m + n) * KS + 32 * kk + 8 * gq];
+#pragma unroll
+      for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)&v_lds[buf][(16 * dd + n) * VS + 8 * gq];
+      C.block(kb, kf, vf, gq);
+    }
+    if (more) stage_store(buf ^ 1);
+    __syncthreads();                               // the other buffer is complete; this one is free
+  }
+  if (active) C.template store<false>(P, q0, 0, gq);
 }
 
 // out[row, head, :] = sum_j w_j o_j / sum_j w_j l_j,  w_j = exp(m_j - max m).
@@ -282,11 +486,13 @@ extern "C" int sl_attention_mfma_head_dim() { return D; }
 // One launch over sequences [seq_begin, seq_begin + num_seqs), all with at
 // most max_q_len tokens.  nsplit > 1 needs part_o / part_ml for the rows
 // [part_row0, part_row0 + part_rows) these sequences own (one token each).
+// Prompt portions go to the workgroups that share keys through LDS once the
+// launch would have shared_min_waves wavefronts of 32 columns or more.
 extern "C" const char* sl_attention_mfma(
     const void* qkv, int row_stride, const void* kc, const void* vc, const int* block_tables,
     int max_pages, const int* cu_q, const int* positions, int seq_begin, int num_seqs,
     int max_q_len, int nh, int nkv, int head_dim, int page, float scale, int window, int nsplit,
-    void* out, float* part_o, float* part_ml, int part_row0, int part_rows, hipStream_t stream) {
+    int shared_min_waves, void* out, float* part_o, float* part_ml, int part_row0, int part_rows, hipStream_t stream) {
   SL_CHECK(head_dim == D, "attention_mfma: built for another head size");
   SL_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: heads must be a multiple of kv heads");
   SL_CHECK(page == 16 || page == 32 || page == 64, "attention_mfma: page size must be 16, 32 or 64");
@@ -317,14 +523,22 @@ extern "C" const char* sl_attention_mfma(
                                                                   part_row0, (__bf16*)out);
     return sl_launch_status();
   }
-  // prompt portions: 32 columns per wavefront measured fastest on MI355X (7B shape,
-  // 2,048 tokens: 133 us a layer against 154 us with 64 columns and 166 us with 16)
+  // Prompt portions.  One wavefront per 32 columns, each reading its keys
+  // straight from the pages, has the most wavefronts in flight and wins while
+  // the chip is not full; with more of them than about two per SIMD the
+  // delivery of operands from L2 limits it and the workgroups that share a
+  // block through LDS win (MI355X, 7B shape, one prompt: 2,048 tokens 97 us
+  // against 108 us, 8,192 tokens 1,050 us against 854 us); the caller sets
+  // the crossover.
+  const long long tiles = (cols + 31) / 32;
+  SL_CHECK(tiles <= 1 << 30, "attention_mfma: too many column tiles");
   if (cols <= 16) {
     attention_mfma_kernel<1, false><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);
-  } else {
-    const long long tiles = (cols + 31) / 32;
-    SL_CHECK(tiles <= 1 << 30, "attention_mfma: too many column tiles");
+  } else if (!SHARED_FITS || tiles * nkv * num_seqs < shared_min_waves) {
     attention_mfma_kernel<2, false><<<dim3((unsigned)tiles, nkv, num_seqs), 64, 0, stream>>>(P);
+  } else {
+    const long long wg = (tiles + SHARED_WAVES - 1) / SHARED_WAVES;
+    attention_mfma_shared_kernel<<<dim3((unsigned)wg, nkv, num_seqs), 64 * SHARED_WAVES, 0, stream>>>(P);
   }
   return sl_launch_status();
 }

@@ -507,6 +507,7 @@ class HipOps:
         return out
 
     TARGET_WAVES = 1024           # wavefronts a decode launch aims for when it splits the context
+    SHARED_ATTENTION_WAVES = 4096  # prompt launches of this many 32-column wavefronts share keys through LDS
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples
@@ -544,8 +545,8 @@ class HipOps:
             fn.restype = ctypes.c_char_p
             self._fn[name] = fn
         if n_pre:
-            self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, 1, _p(out),
-                       None, None, 0, 0)
+            self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, 1,
+                       self.SHARED_ATTENTION_WAVES, _p(out), None, None, 0, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
@@ -555,7 +556,7 @@ class HipOps:
             if nsplit > 1:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
-            self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, _p(out),
+            self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, _p(out),
                        _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0)
 
     # ------------------------------------------------------------- sampling

@@ -392,6 +392,55 @@ def test_paged_attention(both, nh, nkv, D, page, window):
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+@pytest.mark.parametrize("nh,nkv,D,page", [(8, 1, 32, 16), (28, 4, 128, 16), (6, 2, 192, 64),
+                                           (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16)])
+@pytest.mark.parametrize("window", [None, 16, 50])
+def test_prompt_attention_through_lds(nh, nkv, D, page, window):
+    """The prompt kernel whose wavefronts share each block of keys through LDS,
+    forced at sizes far below its crossover: portions that end inside a
+    workgroup's 128 columns, that start deep in a context, and one-token rows."""
+    from servelab_amd.kernels import HipOps
+    dt = torch.bfloat16
+    ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+    ops.SHARED_ATTENTION_WAVES = 0
+    seqs = [(130, 130), (277, 45), (64, 64), (200, 2), (333, 97), (16, 1), (145, 1)]
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=5)
+    scale = 1.0 / math.sqrt(D)
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
+    ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                              types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                       for k, v in vars(batch).items()}),
+                              scale, window)
+    assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+
+
+def test_attention_reference_point_moves_late():
+    """Scores that keep growing along the context, by more than the kernels'
+    lazy-rescale margin from block to block: the running reference of every
+    column has to move many times, in prompt portions and in split decode."""
+    from servelab_amd.kernels import HipOps
+    dt = torch.bfloat16
+    nh, nkv, D, page = 4, 2, 64, 16
+    emu = EmulatedOps(dt)
+    seqs = [(400, 400), (300, 1)]
+    for shared in (0, 1 << 30):
+        ops = HipOps(dt, "cuda:0")
+        ops.SHARED_ATTENTION_WAVES = shared
+        qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=11)
+        # key at position r has r / 2 on channel 0, queries have 1 there: the
+        # score grows by 16 (23 in units of log 2) per block of 32 keys
+        qkv[:, 0:nh * D:D] = 1.0
+        for s, (ctx, _) in enumerate(seqs):
+            for r in range(ctx):
+                kc[int(tables[s, r // page]), :, r % page, 0] = r / 2
+        got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, None)
+        ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                                  types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                           for k, v in vars(batch).items()}),
+                                  1.0, None)
+        assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+
+
 @pytest.mark.parametrize("D,page", [(16, 16), (32, 16), (128, 32)])
 @pytest.mark.parametrize("q_len", [1, 5])
 def test_attention_finds_one_key_at_edges(both, D, page, q_len):
