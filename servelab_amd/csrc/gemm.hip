@@ -541,11 +541,11 @@ extern "C" const char* sl_gemm_wide(const void* x, const void* wt, const float* 
 // The next chunk of x and of W is loaded while the current one is multiplied.
 // When N is small, K is split over `KS` workgroups (grid.y) that write float
 // partials [KS, M, N]; `splitk_reduce_kernel` adds them, the bias, and rounds.
-template <int MB, int NT, int KC>
-__global__ __launch_bounds__(256) void gemm_mid_kernel(
+template <int MB, int NT, int KC, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int out_f32, int gated, int KS) {
-  constexpr int WAVES = 4;
+  constexpr int THREADS = 64 * WAVES;
   __shared__ bf16x8 xs[2][KC][MB][64];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
   const int ntiles = (N + 15) / 16;
@@ -560,30 +560,35 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(
     wp[t] = wt + ((size_t)tile * KT * 64 + lane) * 8;
   }
   // this thread's share of a chunk of x: XF fragments (ks, mb, lane) = (idx / (MB * 64), idx / 64 % MB, idx % 64)
-  constexpr int XF = MB * KC / 4;
+  constexpr int XF = MB * KC * 64 / THREADS;
+  static_assert(XF * THREADS == MB * KC * 64, "a chunk of x must divide evenly over the threads");
   const __bf16* xsrc[XF];
   int xks[XF];
 #pragma unroll
   for (int j = 0; j < XF; ++j) {
-    const int idx = threadIdx.x + 256 * j;
+    const int idx = threadIdx.x + THREADS * j;
     const int fl = idx % 64, mb = idx / 64 % MB;
     xks[j] = idx / (MB * 64);
     const int m = 16 * mb + (fl & 15) < M ? 16 * mb + (fl & 15) : M - 1;
     xsrc[j] = x + (size_t)m * K + 8 * (fl >> 4);
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // Every load of the main loop is issued unconditionally (past the end: from
+  // the last k-step, replaced by zeros when it is stored): a load under a
+  // branch would make each later wait count it as possibly absent, which ends
+  // in waiting for all loads at once.
   auto load_x = [&](int c, bf16x8 (&xr)[XF]) {
 #pragma unroll
     for (int j = 0; j < XF; ++j) {
       const int ks = kbeg + c * KC + xks[j];
-      xr[j] = ks < kend ? *(const bf16x8*)(xsrc[j] + 32 * (size_t)ks) : zero;
+      xr[j] = *(const bf16x8*)(xsrc[j] + 32 * (size_t)(ks < kend ? ks : kend - 1));
     }
   };
-  auto store_x = [&](int buf, const bf16x8 (&xr)[XF]) {
+  auto store_x = [&](int buf, int c, const bf16x8 (&xr)[XF]) {
 #pragma unroll
     for (int j = 0; j < XF; ++j) {
-      const int idx = threadIdx.x + 256 * j;
-      xs[buf][idx / (MB * 64)][idx / 64 % MB][idx % 64] = xr[j];
+      const int idx = threadIdx.x + THREADS * j;
+      xs[buf][idx / (MB * 64)][idx / 64 % MB][idx % 64] = kbeg + c * KC + xks[j] < kend ? xr[j] : zero;
     }
   };
   auto load_w = [&](int c, bf16x8 (&a)[NT][KC]) {
@@ -600,33 +605,62 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int b = 0; b < MB; ++b) acc[t][b] = f32x4{0.f, 0.f, 0.f, 0.f};
-  bf16x8 a[NT][KC], a_next[NT][KC], xr[XF];
-  load_x(0, xr);
-  load_w(0, a);
-  store_x(0, xr);
-  for (int c = 0; c < nchunks; ++c) {
-    __syncthreads();
-    const bool more = c + 1 < nchunks;
-    if (more) {
-      load_x(c + 1, xr);
-      load_w(c + 1, a_next);
-    }
+  // Two sets of W registers, the chunk loop unrolled over them: the loads of
+  // the next chunk stay in flight until its own products need them (a copy
+  // from one set into the other would wait for them at once).
+  bf16x8 a0[NT][KC], a1[NT][KC], xr[XF];
+  // The x operands of a k-step are read from LDS two k-steps before their
+  // products; the scheduling barriers keep the compiler from moving the reads
+  // back next to their use, where every pair of products would wait out the
+  // full latency of LDS (this made the kernel's time grow with the rows of x).
+  auto multiply = [&](int buf, const bf16x8 (&a)[NT][KC]) {
+    bf16x8 bv[2][MB];
 #pragma unroll
-    for (int u = 0; u < KC; ++u)
+    for (int u = 0; u < 2 && u < KC; ++u)
 #pragma unroll
-      for (int b = 0; b < MB; ++b) {
-        const bf16x8 bv = xs[c & 1][u][b][lane];
+      for (int b = 0; b < MB; ++b) bv[u][b] = xs[buf][u][b][lane];
+#pragma unroll
+    for (int u = 0; u < KC; ++u) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int b = 0; b < MB; ++b)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv, acc[t][b], 0, 0, 0);
+          acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv[u & 1][b], acc[t][b], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (u + 2 < KC) {
+#pragma unroll
+        for (int b = 0; b < MB; ++b) bv[u & 1][b] = xs[buf][u + 2][b][lane];
       }
-    if (more) {
-      store_x((c + 1) & 1, xr);
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int u = 0; u < KC; ++u) a[t][u] = a_next[t][u];
     }
+  };
+  load_x(0, xr);
+  load_w(0, a0);
+  store_x(0, 0, xr);
+  int c = 0;
+  for (; c + 2 < nchunks; c += 2) {
+    __syncthreads();
+    load_x(c + 1, xr);
+    load_w(c + 1, a1);
+    multiply(0, a0);
+    store_x(1, c + 1, xr);
+    __syncthreads();
+    load_x(c + 2, xr);
+    load_w(c + 2, a0);
+    multiply(1, a1);
+    store_x(0, c + 2, xr);
+  }
+  // the last one or two chunks
+  __syncthreads();
+  if (c + 1 < nchunks) {
+    load_x(c + 1, xr);
+    load_w(c + 1, a1);
+  }
+  multiply(0, a0);
+  if (c + 1 < nchunks) {
+    store_x(1, c + 1, xr);
+    __syncthreads();
+    multiply(1, a1);
   }
   // lane: column m = 16 b + i of x, rows n = 16 tile + 4 gq + r of W
 #pragma unroll
@@ -685,7 +719,7 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, const float
 // ks > 1: `part` holds ks * M * N floats.
 extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* bias, void* y,
                                    int M, int N, int K, int out_f32, int gated, int ks,
-                                   float* part, hipStream_t stream) {
+                                   int wide_min_wgs, float* part, hipStream_t stream) {
   SL_CHECK(M > 0 && N > 0 && K > 0, "gemm_mid: sizes must be positive");
   SL_CHECK(M <= 64, "gemm_mid: at most 64 rows");
   SL_CHECK(K % 32 == 0, "gemm_mid: K must be a multiple of 32");
@@ -699,10 +733,17 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
   const __bf16* xx = (const __bf16*)x;
   const __bf16* ww = (const __bf16*)wt;
   void* dst = ks > 1 ? (void*)part : y;
-  // two tiles per wavefront and chunks of four k-steps measured fastest (against 1 and 4 tiles, 8 k-steps)
-  const dim3 grid((ntiles + 7) / 8, ks);
-  if (M <= 32) gemm_mid_kernel<2, 2, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
-  else gemm_mid_kernel<4, 2, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+  // chunks of four k-steps, two tiles per wavefront; 8 wavefronts (16 tiles
+  // share one pass over x) when that still leaves wide_min_wgs workgroups
+  const bool wide = ((ntiles + 15) / 16) * ks >= wide_min_wgs;
+  const dim3 grid(wide ? (ntiles + 15) / 16 : (ntiles + 7) / 8, ks);
+  if (wide) {
+    if (M <= 32) gemm_mid_kernel<2, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    else gemm_mid_kernel<4, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+  } else {
+    if (M <= 32) gemm_mid_kernel<2, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    else gemm_mid_kernel<4, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+  }
   const char* e = sl_launch_status();
   if (e || ks == 1) return e;
   const size_t total = (size_t)M * N;

@@ -302,6 +302,7 @@ class HipOps:
         return y
 
     MID_TARGET_WORKGROUPS = 448
+    MID_WIDE_WORKGROUPS = 128      # workgroups of 8 wavefronts (16 tiles of W per pass over x) if this many remain
     MID_MIN_ELEMENTS = 48 << 20   # matrices from this size on take the LDS-staged kernel at 17..64 rows
 
     def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None):
@@ -317,7 +318,7 @@ class HipOps:
         part = self._new((ks, M, N), torch.float32) if ks > 1 else None
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_mid", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
-                   int(out_f32), int(gated), int(ks), _p(part))
+                   int(out_f32), int(gated), int(ks), self.MID_WIDE_WORKGROUPS, _p(part))
         return y
 
     def linear_skinny(self, x, weight, bias, out_f32=False):
