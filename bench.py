@@ -159,15 +159,19 @@ def time_decode(model, batch, ctx_end, steps, warmup, page, seed=0):
     return dt / steps, mean_ctx
 
 
-def time_prefill(model, T, page, repeats, max_chunk, seed=1):
+def time_prefill(model, T, page, repeats, max_chunk, seed=1, tune=True):
     """A prompt of T tokens from an empty cache, in portions of at most
-    ``max_chunk`` tokens (one portion when T fits)."""
+    ``max_chunk`` tokens (one portion when T fits).  ``tune``: before the
+    warm-up run the library's kernels are timed for a portion of that size, as
+    the engine does at start-up with ``tune_products``."""
     import torch
     from servelab_amd.engine import ModelRunner, StepEntry
     runner = ModelRunner(model, -(-T // page) + 8, page, max_num_seqs=4)
     vocab = model.spec.vocab_size
     toks = torch.randint(0, vocab, (T,), generator=torch.Generator().manual_seed(seed)).tolist()
     ops = model.rt.ops
+    if tune:
+        runner.tune_products([min(max_chunk, T)])
 
     def once(tag):
         pos = 0
@@ -208,6 +212,8 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-tune", action="store_true",
+                    help="leave the library's default kernel choice for the prompt products")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
@@ -239,13 +245,15 @@ def main():
             "page_size": page, "prefill_tokens": args.prefill_tokens,
             "decode_mean_context": round(mean_ctx, 1), "sampling": "greedy",
             "weight_layout": model.rt.ops.weight_layout,
+            "library_tuning": "off" if args.no_tune or args.no_prefill else "tunableop",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
     if not args.no_prefill:
         T = args.prefill_tokens
-        pre_s = time_prefill(model, T, page, repeats=3, max_chunk=args.prefill_chunk)
+        pre_s = time_prefill(model, T, page, repeats=3, max_chunk=args.prefill_chunk,
+                             tune=not args.no_tune)
         line["prefill"] = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
                            "frac": round(prefill_flops(cfg, T) / pre_s / PEAK_FLOPS[short], 4)}
     if not args.no_points:

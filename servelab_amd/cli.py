@@ -42,6 +42,9 @@ def build_parser():
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--max-num-seqs", type=int, default=16)
     ap.add_argument("--max-batched-tokens", type=int, default=1024)
+    ap.add_argument("--tune-products", action="store_true",
+                    help="at start-up, time the library's matrix kernels for a full-budget step "
+                         "and keep the fastest (bfloat16 only)")
     return ap
 
 
@@ -81,7 +84,7 @@ def main(argv=None) -> int:
         mc, CacheConfig(block_size=args.block_size, num_blocks=args.num_blocks or None),
         SchedulerConfig(max_num_seqs=args.max_num_seqs,
                         max_num_batched_tokens=args.max_batched_tokens),
-        seed=args.seed, tokenizer=tokenizer, dtype=args.dtype)
+        seed=args.seed, tokenizer=tokenizer, dtype=args.dtype, tune_products=args.tune_products)
     if args.prompt_ids:
         prompts = [[int(t) for t in args.prompt_ids.split(",")]]
     elif tokenizer is not None:

@@ -48,3 +48,4 @@ class EngineConfig:
     seed: int = 1234
     dtype: str = "auto"                    # auto (config.json's torch_dtype) | bfloat16 | float32
     device: str = "cuda:0"
+    tune_products: bool = False            # time the library's kernels for full-budget steps at start-up

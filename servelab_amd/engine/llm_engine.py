@@ -24,7 +24,7 @@ class LLMEngine:
                  scheduler_config: Optional[SchedulerConfig] = None, seed: int = 1234,
                  device: str = "cuda:0", tokenizer=None,
                  clock: Optional[Callable[[], float]] = None, dtype: str = "auto",
-                 model=None, ops=None):
+                 model=None, ops=None, tune_products: bool = False):
         """``model_config.path`` names the model folder (as in the reference,
         servelab/engine/engine.py:86-87); ``model`` may pass an already loaded
         DecoderModel instead."""
@@ -49,6 +49,9 @@ class LLMEngine:
                                   self.scheduler_config.max_num_seqs,
                                   self.cache_config.gpu_memory_utilization)
         self.num_blocks = self.runner.manager.num_pages
+        if tune_products:
+            # a step that uses its whole token budget is the common large step under load
+            self.runner.tune_products([self.scheduler_config.max_num_batched_tokens])
         self.scheduler = Scheduler(self.scheduler_config, self.runner.manager, self.clock,
                                    eos_token_id=model.spec.eos_token_id,
                                    max_positions=model.spec.max_position_embeddings)

@@ -207,6 +207,33 @@ class ModelRunner:
         return logits
 
     @torch.no_grad()
+    def tune_products(self, row_counts, max_ms: int = 30) -> List[int]:
+        """Runs one throw-away prompt portion of each given length with the
+        kernel table's library tuning on, so that the library products of a
+        step with that many rows use the fastest kernel the library has for
+        them.  Lengths the empty pool cannot hold are left out; returns the
+        lengths tuned.  A no-op for kernel tables without library products."""
+        tuning = getattr(self.model.rt.ops, "library_tuning", None)
+        if tuning is None or self.model.rt.act_dtype != torch.bfloat16:
+            return []
+        done = []
+        with tuning(max_ms):
+            for n in sorted(set(int(r) for r in row_counts)):
+                tag = ("tune_products", n)
+                if (n < 1 or n > self.max_positions or not self.manager.can_ever_hold(n)
+                        or not self.open(tag)):
+                    continue
+                try:
+                    self.step([StepEntry(tag, [0] * n, [n - 1])])
+                    done.append(n)
+                except OutOfPages:
+                    pass
+                finally:
+                    self.close(tag)
+        if self.rt.device.type == "cuda":
+            torch.cuda.synchronize(self.rt.device)
+        return done
+
     def step(self, entries: List[StepEntry]) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of
         the entries and of their ``want``."""

@@ -167,3 +167,28 @@ def test_tiled_only_weight_layout_runs_the_whole_model(tmp_path, monkeypatch):
         out += [runner.step([StepEntry("a", [t], [0])]).clone() for t in toks[70:]]
         rows[share] = torch.cat(out)
     assert torch.equal(rows[0.45], rows[0.0])
+
+
+def test_tuned_library_products_keep_the_logits(tmp_path):
+    """Start-up tuning of the library's kernels for a prompt portion of a given
+    size: the portion's logits stay within rounding of the untuned ones and of
+    the plain implementation, the choices land in a file under the temporary
+    folder, and lengths the pool cannot hold are left out."""
+    import os
+    import tempfile
+    folder = make_folder(tmp_path, "B", seed=31)
+    cfg, weights = plain.load_folder(folder)
+    toks = [(7 * i + 3) % cfg["vocab_size"] for i in range(96)]
+    _, model = load_model_on_device(folder, "bfloat16")
+    runner = ModelRunner(model, 16, 16)
+    before = runner.step([StepEntry("a", toks, [0, 50, 95])]).clone()
+    runner.close("a")
+    assert runner.tune_products([96, 100000], max_ms=3) == [96]
+    assert runner.manager.num_free_pages() == 16
+    after = runner.step([StepEntry("b", toks, [0, 50, 95])])
+    ref = plain.forward(cfg, weights, toks)[[0, 50, 95]]
+    tol = tolerance("bfloat16", {"a": ref.numpy()})
+    assert (after.cpu() - ref).abs().max().item() < tol
+    assert (after - before).abs().max().item() < tol
+    name = os.path.join(tempfile.gettempdir(), f"servelab_amd_tunableop_{os.getuid()}.csv")
+    assert os.path.exists(name)
