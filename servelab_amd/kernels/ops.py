@@ -416,7 +416,6 @@ class HipOps:
         if results_file is None:
             results_file = os.path.join(tempfile.gettempdir(),
                                         f"servelab_amd_tunableop_{os.getuid()}.csv")
-        was_tuning = tunable.tuning_is_enabled()
         tunable.set_filename(results_file)
         tunable.set_max_tuning_duration(int(max_ms))
         tunable.enable(True)
@@ -424,7 +423,7 @@ class HipOps:
         try:
             yield
         finally:
-            tunable.tuning_enable(was_tuning)      # the choices made stay in use
+            tunable.tuning_enable(False)           # the choices made stay in use; nothing new is timed
 
     def silu_mul(self, gate_up, block=None):
         T, two_i = gate_up.shape
