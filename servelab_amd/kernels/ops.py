@@ -535,7 +535,7 @@ class HipOps:
         return out
 
     TARGET_WAVES = 1024           # wavefronts a decode launch aims for when it splits the context
-    SHARED_ATTENTION_WAVES = 3072  # prompt launches of this many 32-column wavefronts share keys through LDS
+    SHARED_ATTENTION_WAVES = 2048  # prompt launches of this many 32-column wavefronts share keys through LDS
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples
