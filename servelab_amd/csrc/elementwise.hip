@@ -166,6 +166,74 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restri
   }
 }
 
+// The same work in two vectorised kernels, for head sizes that are multiples
+// of 16 (many-token steps: the per-pair kernel above needs one block of 64
+// threads per token and head and moves 2 bytes per access).
+struct __attribute__((aligned(16))) Act8 { act_t v[8]; };
+struct __attribute__((aligned(16))) F4 { float v[4]; };
+
+// q and k heads: a thread rotates 8 pairs (two 8-channel runs) of one head of
+// one token and writes them back, k also to its cache row.
+__global__ __launch_bounds__(256) void rope_store_qk_kernel(
+    act_t* __restrict__ qkv, const float* __restrict__ cosv, const float* __restrict__ sinv,
+    const int* __restrict__ slots, act_t* __restrict__ kc, int nh, int nkv, int D, int page,
+    int pairs8) {
+  const int t = blockIdx.x, half = D / 2, chunks = half / 8;
+  const int items = (nh + nkv) * chunks;
+  for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < items; w += gridDim.y * blockDim.x) {
+    const int hd = w / chunks, c = w % chunks;
+    const int p1 = pairs8 ? 16 * c : 8 * c, p2 = pairs8 ? p1 + 8 : p1 + half;
+    act_t* x = qkv + ((size_t)t * (nh + 2 * nkv) + hd) * D;
+    Act8 a = *(const Act8*)(x + p1), b = *(const Act8*)(x + p2);
+    if (cosv != nullptr) {
+      const float* cp = cosv + (size_t)t * half + 8 * c;
+      const float* sp = sinv + (size_t)t * half + 8 * c;
+      const F4 c0 = *(const F4*)cp, c1 = *(const F4*)(cp + 4);
+      const F4 s0 = *(const F4*)sp, s1 = *(const F4*)(sp + 4);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float cs = j < 4 ? c0.v[j] : c1.v[j - 4], sn = j < 4 ? s0.v[j] : s1.v[j - 4];
+        const float x1 = to_f(a.v[j]), x2 = to_f(b.v[j]);
+        a.v[j] = from_f<act_t>(x1 * cs - x2 * sn);
+        b.v[j] = from_f<act_t>(x2 * cs + x1 * sn);
+      }
+      *(Act8*)(x + p1) = a;
+      *(Act8*)(x + p2) = b;
+    }
+    if (hd >= nh && kc != nullptr) {
+      const int slot = slots[t];
+      act_t* dst = kc + (((size_t)(slot / page) * nkv + (hd - nh)) * page + slot % page) * D;
+      *(Act8*)(dst + p1) = a;
+      *(Act8*)(dst + p2) = b;
+    }
+  }
+}
+
+// v heads: a block takes 16 consecutive tokens of one kv head through LDS, so
+// that neighbouring lanes write neighbouring slots of a channel's row (tokens
+// of one request usually sit in consecutive slots of a page).
+__global__ __launch_bounds__(256) void store_v_kernel(
+    const act_t* __restrict__ qkv, const int* __restrict__ slots, act_t* __restrict__ vc, int T,
+    int nh, int nkv, int D, int page) {
+  __shared__ act_t tile[16][256 + 2];
+  __shared__ int slot_of[16];
+  const int t0 = blockIdx.x * 16, kvh = blockIdx.y;
+  const int nt = T - t0 < 16 ? T - t0 : 16;
+  if (threadIdx.x < 16) slot_of[threadIdx.x] = threadIdx.x < nt ? slots[t0 + threadIdx.x] : 0;
+  for (int idx = threadIdx.x; idx < nt * D; idx += blockDim.x) {
+    const int i = idx / D, d = idx % D;
+    tile[i][d] = qkv[((size_t)(t0 + i) * (nh + 2 * nkv) + nh + nkv + kvh) * D + d];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 16 * D; idx += blockDim.x) {
+    const int i = idx % 16, d = idx / 16;
+    if (i < nt) {
+      const int slot = slot_of[i];
+      vc[(((size_t)(slot / page) * nkv + kvh) * D + d) * page + slot % page] = tile[i][d];
+    }
+  }
+}
+
 extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* sinv,
                                      const int* slots, void* kc, void* vc, int T, int nh, int nkv,
                                      int D, int page, int pairs8, hipStream_t stream) {
@@ -178,6 +246,18 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
   if (T == 0) return nullptr;
   const int heads = kc != nullptr ? nh + 2 * nkv : nh + nkv;
   if (cosv == nullptr && kc == nullptr) return nullptr;
+  const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kc % 16) == 0 &&
+                       ((uintptr_t)cosv % 16) == 0 && ((uintptr_t)sinv % 16) == 0;
+  if (T >= 16 && D % 16 == 0 && D <= 256 && aligned && nkv <= 65535) {
+    const int items = (nh + nkv) * (D / 16);
+    rope_store_qk_kernel<<<dim3(T, (items + 255) / 256 < 64 ? (items + 255) / 256 : 64), 256, 0, stream>>>(
+        (act_t*)qkv, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, page, pairs8);
+    const char* e = sl_launch_status();
+    if (e || vc == nullptr) return e;
+    store_v_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>((const act_t*)qkv, slots, (act_t*)vc, T,
+                                                                 nh, nkv, D, page);
+    return sl_launch_status();
+  }
   rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, cosv, sinv, slots, (act_t*)kc,
                                                        (act_t*)vc, nh, nkv, D, page, pairs8);
   return sl_launch_status();
