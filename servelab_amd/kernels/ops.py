@@ -598,15 +598,24 @@ class HipOps:
         return out
 
     def sample(self, logits, temperature, top_k, top_p, seeds, draws):
-        """One token per row; rows with temperature 0 take the argmax."""
+        """One token per row; rows with temperature 0 take the argmax.  ``top_k``
+        and ``top_p`` both None: no row is cut, which takes the faster
+        two-stage kernel."""
         R, V = logits.shape
         self._check(logits, torch.float32, None, "logits")
         self._check(temperature, torch.float32, (R,), "temperature")
-        self._check(top_k, torch.int32, (R,), "top_k")
-        self._check(top_p, torch.float32, (R,), "top_p")
         self._check(seeds, torch.int64, (R,), "seeds")
         self._check(draws, torch.int64, (R,), "draws")
+        if (top_k is None) != (top_p is None):
+            raise KernelError("sample: top_k and top_p go together")
         out = self._new((R,), torch.int32)
+        chunks, part = 0, None
+        if top_k is None:
+            chunks = max(1, min(64, V // 2048))
+            part = self._new((R, chunks, 2), torch.float32)
+        else:
+            self._check(top_k, torch.int32, (R,), "top_k")
+            self._check(top_p, torch.float32, (R,), "top_p")
         self._call("sampling", "sl_sample", _p(logits), R, V, _p(temperature), _p(top_k),
-                   _p(top_p), _p(seeds), _p(draws), _p(out))
+                   _p(top_p), _p(seeds), _p(draws), chunks, _p(part), _p(out))
         return out

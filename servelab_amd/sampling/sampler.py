@@ -9,6 +9,7 @@ tokens the request has drawn), so it does not depend on the batch it shares.
 """
 from typing import List, Sequence
 
+import numpy as np
 import torch
 
 
@@ -37,14 +38,18 @@ class Sampler:
             return []
         if all(p.temperature == 0.0 for p in params):
             return self.ops.argmax(logits).tolist()
-        host = torch.tensor(
-            [[p.temperature, p.top_p] for p in params], dtype=torch.float32)
-        ints = torch.tensor([[self.row_seed(p, n), d] for p, n, d in zip(params, numbers, draws)],
-                            dtype=torch.int64)
-        top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32)
-        temperature = host[:, 0].contiguous().to(self.device)
-        top_p = host[:, 1].contiguous().to(self.device)
-        seeds = ints[:, 0].contiguous().to(self.device)
-        counters = ints[:, 1].contiguous().to(self.device)
-        return self.ops.sample(logits, temperature, top_k.to(self.device), top_p, seeds,
-                               counters).tolist()
+        # one host buffer and one copy for the five per-row arrays:
+        # seeds and draw counters (int64), temperature and top_p (float32), top_k (int32)
+        B = len(params)
+        buf = np.empty(7 * B, dtype=np.int32)
+        buf[:2 * B].view(np.int64)[:] = [self.row_seed(p, n) for p, n in zip(params, numbers)]
+        buf[2 * B:4 * B].view(np.int64)[:] = list(draws)
+        buf[4 * B:5 * B].view(np.float32)[:] = [p.temperature for p in params]
+        buf[5 * B:6 * B].view(np.float32)[:] = [p.top_p for p in params]
+        buf[6 * B:] = [p.top_k for p in params]
+        dev = torch.from_numpy(buf).to(self.device)
+        cut = any(p.top_k > 0 or p.top_p < 1.0 for p in params)
+        return self.ops.sample(
+            logits, dev[4 * B:5 * B].view(torch.float32), dev[6 * B:] if cut else None,
+            dev[5 * B:6 * B].view(torch.float32) if cut else None,
+            dev[:2 * B].view(torch.int64), dev[2 * B:4 * B].view(torch.int64)).tolist()

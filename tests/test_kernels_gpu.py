@@ -495,6 +495,8 @@ def test_argmax_and_sampling():
     seeds = torch.full((n,), 1234, dtype=torch.int64).cuda()
     draws = torch.arange(n, dtype=torch.int64).cuda()
     toks = ops.sample(logits, temp, top_k, top_p, seeds, draws)
+    # rows without a cut draw the same token from the two-stage kernel (no top_k / top_p given)
+    assert torch.equal(toks, ops.sample(logits, temp, None, None, seeds, draws))
     freq = torch.bincount(toks.long().cpu(), minlength=V).float() / n
     want = torch.softmax(base / T, -1)
     assert (freq - want).abs().max().item() < 0.015
@@ -522,3 +524,39 @@ def test_argmax_and_sampling():
     toks = ops.sample(logits, temp, top_k, torch.full((n,), p).cuda(), seeds, draws)
     freq = torch.bincount(toks.long().cpu(), minlength=V).float() / n
     assert (freq - wantp).abs().max().item() < 0.015
+
+
+@pytest.mark.parametrize("V", [50000, 50001, 152064])
+def test_sampling_cuts_of_a_wide_vocabulary(V):
+    """top-k and top-p over a wide row (vector loads when the row is 16-byte
+    aligned, scalar ones otherwise): every drawn token lies inside the exact
+    cut, and the draws reach most of what the cut keeps."""
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.float32, "cuda:0")
+    R, T = 48, 0.9
+    logits = 2.5 * randn(1, V, seed=V).repeat(R, 1).contiguous()
+    logits[:, 1234] = logits.max() + 0.5
+    temp = torch.full((R,), T).cuda()
+    seeds = torch.full((R,), 99, dtype=torch.int64).cuda()
+    ones, none = torch.ones(R).cuda(), torch.full((R,), -1, dtype=torch.int32).cuda()
+    probs = torch.softmax(logits[0].double().cpu() / T, -1)
+    sp, si = torch.sort(probs, descending=True)
+    cum = torch.cumsum(sp, 0)
+
+    def draw(top_k, top_p, rounds=20):
+        got = []
+        for j in range(rounds):
+            draws = (torch.arange(R, dtype=torch.int64) + R * j).cuda()
+            got += ops.sample(logits, temp, top_k, top_p, seeds, draws).tolist()
+        return set(got)
+
+    k = 25
+    got = draw(torch.full((R,), k, dtype=torch.int32).cuda(), ones)
+    assert got <= set(si[:k].tolist()) and len(got) > k // 2
+    p = 0.35
+    inside = set(si[(cum <= p + 1e-4) | (torch.arange(V) == 0)].tolist())
+    surely = set(si[(cum <= p - 1e-4) | (torch.arange(V) == 0)].tolist())
+    got = draw(none, torch.full((R,), p).cuda())
+    assert got <= inside and len(got & surely) > min(len(surely), 40) // 2
+    # a top_p below the largest probability keeps that entry alone
+    assert draw(none, torch.full((R,), float(sp[0]) * 0.5).cuda(), rounds=2) == {1234}
