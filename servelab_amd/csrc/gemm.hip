@@ -212,19 +212,29 @@ struct RopeStore {
   int nh, nkv, D, page;
 };
 
-template <bool GATED, bool CONSUMER, bool PRODUCER, int PARTS, bool ROPE = false>
+// NT tiles (16 columns of y each) per workgroup share every load of x: with 8
+// to 16 rows the re-reads of x through L1 are a third to a half of all bytes a
+// CU pulls, and halving them shows (MI355X, gate/up of the 7B shape at 16 rows:
+// 66 us with one tile).  Matrices with few tiles keep one tile per workgroup so
+// that every CU has work.
+template <bool GATED, bool CONSUMER, bool PRODUCER, int PARTS, bool ROPE = false, int NT = 1>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int out_f32, const NormFusion F,
     const RopeStore R = RopeStore{}) {
-  constexpr int WAVES = 8, U = 8;
-  __shared__ f32x4 red[WAVES][64];
+  constexpr int WAVES = 8, U = NT == 1 ? 8 : 4;
+  __shared__ f32x4 red[NT][WAVES][64];
   __shared__ float wsum[WAVES][16];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int ntiles = (N + 15) / 16;
   const int KT = K / 32;
   const int ks0 = (int)((long long)KT * wave / WAVES), ks1 = (int)((long long)KT * (wave + 1) / WAVES);
-  const __bf16* wp = wt + ((size_t)blockIdx.x * KT * 64 + lane) * 8;
+  const __bf16* wp[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int tile = blockIdx.x * NT + t < ntiles ? blockIdx.x * NT + t : ntiles - 1;
+    wp[t] = wt + ((size_t)tile * KT * 64 + lane) * 8;
+  }
   int xrow = i < M ? i : M - 1;
   if (CONSUMER && F.rows != nullptr) xrow = F.rows[xrow];
   const __bf16* xp = x + (size_t)xrow * K + 8 * gq;
@@ -240,30 +250,45 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
       pv[j] = p < F.in_nparts ? F.in_parts[p * 16 + i] : 0.f;
     }
   }
-  const int em = threadIdx.x / 16, en = n0 + threadIdx.x % 16;       // epilogue element of threads < 256
-  float r_old = 0.f, g_next = 0.f;
-  if (PRODUCER && threadIdx.x < 256 && em < M && en < N) {
-    r_old = F.resid[(size_t)em * N + en];
-    g_next = F.next_w[en];
+  const int em = threadIdx.x / 16;                                   // epilogue row of threads < 256
+  float r_old[NT], g_next[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int en = (blockIdx.x * NT + t) * 16 + threadIdx.x % 16;
+    r_old[t] = g_next[t] = 0.f;
+    if (PRODUCER && threadIdx.x < 256 && em < M && en < N) {
+      r_old[t] = F.resid[(size_t)em * N + en];
+      g_next[t] = F.next_w[en];
+    }
   }
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   int ks = ks0;
   for (; ks + U <= ks1; ks += U) {
-    bf16x8 a[U];
+    bf16x8 a[NT][U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) a[u] = *(const bf16x8*)(wp + 512 * (size_t)(ks + u));
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)(ks + u));
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const bf16x8 bv = *(const bf16x8*)(xp + 32 * (size_t)(ks + u));
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv, acc[t], 0, 0, 0);
     }
   }
   for (; ks < ks1; ++ks) {
-    const bf16x8 a = *(const bf16x8*)(wp + 512 * (size_t)ks);
     const bf16x8 bv = *(const bf16x8*)(xp + 32 * (size_t)ks);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bv, acc, 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const bf16x8 a = *(const bf16x8*)(wp[t] + 512 * (size_t)ks);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bv, acc[t], 0, 0, 0);
+    }
   }
-  red[wave][lane] = acc;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) red[t][wave][lane] = acc[t];
   if (CONSUMER) {            // this wavefront's share of the sums of squares, by row
     float sacc = 0.f;
 #pragma unroll
@@ -280,73 +305,79 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     for (int wv = 0; wv < WAVES; ++wv) ss += wsum[wv][tok];
     return rsqrtf(ss / (float)K + F.eps);
   };
-  // lane (m + 16 (n_local / 4)) holds y[m, n_local] in element n_local % 4
-  if (GATED) {
-    if (threadIdx.x < 128) {
-      const int m = threadIdx.x / 8, j = threadIdx.x % 8;
-      const int n = blockIdx.x * 8 + j;
-      if (m < M && n < N / 2) {
-        float gsum = 0.f, usum = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < WAVES; ++wv) {
-          gsum += red[wv][m + 16 * (j / 4)][j % 4];
-          usum += red[wv][m + 16 * (2 + j / 4)][j % 4];
+  for (int t = 0; t < NT; ++t) {
+    const int tile = blockIdx.x * NT + t;
+    if (tile >= ntiles) break;
+    const int n0 = tile * 16;
+    // lane (m + 16 (n_local / 4)) holds y[m, n_local] in element n_local % 4
+    if (GATED) {
+      if (threadIdx.x < 128) {
+        const int m = threadIdx.x / 8, j = threadIdx.x % 8;
+        const int n = tile * 8 + j;
+        if (m < M && n < N / 2) {
+          float gsum = 0.f, usum = 0.f;
+#pragma unroll
+          for (int wv = 0; wv < WAVES; ++wv) {
+            gsum += red[t][wv][m + 16 * (j / 4)][j % 4];
+            usum += red[t][wv][m + 16 * (2 + j / 4)][j % 4];
+          }
+          if (CONSUMER) {
+            const float inv = inv_of(m);
+            gsum *= inv;
+            usum *= inv;
+          }
+          ((__bf16*)y)[(size_t)m * (N / 2) + n] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
         }
-        if (CONSUMER) {
-          const float inv = inv_of(m);
-          gsum *= inv;
-          usum *= inv;
-        }
-        ((__bf16*)y)[(size_t)m * (N / 2) + n] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
       }
+      continue;
     }
-    return;
-  }
-  if (threadIdx.x < 256) {
-    const int m = em, n_local = threadIdx.x % 16, n = en;
-    const bool live = m < M && n < N;
-    float s = 0.f;
+    if (threadIdx.x < 256) {
+      const int m = em, n_local = threadIdx.x % 16, n = n0 + n_local;
+      const bool live = m < M && n < N;
+      float s = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) s += red[wv][m + 16 * (n_local / 4)][n_local % 4];
-    if (CONSUMER && live) s *= inv_of(m);
-    if (live && bias != nullptr) s += bias[n];
-    if (ROPE) {
-      const float partner = __shfl_xor(s, 8, 64);      // the other half of the pair, same row
-      if (!live) return;
-      const int hd = n / R.D, p = n % R.D;
-      if (hd < R.nh + R.nkv) {
-        float val = s;
-        if (R.cosv != nullptr) {
-          const int j = 8 * (p / 16) + p % 8, half = R.D / 2;
-          const float c = R.cosv[(size_t)m * half + j], sn = R.sinv[(size_t)m * half + j];
-          val = p % 16 < 8 ? s * c - partner * sn : s * c + partner * sn;
-        }
-        if (hd < R.nh) {
-          ((__bf16*)y)[(size_t)m * N + n] = (__bf16)val;
+      for (int wv = 0; wv < WAVES; ++wv) s += red[t][wv][m + 16 * (n_local / 4)][n_local % 4];
+      if (CONSUMER && live) s *= inv_of(m);
+      if (live && bias != nullptr) s += bias[n];
+      if (ROPE) {
+        const float partner = __shfl_xor(s, 8, 64);      // the other half of the pair, same row
+        if (!live) continue;
+        const int hd = n / R.D, p = n % R.D;
+        if (hd < R.nh + R.nkv) {
+          float val = s;
+          if (R.cosv != nullptr) {
+            const int j = 8 * (p / 16) + p % 8, half = R.D / 2;
+            const float c = R.cosv[(size_t)m * half + j], sn = R.sinv[(size_t)m * half + j];
+            val = p % 16 < 8 ? s * c - partner * sn : s * c + partner * sn;
+          }
+          if (hd < R.nh) {
+            ((__bf16*)y)[(size_t)m * N + n] = (__bf16)val;
+          } else if (R.slots != nullptr) {
+            const int slot = R.slots[m];
+            R.kc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh)) * R.page + slot % R.page) * R.D + p] = (__bf16)val;
+          }
         } else if (R.slots != nullptr) {
           const int slot = R.slots[m];
-          R.kc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh)) * R.page + slot % R.page) * R.D + p] = (__bf16)val;
+          R.vc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh - R.nkv)) * R.D + p) * R.page + slot % R.page] = (__bf16)s;
         }
-      } else if (R.slots != nullptr) {
-        const int slot = R.slots[m];
-        R.vc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh - R.nkv)) * R.D + p) * R.page + slot % R.page] = (__bf16)s;
+        continue;
       }
-      return;
-    }
-    if (PRODUCER) {
-      float sq = 0.f;
-      if (live) {
-        const float r = r_old + s;
-        F.resid[(size_t)m * N + n] = r;
-        ((__bf16*)y)[(size_t)m * N + n] = (__bf16)(r * g_next);
-        sq = r * r;
-      }
+      if (PRODUCER) {
+        float sq = 0.f;
+        if (live) {
+          const float r = r_old[t] + s;
+          F.resid[(size_t)m * N + n] = r;
+          ((__bf16*)y)[(size_t)m * N + n] = (__bf16)(r * g_next[t]);
+          sq = r * r;
+        }
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);     // over the 16 columns of row m
-      if (n_local == 0) F.out_parts[(size_t)blockIdx.x * 16 + m] = sq;
-    } else if (live) {
-      if (out_f32) ((float*)y)[(size_t)m * N + n] = s;
-      else ((__bf16*)y)[(size_t)m * N + n] = (__bf16)s;
+        for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);     // over the 16 columns of row m
+        if (n_local == 0) F.out_parts[(size_t)tile * 16 + m] = sq;
+      } else if (live) {
+        if (out_f32) ((float*)y)[(size_t)m * N + n] = s;
+        else ((__bf16*)y)[(size_t)m * N + n] = (__bf16)s;
+      }
     }
   }
 }
@@ -354,11 +385,12 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
 // wt: W in the tiled layout, ceil(N / 16) * 16 rows (rows beyond N are zero).
 // At most 16 rows.  Fusion: in_parts != nullptr makes x un-normalised rows
 // (consumer), resid != nullptr makes the result a delta of the stream (producer).
+// pair_tiles: two tiles of W per workgroup (not for producers or q/k/v with rotary).
 extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float* bias, void* y,
                                       int M, int N, int K, int out_f32, int gated,
                                       const float* in_parts, int in_nparts, float eps,
                                       const int* rows, float* resid, const float* next_w,
-                                      float* out_parts, const RopeStore* rope,
+                                      float* out_parts, const RopeStore* rope, int pair_tiles,
                                       hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
   SL_CHECK(M <= 16, "gemm_skinny: at most 16 rows");
@@ -392,6 +424,17 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
     if (!consumer) gemm_skinny_kernel<false, false, false, 1, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
     else if (few) gemm_skinny_kernel<false, true, false, 8, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
     else gemm_skinny_kernel<false, true, false, 16, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+    return sl_launch_status();
+  }
+  const RopeStore none{};
+  if (pair_tiles && !producer) {                 // two tiles per workgroup (the large matrices: gate/up, head)
+    const dim3 grid2(((N + 15) / 16 + 1) / 2);
+    if (consumer && gated && few) gemm_skinny_kernel<true, true, false, 8, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
+    else if (consumer && gated) gemm_skinny_kernel<true, true, false, 16, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
+    else if (consumer && few) gemm_skinny_kernel<false, true, false, 8, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F, none);
+    else if (consumer) gemm_skinny_kernel<false, true, false, 16, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F, none);
+    else if (gated) gemm_skinny_kernel<true, false, false, 1, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
+    else gemm_skinny_kernel<false, false, false, 1, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F, none);
     return sl_launch_status();
   }
   if (producer) gemm_skinny_kernel<false, false, true, 1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);

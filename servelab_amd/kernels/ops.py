@@ -81,6 +81,8 @@ class ScaledRows:
 
 class HipOps:
     ROWS_KERNEL_MAX_M = 16        # the wavefront-per-column GEMM is used up to this many rows
+    PAIR_TILES_MIN = 1024         # few-rows products with this many 16-row tiles of W take two per workgroup ...
+    PAIR_TILES_MIN_ROWS = 4       # ... from this many rows of x on (below, x is too small to matter)
     SKINNY_MAX_M = 64             # the matrix-core few-rows GEMM takes up to this many rows
 
     # Decode reads every weight once per step and is bound by how fast it
@@ -147,7 +149,8 @@ class HipOps:
                    int(out_f32), int(gated), _p(parts), parts.shape[0] if parts is not None else 0,
                    _c_float(scaled.eps if scaled is not None else 0.0),
                    _p(scaled.rows) if scaled is not None else None, _p(resid), _p(next_gain),
-                   _p(out_parts), ctypes.byref(rope) if rope is not None else None)
+                   _p(out_parts), ctypes.byref(rope) if rope is not None else None,
+                   int(M >= self.PAIR_TILES_MIN_ROWS and -(-N // 16) >= self.PAIR_TILES_MIN))
 
     # ------------------------------------------------------------ embedding
     def embed(self, ids, table):
