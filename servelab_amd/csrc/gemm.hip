@@ -511,9 +511,15 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(
           acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv[b][u], acc[t][b], 0, 0, 0);
   };
   if (!AHEAD) {
-    for (int g = 0; g < nfull; ++g) {
+    for (int ks = ks0; ks + U <= ks1; ks += U) {
       bf16x8 a[NT][U], bv[MB][U];
-      load_group(g, a, bv);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)(ks + u));
+#pragma unroll
+        for (int b = 0; b < MB; ++b) bv[b][u] = *(const bf16x8*)(xp[b] + 32 * (size_t)(ks + u));
+      }
       multiply_group(a, bv);
     }
   } else if (nfull > 0) {

@@ -270,13 +270,13 @@ def test_rope_tables(both):
 
 
 @pytest.mark.parametrize("pairs8", [False, True])
-@pytest.mark.parametrize("T", [5, 37, 100])        # per-pair kernel below 16 tokens, vectorised kernels above
+@pytest.mark.parametrize("T", [5, 37, 300])        # per-pair kernel for few tokens, vectorised kernels for many
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (6, 1, 48, 32), (7, 7, 128, 64), (3, 1, 24, 16)])
 def test_rope_store(both, nh, nkv, D, page, pairs8, T):
     ops, emu, dt = both
     if pairs8 and D % 16:
         pytest.skip("the blocked pair order needs head sizes in steps of 16")
-    pages = 9
+    pages = 9 if T < 100 else 30
     qkv = randn(T, (nh + 2 * nkv) * D, dtype=dt, seed=1)
     inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
     pos = torch.arange(100, 100 + T, dtype=torch.int32).cuda()
