@@ -129,13 +129,32 @@ extern "C" const char* sl_rope_tables(const int* pos, const float* inv_freq, flo
 // 8b..8b+7 followed by their partners D/2+8b..D/2+8b+7, so that pair j sits at
 // 16 (j / 8) + j % 8 and 8 further.  Scores do not depend on the order of the
 // channels as long as q and the cached k agree; v keeps its order.
-__global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restrict__ cosv,
+// The float partial sums of a q/k/v product whose K was split over workgroups
+// ([nparts][T][N], bias not yet added): the kernel below then reads its input
+// from them instead of from qkv, which saves the product a kernel that only
+// adds them up.
+struct SplitProduct {
+  const float* parts;            // or nullptr: the input is qkv itself
+  int nparts;
+  size_t stride;                 // T * N
+  const float* bias;             // [N] or nullptr
+};
+
+__global__ void rope_store_kernel(act_t* __restrict__ qkv, const SplitProduct sp,
+                                  const float* __restrict__ cosv,
                                   const float* __restrict__ sinv, const int* __restrict__ slots,
                                   act_t* __restrict__ kc, act_t* __restrict__ vc, int nh, int nkv,
                                   int D, int page, int pairs8) {
   const int t = blockIdx.x, hd = blockIdx.y;
   const int half = D / 2;
-  act_t* x = qkv + ((size_t)t * (nh + 2 * nkv) + hd) * D;
+  const size_t row = ((size_t)t * (nh + 2 * nkv) + hd) * D;
+  act_t* x = qkv + row;
+  auto input = [&](int c) {
+    if (sp.parts == nullptr) return to_f(x[c]);
+    float v = sp.bias != nullptr ? sp.bias[hd * D + c] : 0.f;
+    for (int j = 0; j < sp.nparts; ++j) v += sp.parts[j * sp.stride + row + c];
+    return v;
+  };
   if (hd < nh + nkv) {
     act_t* dst = nullptr;
     if (hd >= nh && kc != nullptr) {
@@ -145,12 +164,15 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restri
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
       const int p1 = pairs8 ? 16 * (j / 8) + j % 8 : j;
       const int p2 = pairs8 ? p1 + 8 : j + half;
-      float x1 = to_f(x[p1]), x2 = to_f(x[p2]);
+      float x1 = input(p1), x2 = input(p2);
       if (cosv != nullptr) {
         const float c = cosv[(size_t)t * half + j], s = sinv[(size_t)t * half + j];
         const float r1 = x1 * c - x2 * s, r2 = x2 * c + x1 * s;
         x1 = r1;
         x2 = r2;
+      }
+      // in place: whatever was rotated; from partial sums: q (k lives on in the pages only)
+      if (sp.parts != nullptr ? hd < nh : cosv != nullptr) {
         x[p1] = from_f<act_t>(x1);
         x[p2] = from_f<act_t>(x2);
       }
@@ -162,7 +184,7 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const float* __restri
   } else if (vc != nullptr) {
     const int slot = slots[t];
     act_t* dst = vc + ((size_t)(slot / page) * nkv + (hd - nh - nkv)) * D * page + slot % page;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[(size_t)d * page] = x[d];
+    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[(size_t)d * page] = from_f<act_t>(input(d));
   }
 }
 
@@ -237,21 +259,27 @@ __global__ __launch_bounds__(256) void store_v_kernel(
   }
 }
 
+// parts != nullptr: the input is the sum of nparts float partial products
+// [nparts][T][N] plus bias; q is then written to qkv, k and v only to the pages.
 extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* sinv,
                                      const int* slots, void* kc, void* vc, int T, int nh, int nkv,
-                                     int D, int page, int pairs8, hipStream_t stream) {
+                                     int D, int page, int pairs8, const float* parts, int nparts,
+                                     const float* bias, hipStream_t stream) {
   SL_CHECK(T >= 0 && nh > 0 && nkv > 0, "rope_store: sizes must be positive");
   SL_CHECK(D > 0 && D % 2 == 0, "rope_store: head_dim must be even");
   SL_CHECK(!pairs8 || D % 16 == 0, "rope_store: the blocked pair order needs head_dim % 16 == 0");
   SL_CHECK((cosv == nullptr) == (sinv == nullptr), "rope_store: cos and sin go together");
   SL_CHECK((kc == nullptr) == (vc == nullptr), "rope_store: k and v pages go together");
   SL_CHECK(kc == nullptr || (slots != nullptr && page > 0), "rope_store: pages need slots");
+  SL_CHECK(parts == nullptr || nparts >= 1, "rope_store: partial products need their count");
+  SL_CHECK(parts != nullptr || bias == nullptr, "rope_store: a bias comes with partial products only");
+  const SplitProduct sp{parts, nparts, (size_t)T * (nh + 2 * nkv) * D, bias};
   if (T == 0) return nullptr;
   const int heads = kc != nullptr ? nh + 2 * nkv : nh + nkv;
-  if (cosv == nullptr && kc == nullptr) return nullptr;
+  if (cosv == nullptr && kc == nullptr && parts == nullptr) return nullptr;
   const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kc % 16) == 0 &&
                        ((uintptr_t)cosv % 16) == 0 && ((uintptr_t)sinv % 16) == 0;
-  if (T >= VECTOR_MIN_TOKENS && D % 16 == 0 && D <= 256 && aligned && nkv <= 65535) {
+  if (parts == nullptr && T >= VECTOR_MIN_TOKENS && D % 16 == 0 && D <= 256 && aligned && nkv <= 65535) {
     const int items = (nh + nkv) * (D / 16);
     rope_store_qk_kernel<<<dim3(T, (items + 255) / 256 < 64 ? (items + 255) / 256 : 64), 256, 0, stream>>>(
         (act_t*)qkv, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, page, pairs8);
@@ -261,7 +289,7 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
                                                                  nh, nkv, D, page);
     return sl_launch_status();
   }
-  rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, cosv, sinv, slots, (act_t*)kc,
+  rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, sp, cosv, sinv, slots, (act_t*)kc,
                                                        (act_t*)vc, nh, nkv, D, page, pairs8);
   return sl_launch_status();
 }

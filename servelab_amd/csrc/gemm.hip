@@ -799,7 +799,8 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, const float
   }
 }
 
-// ks > 1: `part` holds ks * M * N floats.
+// ks > 1: `part` holds ks * M * N floats; with y == nullptr they are left there
+// for the reader to add (and the bias with them).
 extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* bias, void* y,
                                    int M, int N, int K, int out_f32, int gated, int ks,
                                    int wide_min_wgs, float* part, hipStream_t stream) {
@@ -808,6 +809,7 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
   SL_CHECK(K % 32 == 0, "gemm_mid: K must be a multiple of 32");
   SL_CHECK(ks >= 1 && ks <= 16 && ks <= K / 32, "gemm_mid: ks must be in 1..16 and <= K / 32");
   SL_CHECK(ks == 1 || part != nullptr, "gemm_mid: a split of K needs the partial buffer");
+  SL_CHECK(y != nullptr || ks > 1, "gemm_mid: no output");
   SL_CHECK(!gated || (ks == 1 && N % 16 == 0 && bias == nullptr && !out_f32),
            "gemm_mid: the gated form needs ks == 1, N % 16 == 0, no bias, activation output");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
@@ -828,7 +830,16 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
     else gemm_mid_kernel<4, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
   }
   const char* e = sl_launch_status();
-  if (e || ks == 1) return e;
+  if (e || ks == 1 || y == nullptr) return e;
+  const size_t total = (size_t)M * N;
+  splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(part, bias, y, M, N, ks, out_f32);
+  return sl_launch_status();
+}
+
+// y = sum of the ks partial sums [ks, M, N] (+ bias)
+extern "C" const char* sl_splitk_reduce(const float* part, const float* bias, void* y, int M, int N,
+                                        int ks, int out_f32, hipStream_t stream) {
+  SL_CHECK(M > 0 && N > 0 && ks >= 1, "splitk_reduce: sizes must be positive");
   const size_t total = (size_t)M * N;
   splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(part, bias, y, M, N, ks, out_f32);
   return sl_launch_status();

@@ -63,6 +63,17 @@ class Deferred:
         self.x, self.weight, self.bias = x, weight, bias
 
 
+class PartialSums:
+    """A product whose K was split over workgroups, left as float partial sums
+    ``parts`` [ks, T, N] with the bias not yet added, for a reader that adds
+    them up on its way (``rope_store``); ``HipOps.materialize`` makes the plain
+    tensor."""
+    __slots__ = ("parts", "bias")
+
+    def __init__(self, parts, bias):
+        self.parts, self.bias = parts, bias
+
+
 class ScaledRows:
     """Rows [T, H] that are normalised but for the factor rsqrt(mean x^2 + eps):
     ``x`` holds stream * gain in the activation dtype, ``parts`` [nparts, 16] the
@@ -206,6 +217,11 @@ class HipOps:
         """The plain tensor of a ``Deferred`` product (anything else is returned as it is)."""
         if isinstance(value, Deferred):
             return self.linear(value.x, value.weight, value.bias)
+        if isinstance(value, PartialSums):
+            ks, M, N = value.parts.shape
+            y = self._new((M, N))
+            self._call("gemm", "sl_splitk_reduce", _p(value.parts), _p(value.bias), _p(y), M, N, ks, 0)
+            return y
         return value
 
     def _produce_scaled_rows(self, resid, d, gain, eps):
@@ -308,20 +324,27 @@ class HipOps:
         return y
 
     MID_TARGET_WORKGROUPS = 448
+    MID_PARTIAL_WORKGROUPS = 128   # fewer splits when the reader adds the partial sums (their bytes count twice)
     MID_WIDE_WORKGROUPS = 128      # workgroups of 8 wavefronts (16 tiles of W per pass over x) if this many remain
     MID_MIN_ELEMENTS = 48 << 20   # matrices from this size on take the LDS-staged kernel at 17..64 rows
 
-    def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None):
+    def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None, partial=False):
         """17..64 rows with x staged through LDS; K split over workgroups when
-        N alone gives too few of them."""
+        N alone gives too few of them.  ``partial``: a split product comes back
+        as ``PartialSums`` for its reader to add up."""
         M, K = x.shape
         N = weight.shape[0]
         if weight.tiled is None:
             raise KernelError("linear_mid needs the tiled copy of the weight")
         wgs = -(-(-(-N // 16)) // 8)
         if ks is None:
-            ks = 1 if gated else max(1, min(16, K // 32 // 4, -(-self.MID_TARGET_WORKGROUPS // wgs)))
+            target = self.MID_PARTIAL_WORKGROUPS if partial else self.MID_TARGET_WORKGROUPS
+            ks = 1 if gated else max(1, min(16, K // 32 // 4, -(-target // wgs)))
         part = self._new((ks, M, N), torch.float32) if ks > 1 else None
+        if partial and ks > 1:
+            self._call("gemm", "sl_gemm_mid", _p(x), _p(weight.tiled), None, None, M, N, K,
+                       0, 0, int(ks), self.MID_WIDE_WORKGROUPS, _p(part))
+            return PartialSums(part, bias)
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_mid", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                    int(out_f32), int(gated), int(ks), self.MID_WIDE_WORKGROUPS, _p(part))
@@ -459,13 +482,21 @@ class HipOps:
         return pages
 
     def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                   pairs8=False):
+                   pairs8=False, split=None):
         """Rotate q and k of ``qkv`` in place (``cos`` None: no rotation) and write
         k and v to their cache rows (``k_cache`` None: no write).  ``pairs8``:
         the channels of q and k heads come in blocks of 8 channels and their 8
-        partners (the order ``qkv_rope_store`` uses), else first and second half."""
+        partners (the order ``qkv_rope_store`` uses), else first and second half.
+        ``split``: the product arrives as ``PartialSums``; ``qkv`` is then only
+        written (its q columns)."""
         T = qkv.shape[0]
         self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
+        parts = bias = None
+        if split is not None:
+            parts, bias = split.parts, split.bias
+            self._check(parts, torch.float32, (parts.shape[0], T, (nh + 2 * nkv) * D), "partial sums")
+            if bias is not None:
+                self._check(bias, torch.float32, ((nh + 2 * nkv) * D,), "bias")
         if cos is not None:
             self._check(cos, torch.float32, (T, D // 2), "cos")
             self._check(sin, torch.float32, (T, D // 2), "sin")
@@ -473,7 +504,8 @@ class HipOps:
             self._check_pages(k_cache, v_cache, nkv, D, page_size)
             self._check(slots, torch.int32, (T,), "slots")
         self._call("elementwise", "sl_rope_store", _p(qkv), _p(cos), _p(sin), _p(slots),
-                   _p(k_cache), _p(v_cache), T, nh, nkv, D, page_size, int(pairs8))
+                   _p(k_cache), _p(v_cache), T, nh, nkv, D, page_size, int(pairs8),
+                   _p(parts), parts.shape[0] if parts is not None else 0, _p(bias))
 
     def qkv_rope_store(self, x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
                        page_size):
@@ -491,7 +523,18 @@ class HipOps:
         fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
                  and weight.tiled is not None and weight.shape == (N, K))
         if not fused:
-            qkv = self.linear(x, weight, bias)
+            if (self.act_dtype == torch.bfloat16 and self.WIDE_MIN_M <= M <= self.SKINNY_MAX_M
+                    and weight.tiled is not None and K % 32 == 0 and not isinstance(x, ScaledRows)):
+                # K split over workgroups; the rotation kernel adds the partial sums up
+                product = self.linear_mid(x, weight, bias, partial=True)
+                if isinstance(product, PartialSums):
+                    qkv = self._new((M, N))
+                    self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                                    True, split=product)
+                    return qkv
+                qkv = product
+            else:
+                qkv = self.linear(x, weight, bias)
             self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True)
             return qkv
         scaled = x if isinstance(x, ScaledRows) else None

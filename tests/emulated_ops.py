@@ -85,8 +85,8 @@ class EmulatedOps:
         k = qkv[:, nh * D:(nh + nkv) * D].view(T, nkv, D)
         v = qkv[:, (nh + nkv) * D:].view(T, nkv, D)
         page, off = (slots // page_size).long(), (slots % page_size).long()
-        k_cache[page, :, off, :] = k
-        v_cache[page, :, :, off] = v
+        k_cache[page, :, off, :] = k.to(k_cache.dtype)
+        v_cache[page, :, :, off] = v.to(v_cache.dtype)
 
     def qkv_rope_store(self, x, w, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size):
         qkv = self.linear(x, w, bias)

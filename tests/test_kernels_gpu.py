@@ -299,6 +299,36 @@ def test_rope_store(both, nh, nkv, D, page, pairs8, T):
     assert torch.equal(kc[0], k_before)
 
 
+@pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (28, 4, 128, 16), (5, 1, 48, 32)])
+def test_rope_store_from_partial_sums(both, nh, nkv, D, page):
+    """The q/k/v product arrives as float partial sums of a split K plus a bias:
+    rotation and cache write see their sum; q lands in the buffer."""
+    from servelab_amd.kernels.ops import PartialSums
+    ops, emu, dt = both
+    T, pages, N = 40, 9, (nh + 2 * nkv) * D
+    parts = randn(3, T, N, seed=1)
+    bias = randn(N, seed=2)
+    inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
+    cos, sin = emu.rope_tables(torch.arange(50, 50 + T, dtype=torch.int32).cuda(), inv)
+    slots = torch.randperm(pages * page)[:T].to(torch.int32).cuda()
+    kc = [randn(pages, nkv, page, D, dtype=dt, seed=7) for _ in range(2)]
+    vc = [randn(pages, nkv, D, page, dtype=dt, seed=8) for _ in range(2)]
+    for b in (bias, None):
+        for c, s_ in ((cos, sin), (None, None)):
+            full = parts.sum(0) + (b if b is not None else 0)
+            q1 = torch.zeros(T, N, dtype=dt, device="cuda")
+            ops.rope_store(q1, nh, nkv, D, c, s_, slots, kc[0], vc[0], page, D % 16 == 0,
+                           split=PartialSums(parts, b))
+            q2 = full.clone()                                    # the reference rotates in float32
+            EmulatedOps(torch.float32).rope_store(q2, nh, nkv, D, c, s_, slots, kc[1], vc[1], page,
+                                                  D % 16 == 0)
+            assert rel_err(q1[:, :nh * D], q2[:, :nh * D]) < ELEM_TOL[dt] * 2
+            assert rel_err(kc[0], kc[1]) < ELEM_TOL[dt] * 2
+            assert rel_err(vc[0], vc[1]) < ELEM_TOL[dt] * 2
+    if dt == torch.bfloat16:
+        assert rel_err(ops.materialize(PartialSums(parts, bias)), parts.sum(0) + bias) < ELEM_TOL[dt] * 2
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 40])
 @pytest.mark.parametrize("nh,nkv,D,page,H", [(4, 2, 16, 16, 64), (28, 4, 128, 16, 256), (5, 1, 48, 32, 96)])
 def test_qkv_rope_store(M, nh, nkv, D, page, H):
