@@ -385,7 +385,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
 // wt: W in the tiled layout, ceil(N / 16) * 16 rows (rows beyond N are zero).
 // At most 16 rows.  Fusion: in_parts != nullptr makes x un-normalised rows
 // (consumer), resid != nullptr makes the result a delta of the stream (producer).
-// pair_tiles: two tiles of W per workgroup (not for producers or q/k/v with rotary).
+// pair_tiles: two tiles of W per workgroup.
 extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float* bias, void* y,
                                       int M, int N, int K, int out_f32, int gated,
                                       const float* in_parts, int in_nparts, float eps,
@@ -421,15 +421,23 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
     SL_CHECK((R.cosv == nullptr) == (R.sinv == nullptr), "gemm_skinny: cos and sin go together");
     SL_CHECK(R.slots == nullptr || (R.kc != nullptr && R.vc != nullptr && R.page > 0),
              "gemm_skinny: cache rows need the pages");
-    if (!consumer) gemm_skinny_kernel<false, false, false, 1, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
-    else if (few) gemm_skinny_kernel<false, true, false, 8, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
-    else gemm_skinny_kernel<false, true, false, 16, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+    const dim3 grid2(((N + 15) / 16 + 1) / 2);
+    if (pair_tiles) {
+      if (!consumer) gemm_skinny_kernel<false, false, false, 1, true, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+      else if (few) gemm_skinny_kernel<false, true, false, 8, true, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+      else gemm_skinny_kernel<false, true, false, 16, true, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+    } else {
+      if (!consumer) gemm_skinny_kernel<false, false, false, 1, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+      else if (few) gemm_skinny_kernel<false, true, false, 8, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+      else gemm_skinny_kernel<false, true, false, 16, true><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, R);
+    }
     return sl_launch_status();
   }
   const RopeStore none{};
-  if (pair_tiles && !producer) {                 // two tiles per workgroup (the large matrices: gate/up, head)
+  if (pair_tiles) {                              // two tiles per workgroup
     const dim3 grid2(((N + 15) / 16 + 1) / 2);
-    if (consumer && gated && few) gemm_skinny_kernel<true, true, false, 8, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
+    if (producer) gemm_skinny_kernel<false, false, true, 1, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
+    else if (consumer && gated && few) gemm_skinny_kernel<true, true, false, 8, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
     else if (consumer && gated) gemm_skinny_kernel<true, true, false, 16, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
     else if (consumer && few) gemm_skinny_kernel<false, true, false, 8, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F, none);
     else if (consumer) gemm_skinny_kernel<false, true, false, 16, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F, none);

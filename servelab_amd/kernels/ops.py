@@ -92,8 +92,6 @@ class ScaledRows:
 
 class HipOps:
     ROWS_KERNEL_MAX_M = 16        # the wavefront-per-column GEMM is used up to this many rows
-    PAIR_TILES_MIN = 1024         # few-rows products with this many 16-row tiles of W take two per workgroup ...
-    PAIR_TILES_MIN_ROWS = 4       # ... from this many rows of x on (below, x is too small to matter)
     SKINNY_MAX_M = 64             # the matrix-core few-rows GEMM takes up to this many rows
 
     # Decode reads every weight once per step and is bound by how fast it
@@ -123,6 +121,7 @@ class HipOps:
         self._fn = {}
         self._bias_cache = {}
         self.use_mfma_attention = True
+        self._num_cus = max(1, torch.cuda.get_device_properties(self.device).multi_processor_count)
         self.fuse_norms = act_dtype == torch.bfloat16
         self.fuse_rope = act_dtype == torch.bfloat16
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
@@ -152,6 +151,20 @@ class HipOps:
     def _new(self, shape, dtype=None):
         return torch.empty(shape, dtype=dtype or self.act_dtype, device=self.device)
 
+    def _pair_tiles(self, M, N, K) -> bool:
+        """Whether a few-rows product gives its workgroups two tiles of W (16
+        rows each) instead of one.  These kernels are bound by what the busiest
+        CU has to pull through its L1 (about 37 GB/s a CU on MI355X, whatever
+        hits L2), W and x alike: the cost of a choice is the number of
+        workgroups the busiest CU gets times the bytes of one.  Two tiles share
+        one pass over x, which wins when x is not small against W and when one
+        tile each would give some CUs two workgroups and the rest one."""
+        tiles = -(-N // 16)
+        w, x = 16 * K, min(M, 16) * K                     # bytes / 2 of a tile of W and of x
+        one = -(-tiles // self._num_cus) * (w + x)
+        two = -(-(-(-tiles // 2)) // self._num_cus) * (2 * w + x)
+        return tiles >= 2 and two < 0.97 * one
+
     def _skinny(self, x, weight, bias, y, M, N, K, out_f32=False, gated=False, scaled=None,
                 resid=None, next_gain=None, out_parts=None, rope=None):
         """One call of the few-rows kernel (at most 16 rows) in any of its forms."""
@@ -161,7 +174,7 @@ class HipOps:
                    _c_float(scaled.eps if scaled is not None else 0.0),
                    _p(scaled.rows) if scaled is not None else None, _p(resid), _p(next_gain),
                    _p(out_parts), ctypes.byref(rope) if rope is not None else None,
-                   int(M >= self.PAIR_TILES_MIN_ROWS and -(-N // 16) >= self.PAIR_TILES_MIN))
+                   int(self._pair_tiles(M, N, K)))
 
     # ------------------------------------------------------------ embedding
     def embed(self, ids, table):
