@@ -165,6 +165,7 @@ extern "C" const char* sl_gemm_tiled(const void* x, const void* w, const float* 
 // M repeat the last row and are not stored).
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
 //
 // GATED: the 16 rows of a tile are 8 gate rows followed by the 8 up rows of the
@@ -640,15 +641,24 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
   __shared__ bf16x8 xs[2][KC][MB][64];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
   const int ntiles = (N + 15) / 16;
-  const int tile0 = (blockIdx.x * WAVES + wave) * NT;
+  // The workgroups share the tiles as evenly as the grid allows: workgroup g of
+  // G takes tiles [ntiles g / G, ntiles (g + 1) / G), at most WAVES * NT of
+  // them; wavefront v takes the v-th and the (WAVES + v)-th.  A wavefront
+  // without a (second) tile loads its first one again, which hits L1 and costs
+  // no bandwidth, and drops the result.
+  const int tbeg = (int)((long long)ntiles * blockIdx.x / gridDim.x);
+  const int tcount = (int)((long long)ntiles * (blockIdx.x + 1) / gridDim.x) - tbeg;
+  int tile_of[NT];
+  bool live[NT];
   const int KT = K / 32;
   const int kbeg = (int)((long long)KT * blockIdx.y / KS), kend = (int)((long long)KT * (blockIdx.y + 1) / KS);
   const int nchunks = (kend - kbeg + KC - 1) / KC;
   const __bf16* wp[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int tile = tile0 + t < ntiles ? tile0 + t : ntiles - 1;
-    wp[t] = wt + ((size_t)tile * KT * 64 + lane) * 8;
+    live[t] = WAVES * t + wave < tcount;
+    tile_of[t] = live[t] ? tbeg + WAVES * t + wave : (t > 0 && live[0] ? tile_of[0] : tbeg);
+    wp[t] = wt + ((size_t)tile_of[t] * KT * 64 + lane) * 8;
   }
   // this thread's share of a chunk of x: XF fragments (ks, mb, lane) = (idx / (MB * 64), idx / 64 % MB, idx % 64)
   constexpr int XF = MB * KC * 64 / THREADS;
@@ -756,8 +766,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
   // lane: column m = 16 b + i of x, rows n = 16 tile + 4 gq + r of W
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    if (tile0 + t >= ntiles) continue;
-    const int n = (tile0 + t) * 16 + 4 * gq;
+    if (!live[t]) continue;
+    const int n = tile_of[t] * 16 + 4 * gq;
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
       const int m = 16 * b + i;
@@ -767,7 +777,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) up[r] = __shfl(acc[t][b][r], lane + 32, 64);
         if (gq < 2 && m < M) {
-          __bf16* o = (__bf16*)y + (size_t)m * (N / 2) + (tile0 + t) * 8 + 4 * gq;
+          __bf16* o = (__bf16*)y + (size_t)m * (N / 2) + tile_of[t] * 8 + 4 * gq;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float g = acc[t][b][r];
@@ -777,19 +787,37 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
         continue;
       }
       if (m >= M) continue;
+      // four consecutive columns per lane: one 16-byte (8-byte) store where the row allows it
+      const bool whole = n + 3 < N && N % 4 == 0;
       if (KS > 1) {
         float* o = (float*)y + ((size_t)blockIdx.y * M + m) * N + n;
+        if (whole) {
+          *(f32x4*)o = acc[t][b];
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (n + r < N) o[r] = acc[t][b][r];
+          for (int r = 0; r < 4; ++r)
+            if (n + r < N) o[r] = acc[t][b][r];
+        }
         continue;
       }
+      f32x4 v = acc[t][b];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        if (n + r >= N) continue;
-        const float v = acc[t][b][r] + (bias != nullptr ? bias[n + r] : 0.f);
-        if (out_f32) ((float*)y)[(size_t)m * N + n + r] = v;
-        else ((__bf16*)y)[(size_t)m * N + n + r] = (__bf16)v;
+      for (int r = 0; r < 4; ++r)
+        if (bias != nullptr && n + r < N) v[r] += bias[n + r];
+      if (whole && out_f32) {
+        *(f32x4*)((float*)y + (size_t)m * N + n) = v;
+      } else if (whole) {
+        bf16x4 h;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) h[r] = (__bf16)v[r];
+        *(bf16x4*)((__bf16*)y + (size_t)m * N + n) = h;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (n + r >= N) continue;
+          if (out_f32) ((float*)y)[(size_t)m * N + n + r] = v[r];
+          else ((__bf16*)y)[(size_t)m * N + n + r] = (__bf16)v[r];
+        }
       }
     }
   }
@@ -811,7 +839,7 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, const float
 // for the reader to add (and the bias with them).
 extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* bias, void* y,
                                    int M, int N, int K, int out_f32, int gated, int ks,
-                                   int wide_min_wgs, float* part, hipStream_t stream) {
+                                   int wide_min_wgs, int num_cus, float* part, hipStream_t stream) {
   SL_CHECK(M > 0 && N > 0 && K > 0, "gemm_mid: sizes must be positive");
   SL_CHECK(M <= 64, "gemm_mid: at most 64 rows");
   SL_CHECK(K % 32 == 0, "gemm_mid: K must be a multiple of 32");
@@ -827,9 +855,16 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
   const __bf16* ww = (const __bf16*)wt;
   void* dst = ks > 1 ? (void*)part : y;
   // chunks of four k-steps, two tiles per wavefront; 8 wavefronts (16 tiles
-  // share one pass over x) when that still leaves wide_min_wgs workgroups
-  const bool wide = ((ntiles + 15) / 16) * ks >= wide_min_wgs;
-  const dim3 grid(wide ? (ntiles + 15) / 16 : (ntiles + 7) / 8, ks);
+  // share one pass over x) when that still leaves wide_min_wgs workgroups.
+  // An unsplit product that would keep more than half the CUs busy that way is
+  // spread over a whole multiple of the CUs instead, fewer tiles each: the time
+  // of these products is what the busiest CU has to pull through its L1.
+  const int wide_min = ks > 1 && 4 * num_cus / 5 > wide_min_wgs ? 4 * num_cus / 5 : wide_min_wgs;   // a split must keep most CUs busy
+  const bool wide = ((ntiles + 15) / 16) * ks >= wide_min;
+  int groups = wide ? (ntiles + 15) / 16 : (ntiles + 7) / 8;
+  if (ks == 1 && wide && num_cus > 0 && 2 * groups > num_cus)
+    groups = num_cus * ((groups + num_cus - 1) / num_cus);
+  const dim3 grid(groups, ks);
   if (wide) {
     if (M <= 32) gemm_mid_kernel<2, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
     else gemm_mid_kernel<4, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);

@@ -336,10 +336,14 @@ class HipOps:
                    int(out_f32), int(gated))
         return y
 
-    MID_TARGET_WORKGROUPS = 448
+    MID_TARGET_WORKGROUPS = 224    # K is split until about this many workgroups stream W (fewer splits, fewer partial sums)
     MID_PARTIAL_WORKGROUPS = 128   # fewer splits when the reader adds the partial sums (their bytes count twice)
     MID_WIDE_WORKGROUPS = 128      # workgroups of 8 wavefronts (16 tiles of W per pass over x) if this many remain
-    MID_MIN_ELEMENTS = 48 << 20   # matrices from this size on take the LDS-staged kernel at 17..64 rows
+    MID_MIN_ELEMENTS = 48 << 20   # matrices from this size on take the LDS-staged kernel at 17..32 rows ...
+    MID_MIN_ELEMENTS_MANY = 8 << 20   # ... and from this size on at 33..64 rows (x costs more there)
+
+    def _takes_mid(self, M, N, K) -> bool:
+        return N * K >= (self.MID_MIN_ELEMENTS if M <= 32 else self.MID_MIN_ELEMENTS_MANY)
 
     def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None, partial=False):
         """17..64 rows with x staged through LDS; K split over workgroups when
@@ -356,11 +360,11 @@ class HipOps:
         part = self._new((ks, M, N), torch.float32) if ks > 1 else None
         if partial and ks > 1:
             self._call("gemm", "sl_gemm_mid", _p(x), _p(weight.tiled), None, None, M, N, K,
-                       0, 0, int(ks), self.MID_WIDE_WORKGROUPS, _p(part))
+                       0, 0, int(ks), self.MID_WIDE_WORKGROUPS, self._num_cus, _p(part))
             return PartialSums(part, bias)
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_mid", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
-                   int(out_f32), int(gated), int(ks), self.MID_WIDE_WORKGROUPS, _p(part))
+                   int(out_f32), int(gated), int(ks), self.MID_WIDE_WORKGROUPS, self._num_cus, _p(part))
         return y
 
     def linear_skinny(self, x, weight, bias, out_f32=False):
@@ -369,7 +373,7 @@ class HipOps:
         if weight.tiled is None:
             raise KernelError("linear_skinny needs the tiled copy of the weight")
         if M >= self.WIDE_MIN_M:
-            if N * K >= self.MID_MIN_ELEMENTS:
+            if self._takes_mid(M, N, K):
                 return self.linear_mid(x, weight, bias, out_f32)
             return self.linear_wide(x, weight, bias, out_f32)
         y = self._new((M, N), torch.float32 if out_f32 else None)
@@ -407,7 +411,7 @@ class HipOps:
                 and N % 16 == 0):
             self._check(x, self.act_dtype, None, "x")
             if M >= self.WIDE_MIN_M:
-                if N * K >= self.MID_MIN_ELEMENTS:
+                if self._takes_mid(M, N, K):
                     return self.linear_mid(x, weight, None, gated=True)
                 return self.linear_wide(x, weight, None, gated=True)
             y = self._new((M, N // 2))
