@@ -66,8 +66,8 @@ class Deferred:
 class PartialSums:
     """A product whose K was split over workgroups, left as float partial sums
     ``parts`` [ks, T, N] with the bias not yet added, for a reader that adds
-    them up on its way (``rope_store``); ``HipOps.materialize`` makes the plain
-    tensor."""
+    them up on its way (``rope_store``, ``add_rmsnorm``); ``HipOps.materialize``
+    makes the plain tensor."""
     __slots__ = ("parts", "bias")
 
     def __init__(self, parts, bias):
@@ -198,12 +198,22 @@ class HipOps:
             if fuse:
                 return self._produce_scaled_rows(resid, delta, weight, eps)
             delta = self.materialize(delta)
+        out = self._new((T, H))
+        self._call("norm", "sl_add_rmsnorm", _p(resid), *self._delta_args(delta, T, H), None,
+                   _p(weight), _p(out), T, H, _c_float(eps))
+        return out
+
+    def _delta_args(self, delta, T, H):
+        """(delta, parts, nparts, T, bias) of the norm kernels for any kind of delta."""
+        if isinstance(delta, PartialSums):
+            ks = delta.parts.shape[0]
+            self._check(delta.parts, torch.float32, (ks, T, H), "partial sums")
+            if delta.bias is not None:
+                self._check(delta.bias, torch.float32, (H,), "bias")
+            return None, _p(delta.parts), ks, T, _p(delta.bias)
         if delta is not None:
             self._check(delta, self.act_dtype, (T, H), "delta")
-        out = self._new((T, H))
-        self._call("norm", "sl_add_rmsnorm", _p(resid), _p(delta), None, _p(weight), _p(out),
-                   T, H, _c_float(eps))
-        return out
+        return _p(delta), None, 0, T, None
 
     def rows_add_rmsnorm(self, resid, delta, rows, weight, eps, fuse=False):
         """The normed rows ``rows`` of resid + delta.  The stream is left as it
@@ -219,11 +229,9 @@ class HipOps:
                 scaled.rows = rows
                 return scaled
             delta = self.materialize(delta)
-        if delta is not None:
-            self._check(delta, self.act_dtype, (T, H), "delta")
         out = self._new((R, H))
-        self._call("norm", "sl_add_rmsnorm", _p(resid), _p(delta), _p(rows), _p(weight), _p(out),
-                   R, H, _c_float(eps))
+        self._call("norm", "sl_add_rmsnorm", _p(resid), *self._delta_args(delta, T, H), _p(rows),
+                   _p(weight), _p(out), R, H, _c_float(eps))
         return out
 
     def materialize(self, value):
@@ -313,6 +321,11 @@ class HipOps:
             if K % 4 == 0 and M <= self.ROWS_KERNEL_MAX_M:
                 return self.linear_rows(x, weight.w, bias, out_f32)
             return self.linear_tiled(x, weight.w, bias, out_f32)
+        if (defer and self.fuse_norms and not out_f32 and self.WIDE_MIN_M <= M <= self.SKINNY_MAX_M
+                and weight.tiled is not None and K % 32 == 0 and N % 4 == 0
+                and self._takes_mid(M, N, K)):
+            return self.linear_mid(x, weight, bias, partial=True,     # the norm adds the partial sums
+                                   target=self.MID_DEFERRED_WORKGROUPS)
         if M <= self.SKINNY_MAX_M and weight.tiled is not None:
             return self.linear_skinny(x, weight, bias, out_f32)
         w = self.rows_of(weight)
@@ -337,6 +350,7 @@ class HipOps:
         return y
 
     MID_TARGET_WORKGROUPS = 224    # K is split until about this many workgroups stream W (fewer splits, fewer partial sums)
+    MID_DEFERRED_WORKGROUPS = 224  # the same when the next norm adds the partial sums of a residual delta
     MID_PARTIAL_WORKGROUPS = 128   # fewer splits when the reader adds the partial sums (their bytes count twice)
     MID_WIDE_WORKGROUPS = 128      # workgroups of 8 wavefronts (16 tiles of W per pass over x) if this many remain
     MID_MIN_ELEMENTS = 48 << 20   # matrices from this size on take the LDS-staged kernel at 17..32 rows ...
@@ -345,7 +359,8 @@ class HipOps:
     def _takes_mid(self, M, N, K) -> bool:
         return N * K >= (self.MID_MIN_ELEMENTS if M <= 32 else self.MID_MIN_ELEMENTS_MANY)
 
-    def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None, partial=False):
+    def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None, partial=False,
+                   target=None):
         """17..64 rows with x staged through LDS; K split over workgroups when
         N alone gives too few of them.  ``partial``: a split product comes back
         as ``PartialSums`` for its reader to add up."""
@@ -355,7 +370,8 @@ class HipOps:
             raise KernelError("linear_mid needs the tiled copy of the weight")
         wgs = -(-(-(-N // 16)) // 8)
         if ks is None:
-            target = self.MID_PARTIAL_WORKGROUPS if partial else self.MID_TARGET_WORKGROUPS
+            if target is None:
+                target = self.MID_PARTIAL_WORKGROUPS if partial else self.MID_TARGET_WORKGROUPS
             ks = 1 if gated else max(1, min(16, K // 32 // 4, -(-target // wgs)))
         part = self._new((ks, M, N), torch.float32) if ks > 1 else None
         if partial and ks > 1:

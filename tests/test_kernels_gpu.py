@@ -72,6 +72,55 @@ def test_rows_add_rmsnorm(both):
     assert rel_err(got, emu.rows_add_rmsnorm(resid, None, rows, w, 1e-6)) < ELEM_TOL[dt] * 2
 
 
+@pytest.mark.parametrize("T,H,ks,bias", [(20, 200, 3, True), (64, 3584, 8, False), (33, 1000, 1, True),
+                                         (17, 130, 5, False)])
+def test_norm_adds_partial_sums(both, T, H, ks, bias):
+    """A delta given as the float partial sums of a split product (and a bias):
+    the norm adds them up itself, over all rows and over chosen rows."""
+    from servelab_amd.kernels.ops import PartialSums
+    ops, emu, dt = both
+    resid = randn(T, H, seed=1)
+    parts = randn(ks, T, H, seed=2)
+    b = randn(H, seed=4) if bias else None
+    w = 1 + 0.1 * randn(H, seed=3)
+    delta = parts.sum(0) + (b if bias else 0)
+    r1, r2 = resid.clone(), resid.clone()
+    got = ops.add_rmsnorm(r1, PartialSums(parts, b), w, 1e-5)
+    r2 += delta
+    want = (r2 * torch.rsqrt(r2.pow(2).mean(-1, keepdim=True) + 1e-5) * w).to(dt)
+    assert (r1 - r2).abs().max().item() < 1e-5
+    assert rel_err(got, want) < ELEM_TOL[dt] * 2
+    rows = torch.tensor([T - 1, 0, 7, 7], dtype=torch.int32).cuda()
+    before = resid.clone()
+    got = ops.rows_add_rmsnorm(resid, PartialSums(parts, b), rows, w, 1e-5)
+    assert torch.equal(resid, before)
+    assert rel_err(got, want[rows.long()]) < ELEM_TOL[dt] * 2
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 3584, 3584), (64, 3584, 18944), (40, 132, 352), (33, 1000, 64)])
+def test_deferred_product_of_many_rows(M, N, K):
+    """``linear(..., defer=True)`` at 17 to 64 rows: whatever comes back (partial
+    sums of a split K, or the plain product), the norm that takes it as its
+    delta must see x W^T + bias."""
+    from servelab_amd.kernels import HipOps
+    dt = torch.bfloat16
+    ops = HipOps(dt, "cuda:0")
+    x, w, b = randn(M, K, dtype=dt, seed=1), (0.05 * randn(N, K, seed=2)).to(dt), randn(N, seed=3)
+    weight = ops.prepare_weight(w)
+    gain = 1 + 0.1 * randn(N, seed=4)
+    resid = randn(M, N, seed=5)
+    for bias in (None, b):
+        delta = ops.linear(x, weight, bias, defer=True)
+        r1 = resid.clone()
+        got = ops.add_rmsnorm(r1, delta, gain, 1e-6)
+        r2 = resid + x.float() @ w.float().T + (bias if bias is not None else 0)
+        want = r2 * torch.rsqrt(r2.pow(2).mean(-1, keepdim=True) + 1e-6) * gain
+        assert rel_err(r1, r2) < 2 ** -7
+        assert rel_err(got, want) < 2 ** -6
+        plain = ops.materialize(delta)
+        assert rel_err(plain, x.float() @ w.float().T + (bias if bias is not None else 0)) < 2 ** -6
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1000, 64), (3, 130, 200), (8, 512, 3584), (16, 96, 352),
                                    (17, 200, 136), (70, 1000, 128), (130, 352, 64)])
 @pytest.mark.parametrize("bias", [False, True])
