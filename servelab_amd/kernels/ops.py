@@ -300,7 +300,14 @@ class HipOps:
     def linear(self, x, weight, bias, out_f32=False, defer=False):
         """y = x W^T (+ bias); ``weight`` is a LinearWeight or a plain [N, K] tensor.
         ``defer``: y will only be added to the residual stream, so the product
-        may be left to the norm that adds it (a ``Deferred`` comes back then)."""
+        may be left to the norm that adds it: up to 16 rows a ``Deferred`` comes
+        back (the norm's kernel runs the product), at 17..64 rows ``PartialSums``
+        of a product whose K was split (the norm adds them up).
+
+        bfloat16, by rows of x: 1..16 the few-rows kernel over the tiled weight,
+        17..64 the wide or the LDS-staged kernel (by the size of W), more the
+        library.  float32: the wavefront-per-column kernel up to 16 rows, the
+        tiled FMA kernel above; never a library product."""
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
         if isinstance(x, ScaledRows):
