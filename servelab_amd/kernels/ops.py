@@ -620,7 +620,7 @@ class HipOps:
                    int(window or 0), _p(out))
         return out
 
-    TARGET_WAVES = 1024           # wavefronts a decode launch aims for when it splits the context
+    TARGET_WAVES = 512            # wavefronts a decode launch aims for when it splits the context
     SHARED_ATTENTION_WAVES = 2048  # prompt launches of this many 32-column wavefronts share keys through LDS
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
