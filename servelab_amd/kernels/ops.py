@@ -655,7 +655,10 @@ class HipOps:
         return out
 
     TARGET_WAVES = 512            # wavefronts a decode launch aims for when it splits the context
-    SHARED_ATTENTION_WAVES = 2048  # prompt launches of this many 32-column wavefronts share keys through LDS
+    # Prompt launches share keys through LDS when they have at least MIN_WAVES 32-column wavefronts (enough
+    # workgroups of four) and WAVES of them counted once per 2,048 tokens of context (what each pulls from L2).
+    SHARED_ATTENTION_WAVES = 2048
+    SHARED_ATTENTION_MIN_WAVES = 1024
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples
@@ -693,8 +696,11 @@ class HipOps:
             fn.restype = ctypes.c_char_p
             self._fn[name] = fn
         if n_pre:
+            waves = -(-batch.max_q_len * (nh // nkv) // 32) * nkv * n_pre
+            shared = (waves >= self.SHARED_ATTENTION_MIN_WAVES and
+                      waves * max(1, batch.max_ctx_len // 2048) >= self.SHARED_ATTENTION_WAVES)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, 1,
-                       self.SHARED_ATTENTION_WAVES, _p(out), None, None, 0, 0)
+                       0 if shared else 1 << 30, _p(out), None, None, 0, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
