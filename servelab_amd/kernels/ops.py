@@ -512,7 +512,10 @@ class HipOps:
         later process reads instead of timing again.  The library's pick for
         the 7B shape's prompt products measured 26 % slower than the tuned one
         on MI355X."""
-        tunable = torch.cuda.tunable
+        tunable = getattr(torch.cuda, "tunable", None)
+        if tunable is None:                      # a PyTorch without TunableOp: the library's defaults stay
+            yield
+            return
         if results_file is None:
             results_file = os.path.join(tempfile.gettempdir(),
                                         f"servelab_amd_tunableop_{os.getuid()}.csv")
