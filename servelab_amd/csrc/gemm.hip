@@ -2,9 +2,9 @@
 // (checkpoint layout, servelab/parallel/layers.py:164-180).  Accumulation is
 // float with plain FMA in both builds; the float build is the true 32-bit path.
 //
-//   sl_gemm_rows  few rows (decode): one wavefront per output column streams
-//                 one row of W with 16-byte loads; bound by reading W once
-//                 per group of SL_ROWS rows of x.
+//   sl_gemm_rows  few rows (decode): a wavefront streams the rows of W of one
+//                 or four output columns with 16-byte loads against up to 8
+//                 rows of x at a time.
 //   sl_gemm_tiled any M: 64x64 LDS tiles, 4x4 outputs per thread.
 #include "common.h"
 
@@ -17,41 +17,57 @@
 struct __attribute__((aligned(16))) vec_t { act_t v[SL_VEC]; };
 
 // ------------------------------------------------------------------ few rows
-template <int MB>
+// A wavefront owns NC consecutive output columns: every 16-byte piece of x it
+// loads meets NC rows of W, so x is read once per NC columns instead of once
+// per column (with 8 rows of x that was 8 times the bytes of W itself).
+template <int MB, int NC>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(
     const act_t* __restrict__ x, const act_t* __restrict__ w, const float* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int out_f32) {
   const int lane = threadIdx.x % SL_WAVE;
-  const int n = blockIdx.x * (blockDim.x / SL_WAVE) + threadIdx.x / SL_WAVE;
-  if (n >= N) return;
-  const act_t* wr = w + (size_t)n * K;
+  const int n0 = (blockIdx.x * (blockDim.x / SL_WAVE) + threadIdx.x / SL_WAVE) * NC;
+  if (n0 >= N) return;
+  const act_t* wr[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) wr[c] = w + (size_t)(n0 + c < N ? n0 + c : N - 1) * K;
   for (int m0 = 0; m0 < M; m0 += MB) {
-    float acc[MB];
+    float acc[MB][NC];
 #pragma unroll
-    for (int i = 0; i < MB; ++i) acc[i] = 0.f;
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) acc[i][c] = 0.f;
     for (int k = lane * SL_VEC; k < K; k += SL_WAVE * SL_VEC) {
-      const vec_t wv = *(const vec_t*)(wr + k);
-      float wf[SL_VEC];
+      float wf[NC][SL_VEC];
 #pragma unroll
-      for (int j = 0; j < SL_VEC; ++j) wf[j] = to_f(wv.v[j]);
+      for (int c = 0; c < NC; ++c) {
+        const vec_t wv = *(const vec_t*)(wr[c] + k);
+#pragma unroll
+        for (int j = 0; j < SL_VEC; ++j) wf[c][j] = to_f(wv.v[j]);
+      }
 #pragma unroll
       for (int i = 0; i < MB; ++i) {
         if (m0 + i < M) {
           const vec_t xv = *(const vec_t*)(x + (size_t)(m0 + i) * K + k);
 #pragma unroll
-          for (int j = 0; j < SL_VEC; ++j) acc[i] += wf[j] * to_f(xv.v[j]);
+          for (int j = 0; j < SL_VEC; ++j) {
+            const float xf = to_f(xv.v[j]);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) acc[i][c] += wf[c][j] * xf;
+          }
         }
       }
     }
 #pragma unroll
-    for (int i = 0; i < MB; ++i) {
-      const float s = wave_sum(acc[i]);
-      if (lane == 0 && m0 + i < M) {
-        const float r = s + (bias != nullptr ? bias[n] : 0.f);
-        if (out_f32) ((float*)y)[(size_t)(m0 + i) * N + n] = r;
-        else ((act_t*)y)[(size_t)(m0 + i) * N + n] = from_f<act_t>(r);
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const float s = wave_sum(acc[i][c]);
+        if (lane == 0 && m0 + i < M && n0 + c < N) {
+          const float r = s + (bias != nullptr ? bias[n0 + c] : 0.f);
+          if (out_f32) ((float*)y)[(size_t)(m0 + i) * N + n0 + c] = r;
+          else ((act_t*)y)[(size_t)(m0 + i) * N + n0 + c] = from_f<act_t>(r);
+        }
       }
-    }
   }
 }
 
@@ -63,19 +79,18 @@ extern "C" const char* sl_gemm_rows(const void* x, const void* w, const float* b
            "gemm_rows: x and W must be 16-byte aligned");
   if (M == 0) return nullptr;
   const int waves = 4;
-  const dim3 grid((N + waves - 1) / waves);
-  if (M == 1)
-    gemm_rows_kernel<1><<<grid, waves * SL_WAVE, 0, stream>>>(
-        (const act_t*)x, (const act_t*)w, bias, y, M, N, K, out_f32);
-  else if (M == 2)
-    gemm_rows_kernel<2><<<grid, waves * SL_WAVE, 0, stream>>>(
-        (const act_t*)x, (const act_t*)w, bias, y, M, N, K, out_f32);
-  else if (M <= 4)
-    gemm_rows_kernel<4><<<grid, waves * SL_WAVE, 0, stream>>>(
-        (const act_t*)x, (const act_t*)w, bias, y, M, N, K, out_f32);
-  else
-    gemm_rows_kernel<8><<<grid, waves * SL_WAVE, 0, stream>>>(
-        (const act_t*)x, (const act_t*)w, bias, y, M, N, K, out_f32);
+  const act_t* xx = (const act_t*)x;
+  const act_t* ww = (const act_t*)w;
+  // one row of x: a column per wavefront keeps the most wavefronts in flight;
+  // more rows: 4 columns per wavefront share each load of x
+  if (M == 1) {
+    gemm_rows_kernel<1, 1><<<(N + waves - 1) / waves, waves * SL_WAVE, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+    return sl_launch_status();
+  }
+  const dim3 grid((N + 4 * waves - 1) / (4 * waves));
+  if (M == 2) gemm_rows_kernel<2, 4><<<grid, waves * SL_WAVE, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+  else if (M <= 4) gemm_rows_kernel<4, 4><<<grid, waves * SL_WAVE, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+  else gemm_rows_kernel<8, 4><<<grid, waves * SL_WAVE, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
   return sl_launch_status();
 }
 
