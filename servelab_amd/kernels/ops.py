@@ -651,12 +651,21 @@ class HipOps:
             self._attention_mfma(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
                                  batch, scale, window, out)
             return out
+        # few tokens (a decode step): the keys of every (token, head) are shared out over several
+        # wavefronts; the count depends on the number of tokens only, so that a captured step and an
+        # eager one add up in the same order
+        nsplit = 1 if batch.max_q_len > 1 else max(1, min(64, self.GENERAL_ATTENTION_WAVES // (T * nh)))
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = self._new((T, nh, nsplit, D), torch.float32)
+            part_ml = self._new((T, nh, nsplit, 2), torch.float32)
         self._call("attention", "sl_attention_general", _p(qkv), (nh + 2 * nkv) * D, _p(k_cache),
                    _p(v_cache), _p(block_tables), max_pages, _p(batch.tok_seq),
                    _p(batch.positions), T, nh, nkv, D, page_size, _c_float(scale),
-                   int(window or 0), _p(out))
+                   int(window or 0), _p(out), nsplit, _p(part_o), _p(part_ml))
         return out
 
+    GENERAL_ATTENTION_WAVES = 4096  # the general kernel's decode launches aim for this many wavefronts
     TARGET_WAVES = 512            # wavefronts a decode launch aims for when it splits the context
     # Prompt launches share keys through LDS when they have at least MIN_WAVES 32-column wavefronts (enough
     # workgroups of four) and WAVES of them counted once per 2,048 tokens of context (what each pulls from L2).

@@ -523,6 +523,25 @@ def test_attention_reference_point_moves_late():
         assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+@pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (7, 7, 48, 32), (5, 5, 80, 16), (28, 4, 128, 16)])
+@pytest.mark.parametrize("window", [None, 50])
+def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window):
+    """Single-token rows only: the general kernel (float32, and bfloat16 head
+    sizes the matrix-core kernels refuse) and the matrix-core kernel both split
+    every row's keys over several wavefronts and merge the shares; contexts of
+    1 token, of less than a share each, and of hundreds."""
+    ops, emu, dt = both
+    seqs = [(1, 1), (5, 1), (64, 1), (65, 1), (333, 1), (700, 1), (129, 1)]
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=9)
+    scale = 1.0 / math.sqrt(D)
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
+    ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                              types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                       for k, v in vars(batch).items()}),
+                              scale, window)
+    assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+
+
 @pytest.mark.parametrize("D,page", [(16, 16), (32, 16), (128, 32)])
 @pytest.mark.parametrize("q_len", [1, 5])
 def test_attention_finds_one_key_at_edges(both, D, page, q_len):
