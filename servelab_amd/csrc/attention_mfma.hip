@@ -329,7 +329,9 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   constexpr int NB = 2, THREADS = 64 * SHARED_WAVES, COLS = 16 * NB * SHARED_WAVES;
   __shared__ __attribute__((aligned(16))) __bf16 k_lds[2][SHARED_FITS ? 32 * KS : 8];
   __shared__ __attribute__((aligned(16))) __bf16 v_lds[2][SHARED_FITS ? D * VS : 8];
-  const int t = threadIdx.x, wave = t >> 6, lane = t & 63, n = lane & 15, gq = lane >> 4;
+  // (wave as a scalar: the products below sit under conditions that depend on it, and matrix
+  // instructions ignore the execution mask)
+  const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63, n = lane & 15, gq = lane >> 4;
   const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
   const int g = P.nh / P.nkv;
   const int q0 = P.cu_q[seq];

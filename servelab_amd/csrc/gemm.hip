@@ -241,7 +241,11 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
   constexpr int WAVES = 8, U = NT == 1 ? 8 : 4;
   __shared__ f32x4 red[NT][WAVES][64];
   __shared__ float wsum[WAVES][16];
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
+  // the wavefront's index as a scalar: what depends on it (its share of K, its tiles) then steers
+  // real branches; matrix instructions ignore the execution mask, so they must not sit under a
+  // condition the compiler takes for divergent and may turn into masking
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
   const int ntiles = (N + 15) / 16;
   const int KT = K / 32;
   const int ks0 = (int)((long long)KT * wave / WAVES), ks1 = (int)((long long)KT * (wave + 1) / WAVES);
@@ -295,13 +299,24 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv, acc[t], 0, 0, 0);
     }
   }
-  for (; ks < ks1; ++ks) {
-    const bf16x8 bv = *(const bf16x8*)(xp + 32 * (size_t)ks);
+  if (ks < ks1) {
+    // the last k-steps, fewer than U: all their loads are issued before the
+    // first product, so they cost one trip to memory, not one each
+    bf16x8 a[NT][U], bv[U];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const bf16x8 a = *(const bf16x8*)(wp[t] + 512 * (size_t)ks);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bv, acc[t], 0, 0, 0);
-    }
+    for (int u = 0; u < U - 1; ++u)
+      if (ks + u < ks1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)(ks + u));
+        bv[u] = *(const bf16x8*)(xp + 32 * (size_t)(ks + u));
+      }
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u)
+      if (ks + u < ks1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv[u], acc[t], 0, 0, 0);
+      }
   }
 #pragma unroll
   for (int t = 0; t < NT; ++t) red[t][wave][lane] = acc[t];
@@ -485,7 +500,11 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(
     void* __restrict__ y, int M, int N, int K, int out_f32) {
   constexpr int WAVES = 8, U = 2, NT = 2;
   __shared__ f32x4 red[WAVES][MB][64];
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
+  // the wavefront's index as a scalar: what depends on it (its share of K, its tiles) then steers
+  // real branches; matrix instructions ignore the execution mask, so they must not sit under a
+  // condition the compiler takes for divergent and may turn into masking
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
   const int ntiles = (N + 15) / 16;
   const int tile0 = blockIdx.x * NT;
   const int KT = K / 32;
@@ -654,7 +673,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
     void* __restrict__ y, int M, int N, int K, int out_f32, int gated, int KS) {
   constexpr int THREADS = 64 * WAVES;
   __shared__ bf16x8 xs[2][KC][MB][64];
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
+  // the wavefront's index as a scalar: what depends on it (its share of K, its tiles) then steers
+  // real branches; matrix instructions ignore the execution mask, so they must not sit under a
+  // condition the compiler takes for divergent and may turn into masking
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
   const int ntiles = (N + 15) / 16;
   // The workgroups share the tiles as evenly as the grid allows: workgroup g of
   // G takes tiles [ntiles g / G, ntiles (g + 1) / G), at most WAVES * NT of

@@ -45,14 +45,12 @@ class _RopeStore(ctypes.Structure):
 class LinearWeight:
     """A weight matrix [N, K] as the products read it: row-major (``w``) for
     products with many rows, tiled (``tiled``, bfloat16 only) for the few-rows
-    kernels that decode steps use.  Both, or one of them.  ``pairing`` keeps
-    what ``HipOps`` measured for this matrix (see ``_pair_tiles``)."""
-    __slots__ = ("w", "tiled", "shape", "pairing")
+    kernels that decode steps use.  Both, or one of them."""
+    __slots__ = ("w", "tiled", "shape")
 
     def __init__(self, w, tiled=None, shape=None):
         self.w, self.tiled = w, tiled
         self.shape = tuple(w.shape) if w is not None else tuple(shape)
-        self.pairing = {}
 
 
 class Deferred:
@@ -123,7 +121,6 @@ class HipOps:
         self._fn = {}
         self._bias_cache = {}
         self.use_mfma_attention = True
-        self.measure_pairing = True
         self._num_cus = max(1, torch.cuda.get_device_properties(self.device).multi_processor_count)
         self.fuse_norms = act_dtype == torch.bfloat16
         self.fuse_rope = act_dtype == torch.bfloat16
@@ -154,50 +151,23 @@ class HipOps:
     def _new(self, shape, dtype=None):
         return torch.empty(shape, dtype=dtype or self.act_dtype, device=self.device)
 
-    def _pair_tiles(self, M, N, K, weight=None) -> bool:
+    def _pair_tiles(self, M, N, K) -> bool:
         """Whether a few-rows product gives its workgroups two tiles of W (16
-        rows each) instead of one.  Two tiles share one pass over x, and these
+        rows each) instead of one.  Two tiles share one pass over x; these
         kernels are bound by what the busiest CU has to pull through its L1
         (about 37 GB/s a CU on MI355X, W and the re-read x alike) unless HBM
-        is slower still; but how well one tile each already shares x between
-        the workgroups of a CU, and how the two streams of a pair fall on the
-        memory channels, depends on the matrix (7B and 32B shapes gain 3-25 %
-        from pairs at 8-16 rows, K = 8192 loses 5-20 % below 16 rows).  So the
-        choice is measured once per matrix and row bucket, outside graph
-        capture; both forms sum in the same order and give identical bits.
-        Without a matrix to measure, a byte count per busiest CU decides."""
+        is slower still, so the choice goes by the workgroups the busiest CU
+        gets times the bytes of one.  Up to 8 rows x is small enough that the
+        two forms measured within a few per cent of each other on the 7B, 32B
+        and 72B shapes (pairs lose 7 % where K = 8192), so one tile stays; at 16
+        rows pairs gain 15-25 % on the large matrices."""
         tiles = -(-N // 16)
-        if tiles < 2 or M <= 4:                            # x of up to 4 rows is too small to matter
+        if tiles < 2 or M <= 8:
             return False
-        bucket = 8 if M <= 8 else 16
-        if weight is not None and self.measure_pairing:
-            got = weight.pairing.get(bucket)
-            if got is None and not torch.cuda.is_current_stream_capturing():
-                got = weight.pairing[bucket] = self._measure_pairing(weight, bucket, N, K)
-            if got is not None:
-                return got
         w, x = 16 * K, min(M, 16) * K                     # bytes / 2 of a tile of W and of x
         one = -(-tiles // self._num_cus) * (w + x)
         two = -(-(-(-tiles // 2)) // self._num_cus) * (2 * w + x)
         return two < 0.97 * one
-
-    def _measure_pairing(self, weight, rows, N, K) -> bool:
-        x = torch.zeros((rows, K), dtype=self.act_dtype, device=self.device)
-        y = self._new((rows, N))
-        best = []
-        for pair in (0, 1):
-            times = []
-            for i in range(4):
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), None, _p(y), rows, N, K,
-                           0, 0, None, 0, _c_float(0.0), None, None, None, None, None, pair)
-                b.record()
-                b.synchronize()
-                if i:
-                    times.append(a.elapsed_time(b))
-            best.append(min(times))
-        return best[1] < 0.98 * best[0]
 
     def _skinny(self, x, weight, bias, y, M, N, K, out_f32=False, gated=False, scaled=None,
                 resid=None, next_gain=None, out_parts=None, rope=None):
@@ -208,7 +178,7 @@ class HipOps:
                    _c_float(scaled.eps if scaled is not None else 0.0),
                    _p(scaled.rows) if scaled is not None else None, _p(resid), _p(next_gain),
                    _p(out_parts), ctypes.byref(rope) if rope is not None else None,
-                   int(self._pair_tiles(M, N, K, weight)))
+                   int(self._pair_tiles(M, N, K)))
 
     # ------------------------------------------------------------ embedding
     def embed(self, ids, table):
