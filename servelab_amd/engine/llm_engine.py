@@ -50,8 +50,15 @@ class LLMEngine:
                                   self.cache_config.gpu_memory_utilization)
         self.num_blocks = self.runner.manager.num_pages
         if tune_products:
-            # a step that uses its whole token budget is the common large step under load
-            self.runner.tune_products([self.scheduler_config.max_num_batched_tokens])
+            # a step that uses its whole token budget is the common large step under load;
+            # decode steps of more requests than the few-rows kernels take are library products too
+            rows = [self.scheduler_config.max_num_batched_tokens]
+            library_rows = getattr(model.rt.ops, "library_rows", None)
+            if library_rows is not None:
+                first = model.rt.ops.SKINNY_MAX_M + 1
+                rows += sorted({library_rows(n)
+                                for n in range(first, self.scheduler_config.max_num_seqs + 1)})
+            self.runner.tune_products(rows)
         self.scheduler = Scheduler(self.scheduler_config, self.runner.manager, self.clock,
                                    eos_token_id=model.spec.eos_token_id,
                                    max_positions=model.spec.max_position_embeddings)

@@ -310,7 +310,8 @@ class HipOps:
 
         bfloat16, by rows of x: 1..16 the few-rows kernel over the tiled weight,
         17..64 the wide or the LDS-staged kernel (by the size of W), more the
-        library.  float32: the wavefront-per-column kernel up to 16 rows, the
+        library, or 64 rows at a time through those kernels when the result is
+        wanted in float32.  float32: the wavefront-per-column kernel up to 16 rows, the
         tiled FMA kernel above; never a library product."""
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
@@ -339,6 +340,13 @@ class HipOps:
                                    target=self.MID_DEFERRED_WORKGROUPS)
         if M <= self.SKINNY_MAX_M and weight.tiled is not None:
             return self.linear_skinny(x, weight, bias, out_f32)
+        if out_f32 and weight.tiled is not None:
+            # float32 results of many rows (logits of every position): W is
+            # streamed once per 64 rows by the few-rows kernels, several times
+            # faster than the plain tiled kernel below
+            step = self.SKINNY_MAX_M
+            return torch.cat([self.linear_skinny(x[i:i + step], weight, bias, True)
+                              for i in range(0, M, step)])
         w = self.rows_of(weight)
         if M <= self.ROWS_KERNEL_MAX_M and K % 8 == 0:
             return self.linear_rows(x, w, bias, out_f32)
@@ -460,16 +468,33 @@ class HipOps:
         self._call("gemm", "sl_gemm_tiled", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32))
         return y
 
+    LIBRARY_ROW_STEP = 32         # library products of fewer than LIBRARY_PADDED_MAX_M rows run on a
+    LIBRARY_PADDED_MAX_M = 512    # multiple of this many: few distinct shapes, each of which can be tuned
+
+    def library_rows(self, M: int) -> int:
+        """The number of rows a library product of M rows of x runs with."""
+        if M >= self.LIBRARY_PADDED_MAX_M:
+            return M
+        return -(-M // self.LIBRARY_ROW_STEP) * self.LIBRARY_ROW_STEP
+
     def linear_library(self, x, w, bias):
         if self.act_dtype != torch.bfloat16:
             raise KernelError("the library GEMM is for the bfloat16 table only")
+        M = x.shape[0]
+        rows = self.library_rows(M)
+        if rows != M:
+            # the rows beyond M hold whatever the buffer held: every row of a
+            # product depends on its own row of x only, and they are cut off below
+            padded = self._new((rows, x.shape[1]))
+            padded[:M].copy_(x)
+            x = padded
         if bias is None:
-            return torch.mm(x, w.t())
+            return torch.mm(x, w.t())[:M]
         entry = self._bias_cache.get(id(bias))       # (the float bias itself, its bfloat16 copy)
         if entry is None or entry[0] is not bias:
             entry = (bias, bias.to(torch.bfloat16))
             self._bias_cache[id(bias)] = entry
-        return torch.addmm(entry[1], x, w.t())
+        return torch.addmm(entry[1], x, w.t())[:M]
 
     @contextlib.contextmanager
     def library_tuning(self, max_ms: int = 30, results_file: Optional[str] = None):

@@ -139,6 +139,22 @@ def test_linear(both, M, N, K, bias):
         assert rel_err(got, ref) < tol, (M, N, K, out_f32)
 
 
+def test_library_product_pads_its_rows_harmlessly():
+    """Library products of fewer than 512 rows run on a multiple of 32 rows; what
+    the extra rows hold (here: NaN, left behind in the allocator's block) reaches
+    no result row."""
+    from servelab_amd.kernels import HipOps
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    assert [ops.library_rows(m) for m in (65, 96, 97, 511, 512, 700)] == [96, 96, 128, 512, 512, 700]
+    x, w, b = randn(70, 128, dtype=torch.bfloat16, seed=1), randn(200, 128, dtype=torch.bfloat16, scale=0.05, seed=2), randn(200, seed=3)
+    for bias in (None, b):
+        junk = torch.full((96, 128), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+        del junk
+        got = ops.linear_library(x, w, bias)
+        assert got.shape == (70, 200) and got.is_contiguous() and torch.isfinite(got.float()).all()
+        assert rel_err(got, emu.linear(x, w, bias)) < 2 ** -7
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 50, 64), (7, 1000, 3584), (16, 17, 96), (33, 200, 352), (64, 130, 1024)])
 def test_linear_skinny(M, N, K):
     """The matrix-core few-rows kernel alone (bfloat16): ragged M and N."""
