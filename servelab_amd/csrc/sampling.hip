@@ -1,4 +1,4 @@
-// Sampling from float32 logits [R, V]: one block per row.
+// Sampling from float32 logits [R, V].
 //
 //   argmax        first maximal index (servelab/engine/sampler.py:23-24).
 //   sample        temperature 0 => argmax; else a draw from
@@ -216,29 +216,241 @@ __global__ __launch_bounds__(1024) void sample_kernel(
   if (threadIdx.x == 0) out[r] = g.i;
 }
 
+// ---------------------------------------------------------------------------
+// Cuts of a wide vocabulary, on many workgroups.  One workgroup per row (the
+// kernel above) re-reads its row for every pass of the search through one CU;
+// at 152,064 logits that is most of a millisecond for a handful of rows.  Here
+// a row is split into `chunks` slices, one workgroup each, and the cut is
+// found digit by digit, as in a radix sort: round d counts, for each of the 256
+// values of the d-th byte of the ordered bit pattern, the logits that carry it
+// (among those that match the bytes already decided) and the mass of their
+// weights.  The next launch adds the slices' tables up, walks them from the
+// top and decides that byte: the byte in which the k-th largest logit lies
+// (top-k), or in which the cumulative mass passes top_p times the whole
+// (top-p).  After four rounds the cut's bit pattern is known exactly.  Masses
+// are integers (weight * 2^32), so the sums do not depend on the order in which
+// workgroups and lanes add, and a seed draws the same token every time.
+// ---------------------------------------------------------------------------
+constexpr int DIGITS = 256;
+constexpr int CUT_ROUNDS = 4;
+constexpr int CUT_THREADS = 256;          // = DIGITS: thread d decides about digit d
+constexpr int CUT_MAX_CHUNKS = 64;
+
+struct CutState {                          // what the rounds so far know of a row's cut
+  uint64_t mass_above;                     // mass of the logits above every pattern that begins with `prefix`
+  uint64_t target;                         // top-p: top_p * the row's whole mass (known after round 0)
+  uint32_t prefix;                         // the leading bytes of the cut's pattern
+  uint32_t count_above;
+  float xmax;
+  int mode;                                // 0: no cut (or greedy), 1: top-k, 2: top-p
+  int k;
+  int pad;
+};
+
+__device__ __forceinline__ int cut_mode(int V, float T, int k, float p) {
+  if (T == 0.f) return 0;
+  if (k > 0 && k < V) return 1;
+  if (k <= 0 && p < 1.f) return 2;
+  return 0;
+}
+
+// The slice [lo, hi) of a row, four logits at a time where it is 16-byte aligned.
+template <class F>
+__device__ __forceinline__ void for_each_in_slice(const float* __restrict__ x, int lo, int hi, F f) {
+  struct __attribute__((aligned(16))) f4 { float v[4]; };
+  int done = lo;
+  if (((uintptr_t)(x + lo) % 16) == 0) {
+    const int n4 = (hi - lo) / 4;
+    const f4* q = (const f4*)(x + lo);
+    for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+      const f4 v = q[i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) f(v.v[j], lo + 4 * i + j);
+    }
+    done = lo + 4 * n4;
+  }
+  for (int i = done + threadIdx.x; i < hi; i += blockDim.x) f(x[i], i);
+}
+
+// Adds up the slices' tables of the round that has just run and decides its
+// digit.  Every workgroup of the next launch does this for itself (the tables
+// of a row are a few tens of KB in L2); all threads return the new state.
+__device__ CutState cut_advance(CutState st, int round, float top_p, int chunks,
+                                const uint32_t* __restrict__ hc, const uint64_t* __restrict__ hm) {
+  __shared__ uint32_t sn[DIGITS];
+  __shared__ uint64_t sm[DIGITS];
+  __shared__ CutState chosen;
+  const int d = threadIdx.x;
+  uint32_t n = 0;
+  uint64_t m = 0;
+  for (int c = 0; c < chunks; ++c) {
+    n += hc[(size_t)c * DIGITS + d];
+    m += hm[(size_t)c * DIGITS + d];
+  }
+  __syncthreads();                         // the arrays may still be read by an earlier call
+  sn[d] = n;
+  sm[d] = m;
+  if (d == 0) {
+    chosen = st;
+    chosen.mode = 0;                       // nothing crosses: the row keeps everything
+  }
+  __syncthreads();
+  // inclusive sums from the top digit down to d
+  for (int step = 1; step < DIGITS; step *= 2) {
+    uint32_t an = 0;
+    uint64_t am = 0;
+    if (d + step < DIGITS) {
+      an = sn[d + step];
+      am = sm[d + step];
+    }
+    __syncthreads();
+    sn[d] += an;
+    sm[d] += am;
+    __syncthreads();
+  }
+  const uint32_t above_n = sn[d] - n;
+  const uint64_t above_m = sm[d] - m;
+  if (round == 0 && st.mode == 2)          // sm[0]: the whole row
+    st.target = (uint64_t)((double)top_p * (double)sm[0]);
+  bool mine;
+  if (st.mode == 1) {
+    const uint32_t need = (uint32_t)st.k - st.count_above;
+    mine = above_n < need && need <= above_n + n;
+  } else {
+    const uint64_t before = st.mass_above + above_m;
+    mine = before <= st.target && before + m > st.target;
+  }
+  if (mine) {
+    CutState r = st;
+    r.prefix = (st.prefix << 8) | (uint32_t)d;
+    r.count_above = st.count_above + above_n;
+    r.mass_above = st.mass_above + above_m;
+    chosen = r;
+  }
+  __syncthreads();
+  return chosen;
+}
+
+__device__ __forceinline__ uint64_t fixed_weight(float v, float xmax, float invT) {
+  return (uint64_t)(weight_of((v - xmax) * invT) * 4294967296.f);
+}
+
+// Round ROUND: decide the digit of the round before (if any), then count this
+// round's digit over the slice.  hc/hm: [2][R][chunks][DIGITS], the rounds
+// alternate between the two halves; states: [CUT_ROUNDS][R].
+template <int ROUND>
+__global__ __launch_bounds__(CUT_THREADS) void cut_round_kernel(
+    const float* __restrict__ logits, int V, int R, int chunks,
+    const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, const Best* __restrict__ maxes,
+    CutState* __restrict__ states, uint32_t* __restrict__ hc, uint64_t* __restrict__ hm) {
+  __shared__ uint32_t cnt[DIGITS];
+  __shared__ unsigned long long mass[DIGITS];
+  const int r = blockIdx.y, c = blockIdx.x, t = threadIdx.x;
+  const float T = temperature[r];
+  const size_t tables = (size_t)R * chunks * DIGITS;
+  CutState st;
+  if (ROUND == 0) {
+    st.mode = cut_mode(V, T, top_k[r], top_p[r]);
+    float xmax = -INFINITY;
+    for (int i = 0; i < chunks; ++i) xmax = fmaxf(xmax, maxes[(size_t)r * chunks + i].v);
+    st.xmax = xmax;
+    st.prefix = 0;
+    st.count_above = 0;
+    st.mass_above = 0;
+    st.target = 0;
+    st.k = top_k[r];
+    st.pad = 0;
+  } else {
+    st = states[(size_t)(ROUND - 1) * R + r];
+    if (st.mode != 0) {
+      const size_t prev = ((ROUND - 1) % 2) * tables + (size_t)r * chunks * DIGITS;
+      st = cut_advance(st, ROUND - 1, top_p[r], chunks, hc + prev, hm + prev);
+    }
+  }
+  if (c == 0 && t == 0) states[(size_t)ROUND * R + r] = st;
+  if (st.mode == 0) return;
+
+  cnt[t] = 0;
+  mass[t] = 0;
+  __syncthreads();
+  const float invT = 1.f / fmaxf(T, 1e-6f);
+  const int per = ((V + chunks - 1) / chunks + 3) & ~3;
+  const int lo = c * per < V ? c * per : V, hi = lo + per < V ? lo + per : V;
+  const bool weigh = st.mode == 2;
+  // neighbours mostly share a digit in the first rounds: a thread adds up a
+  // run of equal digits before it goes to the table
+  int run_digit = -1;
+  uint32_t run_n = 0;
+  uint64_t run_m = 0;
+  auto flush = [&]() {
+    if (run_n) {
+      atomicAdd(&cnt[run_digit], run_n);
+      if (weigh) atomicAdd(&mass[run_digit], (unsigned long long)run_m);
+    }
+  };
+  for_each_in_slice(logits + (size_t)r * V, lo, hi, [&](float v, int) {
+    const uint32_t key = key_of(v);
+    if (ROUND > 0 && (key >> (32 - 8 * ROUND)) != st.prefix) return;
+    const int digit = (int)((key >> (24 - 8 * ROUND)) & 255u);
+    if (digit != run_digit) {
+      flush();
+      run_digit = digit;
+      run_n = 0;
+      run_m = 0;
+    }
+    run_n += 1;
+    if (weigh) run_m += fixed_weight(v, st.xmax, invT);
+  });
+  flush();
+  __syncthreads();
+  const size_t mine = (ROUND % 2) * tables + ((size_t)r * chunks + c) * DIGITS;
+  hc[mine + t] = cnt[t];
+  hm[mine + t] = mass[t];
+}
+
 // Greedy rows of a wide vocabulary: CHUNKS workgroups per row each find the
 // best of a slice, a second small kernel picks among them (ties: first index).
 // With temperatures the same two stages draw from the whole softmax: the
 // winner of logit_i / T + g_i needs neither the maximum nor a cut, so the row
-// is split like a greedy one (rows with temperature 0 stay greedy).
-__global__ __launch_bounds__(256) void argmax_partial_kernel(
-    const float* __restrict__ logits, int V, int chunks, Best* __restrict__ part,
+// is split like a greedy one (rows with temperature 0 stay greedy).  After the
+// rounds above (`states` given) a row draws among the logits its cut keeps.
+__global__ __launch_bounds__(CUT_THREADS) void argmax_partial_kernel(
+    const float* __restrict__ logits, int V, int R, int chunks, Best* __restrict__ part,
     const float* __restrict__ temperature, const int64_t* __restrict__ seeds,
-    const int64_t* __restrict__ draws) {
+    const int64_t* __restrict__ draws, const float* __restrict__ top_p,
+    const CutState* __restrict__ states, const uint32_t* __restrict__ hc,
+    const uint64_t* __restrict__ hm) {
   __shared__ Best sb[16];
   const int r = blockIdx.y, c = blockIdx.x;
   const float* x = logits + (size_t)r * V;
-  const int per = (V + chunks - 1) / chunks;
-  const int lo = c * per, hi = lo + per < V ? lo + per : V;
+  const int per = ((V + chunks - 1) / chunks + 3) & ~3;
+  const int lo = c * per < V ? c * per : V, hi = lo + per < V ? lo + per : V;
   const float T = temperature != nullptr ? temperature[r] : 0.f;
   Best b = {-INFINITY, 0x7fffffff};
   if (T == 0.f) {
-    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) b = better(b, Best{x[i], i});
+    for_each_in_slice(x, lo, hi, [&](float v, int i) { b = better(b, Best{v, i}); });
   } else {
+    uint32_t lowest = 0;                   // patterns from here on stay in the draw
+    if (states != nullptr) {
+      CutState st = states[(size_t)(CUT_ROUNDS - 1) * R + r];
+      if (st.mode != 0) {
+        const size_t last = ((CUT_ROUNDS - 1) % 2) * ((size_t)R * chunks * DIGITS) +
+                            (size_t)r * chunks * DIGITS;
+        st = cut_advance(st, CUT_ROUNDS - 1, top_p[r], chunks, hc + last, hm + last);
+      }
+      // top-k keeps the k-th largest and its equals; top-p keeps what lies
+      // above the logit at which the mass passes the target, and the maximum
+      // in any case (servelab/engine/sampler.py:30-44)
+      if (st.mode == 1 || (st.mode == 2 && st.count_above == 0)) lowest = st.prefix;
+      else if (st.mode == 2) lowest = st.prefix + 1;
+    }
     const float invT = 1.f / fmaxf(T, 1e-6f);
     const uint64_t seed = (uint64_t)seeds[r], draw = (uint64_t)draws[r];
-    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x)
-      b = better(b, Best{x[i] * invT + gumbel_of(uniform01(seed, draw, (uint32_t)i)), i});
+    for_each_in_slice(x, lo, hi, [&](float v, int i) {
+      if (key_of(v) >= lowest)
+        b = better(b, Best{v * invT + gumbel_of(uniform01(seed, draw, (uint32_t)i)), i});
+    });
   }
   b = block_best(b, sb);
   if (threadIdx.x == 0) part[(size_t)r * chunks + c] = b;
@@ -254,43 +466,84 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const Best* __restrict
   if (threadIdx.x == 0) out[r] = b.i;
 }
 
-// part: chunks * R pairs of (float, int) = 8 * chunks * R bytes of scratch.
-extern "C" const char* sl_argmax(const float* logits, int R, int V, int chunks, void* part,
+static size_t align_up(size_t n) { return (n + 255) & ~(size_t)255; }
+
+// Bytes of scratch for a call with these sizes: the slices' bests, and for
+// cuts found on many workgroups also the rows' maxima, states and tables.
+extern "C" size_t sl_sample_workspace(int R, int chunks, int cuts) {
+  const size_t bests = align_up((size_t)R * chunks * sizeof(Best));
+  if (!cuts) return bests;
+  return 2 * bests + align_up((size_t)CUT_ROUNDS * R * sizeof(CutState)) +
+         align_up(2 * (size_t)R * chunks * DIGITS * sizeof(uint64_t)) +
+         align_up(2 * (size_t)R * chunks * DIGITS * sizeof(uint32_t));
+}
+
+extern "C" const char* sl_argmax(const float* logits, int R, int V, int chunks, void* work,
                                  int* out, hipStream_t stream) {
   SL_CHECK(R >= 0 && V > 0, "argmax: sizes must be positive");
-  SL_CHECK(chunks >= 1 && chunks <= 1024 && part != nullptr, "argmax: 1..1024 chunks and scratch");
+  SL_CHECK(chunks >= 1 && chunks <= 1024 && work != nullptr, "argmax: 1..1024 chunks and scratch");
   SL_CHECK(R <= 65535, "argmax: more than 65535 rows");
   if (R == 0) return nullptr;
-  argmax_partial_kernel<<<dim3(chunks, R), 256, 0, stream>>>(logits, V, chunks, (Best*)part, nullptr,
-                                                           nullptr, nullptr);
+  argmax_partial_kernel<<<dim3(chunks, R), CUT_THREADS, 0, stream>>>(
+      logits, V, R, chunks, (Best*)work, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);
   const char* e = sl_launch_status();
   if (e) return e;
-  argmax_final_kernel<<<R, 64, 0, stream>>>((const Best*)part, chunks, out);
+  argmax_final_kernel<<<R, 64, 0, stream>>>((const Best*)work, chunks, out);
   return sl_launch_status();
 }
 
 // top_k == nullptr and top_p == nullptr: every row draws from its whole
-// softmax (or is greedy), in two stages over `chunks` slices of a row; `part`
-// as for sl_argmax.  Otherwise one workgroup per row finds the row's cut first.
+// softmax (or is greedy), in two stages over `chunks` slices of a row.
+// Otherwise the rows' cuts are found first: with chunks >= 2 by the rounds
+// over slices, else by one workgroup per row.  `work`: sl_sample_workspace bytes.
 extern "C" const char* sl_sample(const float* logits, int R, int V, const float* temperature,
                                  const int* top_k, const float* top_p, const int64_t* seeds,
-                                 const int64_t* draws, int chunks, void* part, int* out,
+                                 const int64_t* draws, int chunks, void* work, int* out,
                                  hipStream_t stream) {
   SL_CHECK(R >= 0 && V > 0, "sample: sizes must be positive");
   SL_CHECK(temperature == nullptr || (seeds != nullptr && draws != nullptr),
            "sample: a temperature needs seeds and draw counters");
   SL_CHECK((top_k == nullptr) == (top_p == nullptr), "sample: top_k and top_p go together");
   if (R == 0) return nullptr;
-  if (top_k == nullptr) {
-    SL_CHECK(chunks >= 1 && chunks <= 1024 && part != nullptr, "sample: 1..1024 chunks and scratch");
-    SL_CHECK(R <= 65535, "sample: more than 65535 rows");
-    argmax_partial_kernel<<<dim3(chunks, R), 256, 0, stream>>>(logits, V, chunks, (Best*)part,
-                                                             temperature, seeds, draws);
-    const char* e = sl_launch_status();
-    if (e) return e;
-    argmax_final_kernel<<<R, 64, 0, stream>>>((const Best*)part, chunks, out);
+  if (top_k != nullptr && chunks < 2) {
+    sample_kernel<<<R, 1024, 0, stream>>>(logits, V, temperature, top_k, top_p, seeds, draws, out);
     return sl_launch_status();
   }
-  sample_kernel<<<R, 1024, 0, stream>>>(logits, V, temperature, top_k, top_p, seeds, draws, out);
+  SL_CHECK(chunks >= 1 && chunks <= 1024 && work != nullptr, "sample: 1..1024 chunks and scratch");
+  SL_CHECK(R <= 65535, "sample: more than 65535 rows");
+  Best* bests = (Best*)work;
+  if (top_k == nullptr) {
+    argmax_partial_kernel<<<dim3(chunks, R), CUT_THREADS, 0, stream>>>(
+        logits, V, R, chunks, bests, temperature, seeds, draws, nullptr, nullptr, nullptr, nullptr);
+  } else {
+    SL_CHECK(temperature != nullptr, "sample: cuts need temperatures");
+    SL_CHECK(chunks <= CUT_MAX_CHUNKS, "sample: at most 64 slices a row when cuts are searched");
+    char* at = (char*)work + align_up((size_t)R * chunks * sizeof(Best));
+    Best* maxes = (Best*)at;
+    at += align_up((size_t)R * chunks * sizeof(Best));
+    CutState* states = (CutState*)at;
+    at += align_up((size_t)CUT_ROUNDS * R * sizeof(CutState));
+    uint64_t* hm = (uint64_t*)at;
+    at += align_up(2 * (size_t)R * chunks * DIGITS * sizeof(uint64_t));
+    uint32_t* hc = (uint32_t*)at;
+    const dim3 grid(chunks, R);
+    argmax_partial_kernel<<<grid, CUT_THREADS, 0, stream>>>(
+        logits, V, R, chunks, maxes, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr);
+    cut_round_kernel<0><<<grid, CUT_THREADS, 0, stream>>>(logits, V, R, chunks, temperature, top_k,
+                                                          top_p, maxes, states, hc, hm);
+    cut_round_kernel<1><<<grid, CUT_THREADS, 0, stream>>>(logits, V, R, chunks, temperature, top_k,
+                                                          top_p, maxes, states, hc, hm);
+    cut_round_kernel<2><<<grid, CUT_THREADS, 0, stream>>>(logits, V, R, chunks, temperature, top_k,
+                                                          top_p, maxes, states, hc, hm);
+    cut_round_kernel<3><<<grid, CUT_THREADS, 0, stream>>>(logits, V, R, chunks, temperature, top_k,
+                                                          top_p, maxes, states, hc, hm);
+    const char* e = sl_launch_status();
+    if (e) return e;
+    argmax_partial_kernel<<<grid, CUT_THREADS, 0, stream>>>(
+        logits, V, R, chunks, bests, temperature, seeds, draws, top_p, states, hc, hm);
+  }
+  const char* e = sl_launch_status();
+  if (e) return e;
+  argmax_final_kernel<<<R, 64, 0, stream>>>((const Best*)work, chunks, out);
   return sl_launch_status();
 }

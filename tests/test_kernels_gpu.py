@@ -674,3 +674,41 @@ def test_sampling_cuts_of_a_wide_vocabulary(V):
     assert got <= inside and len(got & surely) > min(len(surely), 40) // 2
     # a top_p below the largest probability keeps that entry alone
     assert draw(none, torch.full((R,), float(sp[0]) * 0.5).cuda(), rounds=2) == {1234}
+
+
+def test_sampling_rows_with_different_rules_in_one_call():
+    """Rows of one call follow their own rule (greedy, top-k, top-p, none) when
+    the cuts are searched by several workgroups a row; rows that are not
+    16-byte aligned, entries at -inf and equal logits at the cut included."""
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.float32, "cuda:0")
+    V, T = 40003, 0.8
+    base = 2.0 * randn(6, V, seed=5)
+    base[4, torch.randperm(V)[: V // 2].cuda()] = -math.inf
+    top = base[5].max().item()
+    base[5, [11, 2222, 33333]] = top + 1.0              # three equal logits at the top
+    logits = base.contiguous()
+    temp = torch.tensor([0.0, T, T, T, T, T]).cuda()
+    top_k = torch.tensor([-1, 1, -1, -1, 40, -1], dtype=torch.int32).cuda()
+    top_p = torch.tensor([1.0, 1.0, 1e-6, 1.0, 1.0, 0.5]).cuda()
+    seeds = torch.arange(6, dtype=torch.int64).cuda()
+    got = [set() for _ in range(6)]
+    for j in range(40):
+        draws = torch.full((6,), j, dtype=torch.int64).cuda()
+        toks = ops.sample(logits, temp, top_k, top_p, seeds, draws).tolist()
+        assert toks == ops.sample(logits, temp, top_k, top_p, seeds, draws).tolist()
+        for r, t in enumerate(toks):
+            got[r].add(t)
+    best = torch.argmax(logits, -1).tolist()
+    assert got[0] == {best[0]} and got[1] == {best[1]} and got[2] == {best[2]}
+    assert len(got[3]) > 20                               # no cut: draws spread over the row
+    assert got[4] <= set(torch.topk(logits[4], 40).indices.tolist()) and len(got[4]) > 10
+    probs = torch.softmax(logits[5].double().cpu() / T, -1)
+    sp, si = torch.sort(probs, descending=True)
+    cum = torch.cumsum(sp, 0)
+    inside = set(si[(cum <= 0.5 + 1e-4) | (torch.arange(V) == 0)].tolist())
+    assert got[5] <= inside and {11, 2222, 33333} & got[5]
+    # the row without a cut draws what the two-stage kernel alone draws
+    draws = torch.zeros(6, dtype=torch.int64).cuda()
+    assert (ops.sample(logits, temp, top_k, top_p, seeds, draws)[3]
+            == ops.sample(logits, temp, None, None, seeds, draws)[3])
