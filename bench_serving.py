@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Generation through ``LLMEngine`` under load, in one process: time to first
+token, time per output token, output throughput and the share of requests
+inside both latency bounds.
+
+The workload and the options are those of the reference's harness
+(servelab/bench/benchmark_serving.py:58-157, servelab/bench/datasets.py:8-20):
+prompts of random token ids whose lengths are Gaussian (``--input-mean``, 40
+around it), a Gaussian number of output tokens (``--output-tokens``, 20 around
+it) with ``ignore_eos``, either a closed loop that keeps ``--concurrency``
+requests in flight (``--load-pattern fixed``) or arrivals with exponential gaps
+at ``--request-rate`` a second against the wall clock (``poisson``).  Token ids
+are uniform over the vocabulary; no public dataset is read.
+
+    python bench_serving.py                       # Qwen2.5-7B shape, random weights
+    python bench_serving.py --model DIR --num-prompts 64 --load-pattern poisson --request-rate 8
+
+The last line printed is one JSON object with the same figures.
+"""
+import argparse
+import json
+import math
+import os
+import random
+import sys
+import time
+from dataclasses import dataclass
+from typing import List
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+@dataclass
+class Request:
+    prompt_token_ids: List[int]
+    output_tokens: int
+
+
+def synthetic_requests(n: int, vocab: int, input_mean: int, output_mean: int, seed: int,
+                       input_std: int = 40, output_std: int = 20, longest: int = 0) -> List[Request]:
+    """``longest`` > 0 bounds prompt + output (the model's positions)."""
+    rng = random.Random(seed)
+    out = []
+    for _ in range(n):
+        n_in = max(8, int(rng.gauss(input_mean, input_std)))
+        n_out = max(1, int(rng.gauss(output_mean, output_std)))
+        if longest:
+            n_in = min(n_in, max(1, longest - n_out))
+        out.append(Request([rng.randrange(vocab) for _ in range(n_in)], n_out))
+    return out
+
+
+def _submit(engine, req: Request, sampling):
+    from servelab_amd import SamplingParams
+    return engine.add_request(
+        prompt_token_ids=req.prompt_token_ids,
+        sampling_params=SamplingParams(max_tokens=req.output_tokens, ignore_eos=True, **sampling))
+
+
+def closed_loop(engine, requests: List[Request], concurrency: int, sampling) -> list:
+    """Keeps ``concurrency`` requests in flight until all are done."""
+    waiting = list(reversed(requests))
+    live, done = set(), []
+    while waiting or live:
+        while waiting and len(live) < concurrency:
+            live.add(_submit(engine, waiting.pop(), sampling))
+        for out in engine.step():
+            if out.request_id in live:
+                live.discard(out.request_id)
+                done.append(out)
+    return done
+
+
+def open_loop(engine, requests: List[Request], rate: float, sampling, seed: int = 7) -> list:
+    """Arrivals with exponential gaps against the wall clock; the engine steps
+    whenever it has work and sleeps until the next arrival otherwise."""
+    rng = random.Random(seed)
+    done, at = [], time.monotonic()
+    for req in requests:
+        while True:
+            now = time.monotonic()
+            if now >= at:
+                break
+            if engine.has_unfinished():
+                done.extend(engine.step())
+            else:
+                time.sleep(min(at - now, 0.001))
+        _submit(engine, req, sampling)
+        at += rng.expovariate(rate)
+    while engine.has_unfinished():
+        done.extend(engine.step())
+    return done
+
+
+def percentile(values: List[float], q: float) -> float:
+    """Linear interpolation between the order statistics."""
+    if not values:
+        return float("nan")
+    v = sorted(values)
+    x = (len(v) - 1) * q / 100.0
+    lo = int(math.floor(x))
+    hi = min(lo + 1, len(v) - 1)
+    return v[lo] + (v[hi] - v[lo]) * (x - lo)
+
+
+def summarise(done: list, elapsed: float, ttft_slo_ms: float, tpot_slo_ms: float) -> dict:
+    """TTFT = first token - arrival; TPOT = (latency - TTFT) / (output tokens - 1)
+    (servelab/bench/benchmark_serving.py:102-113)."""
+    ttft, tpot, pairs, tokens, preemptions = [], [], [], 0, 0
+    for out in done:
+        m = out.metrics
+        n = len(out.outputs[0].token_ids)
+        tokens += n
+        preemptions += m["preemptions"]
+        t = m["ttft"] * 1e3
+        ttft.append(t)
+        if n > 1:
+            p = (m["latency"] - m["ttft"]) / (n - 1) * 1e3
+            tpot.append(p)
+            pairs.append((t, p))
+    good = sum(1 for t, p in pairs if t <= ttft_slo_ms and p <= tpot_slo_ms)
+    return {
+        "requests": len(done), "elapsed_s": round(elapsed, 3),
+        "output_tokens": tokens, "output_throughput_tok_s": round(tokens / elapsed, 1),
+        "ttft_ms_p50": round(percentile(ttft, 50), 2), "ttft_ms_p90": round(percentile(ttft, 90), 2),
+        "ttft_ms_p99": round(percentile(ttft, 99), 2),
+        "tpot_ms_p50": round(percentile(tpot, 50), 3), "tpot_ms_p99": round(percentile(tpot, 99), 3),
+        "goodput": round(good / max(1, len(pairs)), 4), "preemptions": preemptions,
+    }
+
+
+def build_engine(args):
+    from servelab_amd import CacheConfig, LLMEngine, SchedulerConfig, load_config
+    cache = CacheConfig(block_size=args.block_size, num_blocks=args.num_blocks or None,
+                        gpu_memory_utilization=args.gpu_memory_utilization)
+    sched = SchedulerConfig(max_num_seqs=args.max_num_seqs,
+                            max_num_batched_tokens=args.max_batched_tokens,
+                            chunked_prefill=not args.no_chunked_prefill,
+                            policy=args.scheduler_policy)
+    if args.model:
+        cfg = load_config(args.model)
+        return cfg, LLMEngine(cfg, cache, sched, dtype=args.dtype, tune_products=args.tune_products)
+    import bench                                     # random weights of a named shape, made on the device
+    cfg, model, _ = bench.build(argparse.Namespace(shape=args.shape, layers=args.layers,
+                                                   dtype=args.dtype, seed=args.seed))
+    return cfg, LLMEngine(cfg, cache, sched, model=model, tune_products=args.tune_products)
+
+
+def run(args) -> dict:
+    cfg, engine = build_engine(args)
+    sampling = dict(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k)
+    requests = synthetic_requests(args.num_prompts, cfg.vocab_size, args.input_mean,
+                                  args.output_tokens, args.seed,
+                                  longest=cfg.max_position_embeddings)
+    if args.warmup_requests:
+        # the first steps of a process compile nothing, but capture a graph per decode shape
+        warm = synthetic_requests(args.warmup_requests, cfg.vocab_size, args.input_mean, 8,
+                                  args.seed + 1, longest=cfg.max_position_embeddings)
+        closed_loop(engine, warm, min(args.concurrency, len(warm)), sampling)
+    steps0 = engine.num_steps
+    t0 = time.monotonic()
+    if args.load_pattern == "fixed":
+        done = closed_loop(engine, requests, args.concurrency, sampling)
+    else:
+        done = open_loop(engine, requests, args.request_rate, sampling)
+    elapsed = time.monotonic() - t0
+    res = summarise(done, elapsed, args.ttft_slo_ms, args.tpot_slo_ms)
+    res["steps"] = engine.num_steps - steps0
+    res["config"] = {
+        "model": args.model or f"{args.shape} shape, random weights", "dtype": args.dtype,
+        "load_pattern": args.load_pattern,
+        "concurrency": args.concurrency if args.load_pattern == "fixed" else None,
+        "request_rate": args.request_rate if args.load_pattern == "poisson" else None,
+        "num_prompts": args.num_prompts, "input_mean": args.input_mean,
+        "output_tokens": args.output_tokens, "max_num_seqs": args.max_num_seqs,
+        "max_batched_tokens": args.max_batched_tokens, "block_size": args.block_size,
+        "num_blocks": engine.num_blocks, "temperature": args.temperature, "top_p": args.top_p,
+        "top_k": args.top_k,
+    }
+    return res
+
+
+def parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--model", default="", help="model folder; empty = random weights of --shape")
+    ap.add_argument("--shape", default="7b", choices=["7b", "32b", "72b"])
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--num-prompts", type=int, default=32)
+    ap.add_argument("--input-mean", type=int, default=200)
+    ap.add_argument("--output-tokens", type=int, default=64)
+    ap.add_argument("--load-pattern", choices=["fixed", "poisson"], default="fixed")
+    ap.add_argument("--concurrency", type=int, default=8)
+    ap.add_argument("--request-rate", type=float, default=2.0)
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--num-blocks", type=int, default=0, help="0 = from free memory")
+    ap.add_argument("--max-num-seqs", type=int, default=64)
+    ap.add_argument("--max-batched-tokens", type=int, default=2048)
+    ap.add_argument("--no-chunked-prefill", action="store_true")
+    ap.add_argument("--scheduler-policy", default="fcfs", choices=["fcfs", "priority"])
+    ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
+    ap.add_argument("--ttft-slo-ms", type=float, default=2000)
+    ap.add_argument("--tpot-slo-ms", type=float, default=50)
+    ap.add_argument("--temperature", type=float, default=0.0)
+    ap.add_argument("--top-p", type=float, default=1.0)
+    ap.add_argument("--top-k", type=int, default=-1)
+    ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--warmup-requests", type=int, default=4,
+                    help="short requests run before the clock starts (0 = none)")
+    ap.add_argument("--tune-products", action="store_true")
+    return ap
+
+
+def main(argv=None) -> int:
+    args = parser().parse_args(argv)
+    res = run(args)
+    rows = [("requests", res["requests"]), ("elapsed_s", res["elapsed_s"]),
+            ("output_throughput_tok/s", res["output_throughput_tok_s"]),
+            ("TTFT ms p50/p90/p99",
+             f"{res['ttft_ms_p50']:.1f} / {res['ttft_ms_p90']:.1f} / {res['ttft_ms_p99']:.1f}"),
+            ("TPOT ms p50/p99", f"{res['tpot_ms_p50']:.2f} / {res['tpot_ms_p99']:.2f}"),
+            ("goodput (TTFT and TPOT bound)", f"{res['goodput']:.1%}"),
+            ("preemptions", res["preemptions"]), ("engine steps", res["steps"])]
+    width = max(len(k) for k, _ in rows)
+    for k, v in rows:
+        print(f"{k:<{width}}  {v}")
+    print(json.dumps(res), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -192,3 +192,25 @@ def test_tuned_library_products_keep_the_logits(tmp_path):
     assert (after - before).abs().max().item() < tol
     name = os.path.join(tempfile.gettempdir(), f"servelab_amd_tunableop_{os.getuid()}.csv")
     assert os.path.exists(name)
+
+
+@pytest.mark.parametrize("pattern", ["fixed", "poisson"])
+def test_load_benchmark_on_a_tiny_model(tmp_path, pattern):
+    """The load benchmark drives the real engine: every request comes back with
+    its number of tokens, and the figures are those of its outputs."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench_serving as bs
+    folder = make_folder(tmp_path, "B", seed=31)
+    args = bs.parser().parse_args([
+        "--model", folder, "--num-prompts", "9", "--input-mean", "60", "--output-tokens", "10",
+        "--load-pattern", pattern, "--concurrency", "3", "--request-rate", "400",
+        "--num-blocks", "96", "--max-num-seqs", "4", "--max-batched-tokens", "64",
+        "--warmup-requests", "2", "--temperature", "0.7", "--top-p", "0.9"])
+    res = bs.run(args)
+    want = bs.synthetic_requests(9, TINY["B"]["vocab_size"], 60, 10, 42,
+                                 longest=TINY["B"]["max_position_embeddings"])
+    assert res["requests"] == 9 and res["output_tokens"] == sum(r.output_tokens for r in want)
+    assert res["output_throughput_tok_s"] > 0 and res["ttft_ms_p50"] > 0 and res["tpot_ms_p50"] > 0
+    assert res["ttft_ms_p99"] >= res["ttft_ms_p50"] and res["steps"] > 0
