@@ -658,7 +658,7 @@ extern "C" const char* sl_gemm_wide(const void* x, const void* wt, const float* 
   return sl_launch_status();
 }
 
-// ------------------------------------- 17 to 64 rows, x staged through LDS
+// ------------------------------------ 17 to 128 rows, x staged through LDS
 // The kernel above reads x from L2 once per 32 rows of W.  Here a workgroup of
 // 4 wavefronts owns 128 rows of W (each wavefront two tiles over the
 // workgroup's whole share of K, so nothing is reduced across wavefronts) and
@@ -879,7 +879,7 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
                                    int M, int N, int K, int out_f32, int gated, int ks,
                                    int wide_min_wgs, int num_cus, float* part, hipStream_t stream) {
   SL_CHECK(M > 0 && N > 0 && K > 0, "gemm_mid: sizes must be positive");
-  SL_CHECK(M <= 64, "gemm_mid: at most 64 rows");
+  SL_CHECK(M <= 128, "gemm_mid: at most 128 rows");
   SL_CHECK(K % 32 == 0, "gemm_mid: K must be a multiple of 32");
   SL_CHECK(ks >= 1 && ks <= 16 && ks <= K / 32, "gemm_mid: ks must be in 1..16 and <= K / 32");
   SL_CHECK(ks == 1 || part != nullptr, "gemm_mid: a split of K needs the partial buffer");
@@ -905,10 +905,12 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
   const dim3 grid(groups, ks);
   if (wide) {
     if (M <= 32) gemm_mid_kernel<2, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
-    else gemm_mid_kernel<4, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    else if (M <= 64) gemm_mid_kernel<4, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    else gemm_mid_kernel<8, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
   } else {
     if (M <= 32) gemm_mid_kernel<2, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
-    else gemm_mid_kernel<4, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    else if (M <= 64) gemm_mid_kernel<4, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    else gemm_mid_kernel<8, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
   }
   const char* e = sl_launch_status();
   if (e || ks == 1 || y == nullptr) return e;

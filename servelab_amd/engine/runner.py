@@ -36,8 +36,10 @@ class ModelRunner:
         self.max_positions = model.spec.max_position_embeddings
         self.steps = 0
         self.tokens_run = 0
-        # decode steps of up to GRAPH_MAX_SEQS single tokens replay a captured HIP graph
+        # decode steps of up to graph_max_seqs single tokens replay a captured HIP graph; a kernel
+        # table says itself up to how many rows its products stay clear of library calls
         self.use_graphs = (use_graphs and self.rt.device.type == "cuda" and model.spec.graph_safe)
+        self.graph_max_seqs = int(getattr(self.rt.ops, "graph_rows_limit", self.GRAPH_MAX_SEQS))
         self._graphs = {}
         self.graph_replays = 0
         self._decoding = None         # the last graph step, for the next one to continue from
@@ -102,7 +104,7 @@ class ModelRunner:
         """(sequences, context capacity) when the step is a pure decode step
         that a captured graph can run, else None."""
         B = len(packed)
-        if not self.use_graphs or B > self.GRAPH_MAX_SEQS or len(rows) != B:
+        if not self.use_graphs or B > self.graph_max_seqs or len(rows) != B:
             return None
         if any(len(e.tokens) != 1 for e in packed) or rows != list(range(B)):
             return None

@@ -126,6 +126,10 @@ class HipOps:
         self.fuse_rope = act_dtype == torch.bfloat16
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
         self._untiled = None          # scratch for "tiled": the row-major form of one matrix
+        # Up to this many rows no product of a prepared weight goes to the library
+        # (whose kernels may record memsets, which HIP graphs replay wrongly here):
+        # decode steps of at most this many requests can be captured.
+        self.graph_rows_limit = self.MID_MAX_M if act_dtype == torch.bfloat16 else self.SKINNY_MAX_M
 
     # ------------------------------------------------------------ plumbing
     def _call(self, stem, name, *args):
@@ -278,13 +282,19 @@ class HipOps:
         embedding table), so keeping it costs nothing."""
         N, K = w.shape
         self._check(w, self.act_dtype, None, "weight")
-        if self.act_dtype != torch.bfloat16 or K % 32 or self.weight_layout == "rows":
+        if self.act_dtype != torch.bfloat16:
+            return LinearWeight(w)
+        if K % 32 or self.weight_layout == "rows":
+            self.graph_rows_limit = min(self.graph_rows_limit, self.ROWS_KERNEL_MAX_M)
             return LinearWeight(w)
         tiled = torch.empty(-(-N // 16) * 16 * K, dtype=torch.bfloat16, device=self.device)
         self._call("gemm", "sl_tile_weight", _p(w), _p(tiled), N, K)
         if self.weight_layout == "tiled" and not keep_rows:
-            return LinearWeight(None, tiled, (N, K))
-        return LinearWeight(w, tiled)
+            weight = LinearWeight(None, tiled, (N, K))
+        else:
+            weight = LinearWeight(w, tiled)
+        self.graph_rows_limit = min(self.graph_rows_limit, self._few_rows_limit(weight))
+        return weight
 
     def rows_of(self, weight):
         """The row-major matrix of a weight; for a tiled-only weight it is
@@ -309,9 +319,9 @@ class HipOps:
         of a product whose K was split (the norm adds them up).
 
         bfloat16, by rows of x: 1..16 the few-rows kernel over the tiled weight,
-        17..64 the wide or the LDS-staged kernel (by the size of W), more the
-        library, or 64 rows at a time through those kernels when the result is
-        wanted in float32.  float32: the wavefront-per-column kernel up to 16 rows, the
+        17..64 the wide or the LDS-staged kernel (by the size of W; the latter
+        up to 128 rows), more the library, or that many rows at a time through
+        those kernels when the result is wanted in float32.  float32: the wavefront-per-column kernel up to 16 rows, the
         tiled FMA kernel above; never a library product."""
         if not isinstance(weight, LinearWeight):
             weight = LinearWeight(weight)
@@ -333,20 +343,19 @@ class HipOps:
             if K % 4 == 0 and M <= self.ROWS_KERNEL_MAX_M:
                 return self.linear_rows(x, weight.w, bias, out_f32)
             return self.linear_tiled(x, weight.w, bias, out_f32)
-        if (defer and self.fuse_norms and not out_f32 and self.WIDE_MIN_M <= M <= self.SKINNY_MAX_M
-                and weight.tiled is not None and K % 32 == 0 and N % 4 == 0
-                and self._takes_mid(M, N, K)):
+        limit = self._few_rows_limit(weight)
+        if (defer and self.fuse_norms and not out_f32 and self.WIDE_MIN_M <= M <= limit
+                and K % 32 == 0 and N % 4 == 0 and self._takes_mid(M, N, K)):
             return self.linear_mid(x, weight, bias, partial=True,     # the norm adds the partial sums
                                    target=self.MID_DEFERRED_WORKGROUPS)
-        if M <= self.SKINNY_MAX_M and weight.tiled is not None:
+        if M <= limit:
             return self.linear_skinny(x, weight, bias, out_f32)
-        if out_f32 and weight.tiled is not None:
+        if out_f32 and limit:
             # float32 results of many rows (logits of every position): W is
-            # streamed once per 64 rows by the few-rows kernels, several times
-            # faster than the plain tiled kernel below
-            step = self.SKINNY_MAX_M
-            return torch.cat([self.linear_skinny(x[i:i + step], weight, bias, True)
-                              for i in range(0, M, step)])
+            # streamed once per `limit` rows by the few-rows kernels, several
+            # times faster than the plain tiled kernel below
+            return torch.cat([self.linear_skinny(x[i:i + limit], weight, bias, True)
+                              for i in range(0, M, limit)])
         w = self.rows_of(weight)
         if M <= self.ROWS_KERNEL_MAX_M and K % 8 == 0:
             return self.linear_rows(x, w, bias, out_f32)
@@ -378,9 +387,23 @@ class HipOps:
     def _takes_mid(self, M, N, K) -> bool:
         return N * K >= (self.MID_MIN_ELEMENTS if M <= 32 else self.MID_MIN_ELEMENTS_MANY)
 
+    MID_MAX_M = 128               # the LDS-staged kernel takes up to this many rows
+
+    def _few_rows_limit(self, weight) -> int:
+        """Up to how many rows of x a product with this weight stays with the
+        kernels that stream the tiled copy (more rows: the library): none
+        without a tiled copy, SKINNY_MAX_M, or MID_MAX_M where the LDS-staged
+        kernel takes the matrix."""
+        if weight.tiled is None or self.act_dtype != torch.bfloat16:
+            return 0
+        N, K = weight.shape
+        if K % 32 == 0 and N * K >= self.MID_MIN_ELEMENTS_MANY:
+            return self.MID_MAX_M
+        return self.SKINNY_MAX_M
+
     def linear_mid(self, x, weight, bias, out_f32=False, gated=False, ks=None, partial=False,
                    target=None):
-        """17..64 rows with x staged through LDS; K split over workgroups when
+        """17..128 rows with x staged through LDS; K split over workgroups when
         N alone gives too few of them.  ``partial``: a split product comes back
         as ``PartialSums`` for its reader to add up."""
         M, K = x.shape
@@ -442,8 +465,7 @@ class HipOps:
             return self._linear_scaled(x, weight, None, False, True)
         M, K = x.shape
         N = weight.shape[0]
-        if (M <= self.SKINNY_MAX_M and weight.tiled is not None and block == self.GATE_BLOCK
-                and N % 16 == 0):
+        if M <= self._few_rows_limit(weight) and block == self.GATE_BLOCK and N % 16 == 0:
             self._check(x, self.act_dtype, None, "x")
             if M >= self.WIDE_MIN_M:
                 if self._takes_mid(M, N, K):
@@ -595,8 +617,8 @@ class HipOps:
         fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
                  and weight.tiled is not None and weight.shape == (N, K))
         if not fused:
-            if (self.act_dtype == torch.bfloat16 and self.WIDE_MIN_M <= M <= self.SKINNY_MAX_M
-                    and weight.tiled is not None and K % 32 == 0 and not isinstance(x, ScaledRows)):
+            if (self.WIDE_MIN_M <= M <= self._few_rows_limit(weight) and K % 32 == 0
+                    and not isinstance(x, ScaledRows)):
                 # K split over workgroups; the rotation kernel adds the partial sums up
                 product = self.linear_mid(x, weight, bias, partial=True)
                 if isinstance(product, PartialSums):

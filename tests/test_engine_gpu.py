@@ -214,3 +214,43 @@ def test_load_benchmark_on_a_tiny_model(tmp_path, pattern):
     assert res["requests"] == 9 and res["output_tokens"] == sum(r.output_tokens for r in want)
     assert res["output_throughput_tok_s"] > 0 and res["ttft_ms_p50"] > 0 and res["tpot_ms_p50"] > 0
     assert res["ttft_ms_p99"] >= res["ttft_ms_p50"] and res["steps"] > 0
+
+
+def test_decode_graphs_of_a_hundred_requests():
+    """With matrices large enough for the LDS-staged kernel, decode steps of 65
+    to 128 requests hold no library product and replay a graph: same logits as
+    the eager steps, and as each request stepped alone."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    from servelab_amd import Qwen2Config
+    from servelab_amd.engine.session import make_runtime
+    from servelab_amd.parts import DecoderModel, build_model_spec
+    raw = dict(bench.QWEN25_7B, num_hidden_layers=1, hidden_size=3072, num_attention_heads=24,
+               num_key_value_heads=4, intermediate_size=3072, vocab_size=4096)
+    rt = make_runtime(torch.bfloat16, "cuda:0")
+    model = DecoderModel(build_model_spec(Qwen2Config.from_hf(raw)), rt)
+    model.load(bench.RandomCheckpoint(model.spec.param_specs(), 5, rt.device, torch.bfloat16))
+    assert rt.ops.graph_rows_limit == 128
+    B = 100
+    rng = random.Random(9)
+    prompts = {f"r{i}": [rng.randrange(4096) for _ in range(3 + i % 5)] for i in range(B)}
+    runs = {}
+    for use_graphs in (False, True):
+        runner = ModelRunner(model, 2 * B + 8, 16, max_num_seqs=B, use_graphs=use_graphs)
+        for r, p in prompts.items():
+            assert runner.open(r)
+        runner.step([StepEntry(r, p, []) for r, p in prompts.items()])
+        rows = [runner.step([StepEntry(r, [(7 * i + j) % 4096], [0]) for j, r in enumerate(prompts)]).clone()
+                for i in range(4)]
+        runs[use_graphs] = torch.stack(rows)
+        assert runner.graph_replays == (3 if use_graphs else 0)
+    assert torch.equal(runs[True], runs[False])
+    # request 17 alone: the few-rows kernels of one row, not the 128-row one
+    runner = ModelRunner(model, 16, 16, use_graphs=False)
+    runner.open("solo")
+    runner.step([StepEntry("solo", prompts["r17"], [])])
+    for i in range(4):
+        alone = runner.step([StepEntry("solo", [(7 * i + 17) % 4096], [0])])[0]
+        assert (alone - runs[True][i, 17]).abs().max().item() < 0.05 * alone.abs().max().item()

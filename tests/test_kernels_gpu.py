@@ -172,9 +172,10 @@ def test_linear_skinny(M, N, K):
             assert rel_err(got, emu.linear(x, w, bias, out_f32)) < (2e-5 if out_f32 else 2 ** -7)
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048)])
+@pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048),
+                                   (65, 144, 352), (100, 1000, 3584), (128, 4608, 1024), (127, 70, 2048)])
 def test_linear_mid(M, N, K):
-    """The LDS-staged 17..64-row kernel alone: whole K and K split over up to
+    """The LDS-staged 17..128-row kernel alone: whole K and K split over up to
     16 workgroups with the separate reduction, plain and gated."""
     from servelab_amd.kernels import HipOps
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
@@ -712,3 +713,27 @@ def test_sampling_rows_with_different_rules_in_one_call():
     draws = torch.zeros(6, dtype=torch.int64).cuda()
     assert (ops.sample(logits, temp, top_k, top_p, seeds, draws)[3]
             == ops.sample(logits, temp, None, None, seeds, draws)[3])
+
+
+def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
+    """Large matrices take the LDS-staged kernel up to 128 rows (plain, gated,
+    deferred to the norm, with rotation and cache write, float32 logits of more
+    rows in slices of 128); small ones go to the library from 65 rows on."""
+    from servelab_amd.kernels import HipOps
+    from servelab_amd.kernels.ops import PartialSums
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    M, K, N = 100, 3584, 2560                        # N K = 9.2 M elements: the LDS-staged kernel's
+    x = randn(M, K, dtype=torch.bfloat16, seed=1)
+    w = randn(N, K, dtype=torch.bfloat16, scale=0.05, seed=2)
+    weight, b = ops.prepare_weight(w), randn(N, seed=3)
+    assert ops._few_rows_limit(weight) == 128
+    assert ops._few_rows_limit(ops.prepare_weight(w[:256].contiguous())) == 64
+    assert torch.equal(ops.linear(x, weight, b), ops.linear_mid(x, weight, b))
+    assert rel_err(ops.linear(x, weight, b), emu.linear(x, w, b)) < 2 ** -7
+    assert rel_err(ops.gated_linear(x, weight, 8), emu.silu_mul(emu.linear(x, w, None), 8)) < 2 ** -6
+    delta = ops.linear(x, weight[:0] if False else weight, b, defer=True)
+    assert isinstance(delta, PartialSums)
+    assert rel_err(ops.materialize(delta), emu.linear(x, w, b)) < 2 ** -7
+    many = randn(300, K, dtype=torch.bfloat16, seed=4)
+    got = ops.linear(many, weight, b, out_f32=True)
+    assert got.shape == (300, N) and rel_err(got, emu.linear(many, w, b, True)) < 2e-5
