@@ -685,9 +685,11 @@ class HipOps:
     GENERAL_ATTENTION_WAVES = 4096  # the general kernel's decode launches aim for this many wavefronts
     TARGET_WAVES = 512            # wavefronts a decode launch aims for when it splits the context
     # Prompt launches share keys through LDS when they have at least MIN_WAVES 32-column wavefronts (enough
-    # workgroups of four) and WAVES of them counted once per 2,048 tokens of context (what each pulls from L2).
-    SHARED_ATTENTION_WAVES = 2048
+    # workgroups of four, two tiles each) and contexts of MIN_CONTEXT tokens (measured on MI355X, 7B shape:
+    # one prompt of 1,024 tokens 46 us either way, 1,536: 65 against 70 us, 2,048: 80 against 95 us,
+    # 8,192: 737 against 1,125 us; eight prompts of 256: 23.5 against 21.6 us).
     SHARED_ATTENTION_MIN_WAVES = 1024
+    SHARED_ATTENTION_MIN_CONTEXT = 1024
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples
@@ -727,7 +729,7 @@ class HipOps:
         if n_pre:
             waves = -(-batch.max_q_len * (nh // nkv) // 32) * nkv * n_pre
             shared = (waves >= self.SHARED_ATTENTION_MIN_WAVES and
-                      waves * max(1, batch.max_ctx_len // 2048) >= self.SHARED_ATTENTION_WAVES)
+                      batch.max_ctx_len >= self.SHARED_ATTENTION_MIN_CONTEXT)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, 1,
                        0 if shared else 1 << 30, _p(out), None, None, 0, 0)
         if n_dec:

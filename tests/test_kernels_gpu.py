@@ -501,7 +501,7 @@ def test_prompt_attention_through_lds(nh, nkv, D, page, window):
     from servelab_amd.kernels import HipOps
     dt = torch.bfloat16
     ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
-    ops.SHARED_ATTENTION_WAVES = ops.SHARED_ATTENTION_MIN_WAVES = 0
+    ops.SHARED_ATTENTION_MIN_CONTEXT = ops.SHARED_ATTENTION_MIN_WAVES = 0
     seqs = [(130, 130), (277, 45), (64, 64), (200, 2), (333, 97), (16, 1), (145, 1)]
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=5)
     scale = 1.0 / math.sqrt(D)
@@ -524,7 +524,7 @@ def test_attention_reference_point_moves_late():
     seqs = [(400, 400), (300, 1)]
     for shared in (0, 1 << 30):
         ops = HipOps(dt, "cuda:0")
-        ops.SHARED_ATTENTION_WAVES = ops.SHARED_ATTENTION_MIN_WAVES = shared
+        ops.SHARED_ATTENTION_MIN_CONTEXT = ops.SHARED_ATTENTION_MIN_WAVES = shared
         qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=11)
         # key at position r has r / 2 on channel 0, queries have 1 there: the
         # score grows by 16 (23 in units of log 2) per block of 32 keys
