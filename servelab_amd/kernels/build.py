@@ -145,6 +145,23 @@ def ensure(units: Iterable[Unit], force: bool = False, verbose: bool = True) -> 
     return paths
 
 
+def prune(keep: Iterable[str], folder: Optional[str] = None) -> int:
+    """Removes the libraries in the build folder that are not in ``keep``
+    (those of older sources, which no digest names any more); returns how many."""
+    folder = folder or build_dir()
+    keep = {os.path.abspath(p) for p in keep}
+    gone = 0
+    for name in os.listdir(folder):
+        path = os.path.abspath(os.path.join(folder, name))
+        if name.endswith(".so") and path not in keep:
+            try:
+                os.remove(path)
+                gone += 1
+            except OSError:
+                pass
+    return gone
+
+
 def load(u: Unit) -> ctypes.CDLL:
     """The loaded library of a unit (compiled first when none is built)."""
     if u not in _loaded:
@@ -157,7 +174,7 @@ def load(u: Unit) -> ctypes.CDLL:
 DEFAULT_STEMS = ("elementwise", "norm", "gemm", "attention", "sampling")
 
 
-def all_units(head_dims=(16, 32, 64, 128)) -> List[Unit]:
+def all_units(head_dims=(32, 64, 96, 128, 192, 256)) -> List[Unit]:
     units = []
     for dtype in ("bfloat16", "float32"):
         for stem in DEFAULT_STEMS:
