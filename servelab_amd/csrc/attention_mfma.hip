@@ -96,6 +96,7 @@ struct AttnParams {
   float* part_o;                 // [rows, nh, nsplit, D]   (split launches)
   float* part_ml;                // [rows, nh, nsplit, 2]
   int part_row0;                 // token index of partial row 0
+  int pair;                      // prompt workgroups take a late tile and its early mirror
 };
 
 // The columns of one wavefront: queries, running maxima and sums, outputs.
@@ -344,9 +345,12 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   // A workgroup takes a late tile (many key blocks) and then the early tile
   // that mirrors it (few): every workgroup of a sequence then has about the
   // same number of blocks and none is left running alone at the end (MI355X,
-  // 7B shape: 2,048 tokens 108 -> 80 us, 8,192 tokens 807 -> 737 us).
+  // 7B shape: 2,048 tokens 108 -> 80 us, 8,192 tokens 807 -> 737 us).  A
+  // portion deep inside a long context has tiles of nearly one length already;
+  // its caller leaves them unpaired, which makes twice the workgroups.
   for (int half = 0; half < 2; ++half) {
-  if (2 * (int)blockIdx.x + half > ntiles - 1) break;       // no such tile; the whole workgroup leaves together
+  if (P.pair ? 2 * (int)blockIdx.x + half > ntiles - 1 : half > 0 || (int)blockIdx.x >= ntiles)
+    break;                                                  // no such tile; the whole workgroup leaves together
   const int tile = half == 0 ? ntiles - 1 - (int)blockIdx.x : (int)blockIdx.x;
 
   const int wg_c0 = tile * COLS;
@@ -475,12 +479,14 @@ extern "C" int sl_attention_mfma_head_dim() { return D; }
 // most max_q_len tokens.  nsplit > 1 needs part_o / part_ml for the rows
 // [part_row0, part_row0 + part_rows) these sequences own (one token each).
 // Prompt portions go to the workgroups that share keys through LDS once the
-// launch would have shared_min_waves wavefronts of 32 columns or more.
+// launch would have shared_min_waves wavefronts of 32 columns or more;
+// pair_tiles: see the kernel.
 extern "C" const char* sl_attention_mfma(
     const void* qkv, int row_stride, const void* kc, const void* vc, const int* block_tables,
     int max_pages, const int* cu_q, const int* positions, int seq_begin, int num_seqs,
     int max_q_len, int nh, int nkv, int head_dim, int page, float scale, int window, int nsplit,
-    int shared_min_waves, void* out, float* part_o, float* part_ml, int part_row0, int part_rows, hipStream_t stream) {
+    int shared_min_waves, int pair_tiles, void* out, float* part_o, float* part_ml, int part_row0, int part_rows,
+    hipStream_t stream) {
   SL_CHECK(head_dim == D, "attention_mfma: built for another head size");
   SL_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: heads must be a multiple of kv heads");
   SL_CHECK(page == 16 || page == 32 || page == 64, "attention_mfma: page size must be 16, 32 or 64");
@@ -493,7 +499,7 @@ extern "C" const char* sl_attention_mfma(
   const int g = nh / nkv;
   AttnParams P{(const __bf16*)qkv, row_stride, (const __bf16*)kc, (const __bf16*)vc, block_tables,
                max_pages, cu_q, positions, seq_begin, nh, nkv, page, scale, window, nsplit,
-               (__bf16*)out, part_o, part_ml, part_row0};
+               (__bf16*)out, part_o, part_ml, part_row0, pair_tiles};
   const long long cols = (long long)max_q_len * g;
   if (nsplit > 1) {
     SL_CHECK(max_q_len == 1, "attention_mfma: the context is split for single tokens only");
@@ -525,8 +531,9 @@ extern "C" const char* sl_attention_mfma(
   } else if (!SHARED_FITS || tiles * nkv * num_seqs < shared_min_waves) {
     attention_mfma_kernel<2, false><<<dim3((unsigned)tiles, nkv, num_seqs), 64, 0, stream>>>(P);
   } else {
-    const long long wg = (tiles + SHARED_WAVES - 1) / SHARED_WAVES;    // two tiles per workgroup
-    attention_mfma_shared_kernel<<<dim3((unsigned)((wg + 1) / 2), nkv, num_seqs), 64 * SHARED_WAVES, 0, stream>>>(P);
+    const long long wg = (tiles + SHARED_WAVES - 1) / SHARED_WAVES;
+    attention_mfma_shared_kernel<<<dim3((unsigned)(pair_tiles ? (wg + 1) / 2 : wg), nkv, num_seqs),
+                                   64 * SHARED_WAVES, 0, stream>>>(P);
   }
   return sl_launch_status();
 }

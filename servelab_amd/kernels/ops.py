@@ -730,8 +730,11 @@ class HipOps:
             waves = -(-batch.max_q_len * (nh // nkv) // 32) * nkv * n_pre
             shared = (waves >= self.SHARED_ATTENTION_MIN_WAVES and
                       batch.max_ctx_len >= self.SHARED_ATTENTION_MIN_CONTEXT)
+            # tiles of a causal triangle differ in length and are paired; those of a portion
+            # that starts deeper in its context than it is long do not
+            pair = batch.max_ctx_len < 2 * batch.max_q_len
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, 1,
-                       0 if shared else 1 << 30, _p(out), None, None, 0, 0)
+                       0 if shared else 1 << 30, int(pair), _p(out), None, None, 0, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
@@ -741,7 +744,7 @@ class HipOps:
             if nsplit > 1:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
-            self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, _p(out),
+            self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, 0, _p(out),
                        _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0)
 
     # ------------------------------------------------------------- sampling
