@@ -202,6 +202,99 @@ struct Columns {
     }
   }
 
+  // The same block with the work of the NB column tiles side by side instead
+  // of one after the other: all score products first, one check whether any
+  // reference point has to move, then probabilities and output products, so
+  // that the vector work of one tile has matrix work of the other beside it.
+  __device__ __forceinline__ void block_abreast(int kb, const bf16x8 (&kf)[2][KK], const bf16x8 (&vf)[DD],
+                                                int gq) {
+    const int kbase = kb * 32;
+    const bool edge = kb >= full_end || kb < full_begin;
+    f32x4 s0[NB], s1[NB];
+    float s[NB][8], mxs[NB];
+    bool move = false;
+    auto scores = [&](int b) {
+      s0[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+      s1[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        s0[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kk], qf[b][kk], s0[b], 0, 0, 0);
+        s1[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kk], qf[b][kk], s1[b], 0, 0, 0);
+      }
+    };
+    auto maximum = [&](int b) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s[b][j] = j < 4 ? s0[b][j] : s1[b][j - 4];
+      if (edge) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = kbase + 8 * gq + j;
+          if (key > pos_c[b] || key < lo_c[b]) s[b][j] = -INFINITY;
+        }
+      }
+      float mx = fmaxf(fmaxf(fmaxf(s[b][0], s[b][1]), fmaxf(s[b][2], s[b][3])),
+                       fmaxf(fmaxf(s[b][4], s[b][5]), fmaxf(s[b][6], s[b][7])));
+      mxs[b] = column_max(mx) * scale_log2;
+      move = move || mxs[b] > m_run[b] + LAZY;
+    };
+    // in source order the products of tile b + 1 stand before the vector work
+    // of tile b, which can then run while the matrix cores are busy
+    scores(0);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      if (b + 1 < NB) scores(b + 1);
+      maximum(b);
+    }
+    if (__builtin_expect(__any(move), 0)) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const float m_new = fmaxf(m_run[b], mxs[b]);
+        const float alpha = fast_exp2(m_run[b] - (m_new == -INFINITY ? 0.f : m_new));
+        m_run[b] = m_new;
+        l_run[b] *= alpha;
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) o[b][dd] *= alpha;
+      }
+    }
+    bf16x8 pb[NB];
+    float psum[NB];
+    auto probability = [&](int b, int j) {
+      const float neg_m = m_run[b] == -INFINITY ? 0.f : -m_run[b];
+      const float p = fast_exp2(fmaf(s[b][j], scale_log2, neg_m));
+      psum[b] += p;
+      pb[b][j] = (__bf16)p;
+    };
+    psum[0] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) probability(0, j);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      if (b + 1 < NB) psum[b + 1] = 0.f;
+#pragma unroll
+      for (int dd = 0; dd < DD; ++dd) {
+        o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb[b], o[b][dd], 0, 0, 0);
+        if (b + 1 < NB) {                        // the next tile's probabilities, spread over these products
+#pragma unroll
+          for (int j = 8 * dd / DD; j < 8 * (dd + 1) / DD; ++j) probability(b + 1, j);
+        }
+      }
+      l_run[b] += psum[b];
+    }
+    if (NB == 2) {
+      // order asked of the scheduler for the straight-line stretch above: the
+      // first tile's probabilities, then one output product of the first tile
+      // per few vector instructions of the second tile's probabilities, then
+      // the second tile's products (0x402: vector and transcendental, 0x8: matrix)
+      __builtin_amdgcn_sched_group_barrier(0x402, 30, 0);
+#pragma unroll
+      for (int dd = 0; dd < DD; ++dd) {
+        __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x402, 32 / DD, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x8, DD, 0);
+    }
+  }
+
   // lane holds column n, channels 16 dd + 4 gq + r
   template <bool SPLIT>
   __device__ __forceinline__ void store(const AttnParams& P, int q0, int split, int gq) {
@@ -426,7 +519,7 @@ void attention_mfma_shared_kernel(const AttnParams P) {
           kf[m][kk] = *(const bf16x8*)&k_lds[buf][(16 * m + n) * KS + 32 * kk + 8 * gq];
 #pragma unroll
       for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)&v_lds[buf][(16 * dd + n) * VS + 8 * gq];
-      C.block(kb, kf, vf, gq);
+      C.block_abreast(kb, kf, vf, gq);
     }
     if (more) stage_store(buf ^ 1);
     __syncthreads();                               // the other buffer is complete; this one is free
