@@ -441,10 +441,15 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   // 7B shape: 2,048 tokens 108 -> 80 us, 8,192 tokens 807 -> 737 us).  A
   // portion deep inside a long context has tiles of nearly one length already;
   // its caller leaves them unpaired, which makes twice the workgroups.
+  // Unpaired tiles of a long context may also be cut into P.nsplit shares of
+  // their key blocks, a workgroup each, whose partial results the combine
+  // kernel merges: more and shorter workgroups for a launch of few tiles.
+  const int tile_rev = P.pair ? (int)blockIdx.x : (int)blockIdx.x / P.nsplit;
+  const int split = P.pair ? 0 : (int)blockIdx.x % P.nsplit;
   for (int half = 0; half < 2; ++half) {
-  if (P.pair ? 2 * (int)blockIdx.x + half > ntiles - 1 : half > 0 || (int)blockIdx.x >= ntiles)
+  if (P.pair ? 2 * tile_rev + half > ntiles - 1 : half > 0 || tile_rev >= ntiles)
     break;                                                  // no such tile; the whole workgroup leaves together
-  const int tile = half == 0 ? ntiles - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  const int tile = half == 0 ? ntiles - 1 - tile_rev : tile_rev;
 
   const int wg_c0 = tile * COLS;
   const int c0 = wg_c0 + 16 * NB * wave;
@@ -458,7 +463,12 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   const int wg_c_last = wg_c0 + COLS - 1 < ncols - 1 ? wg_c0 + COLS - 1 : ncols - 1;
   int kmin = 0;
   if (P.window > 0 && pos0 + wg_tok_first - P.window + 1 > 0) kmin = pos0 + wg_tok_first - P.window + 1;
-  const int wg_begin = kmin / 32, wg_end = (pos0 + wg_c_last / g) / 32 + 1;
+  int wg_begin = kmin / 32, wg_end = (pos0 + wg_c_last / g) / 32 + 1;
+  if (P.nsplit > 1) {
+    const int nblk = wg_end - wg_begin, first = wg_begin;
+    wg_begin = first + (int)((long long)nblk * split / P.nsplit);
+    wg_end = first + (int)((long long)nblk * (split + 1) / P.nsplit);
+  }
 
   bf16x8 k_stage[STAGE], v_stage[STAGE];
   int pg[2];
@@ -498,11 +508,13 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   };
 
   const int last = wg_end - 1;
+  if (wg_begin < wg_end) {                           // (a share may be empty; the same for the whole workgroup)
   load_pages(wg_begin);
   stage_load(wg_begin);
   load_pages(wg_begin + 1 < last ? wg_begin + 1 : last);
   stage_store(0);
   __syncthreads();
+  }
   for (int kb = wg_begin; kb < wg_end; ++kb) {
     const int buf = (kb - wg_begin) & 1;
     const bool more = kb + 1 < wg_end;
@@ -524,7 +536,10 @@ void attention_mfma_shared_kernel(const AttnParams P) {
     if (more) stage_store(buf ^ 1);
     __syncthreads();                               // the other buffer is complete; this one is free
   }
-  if (active) C.template store<false>(P, q0, 0, gq);
+  if (active) {
+    if (P.nsplit > 1) C.template store<true>(P, q0, split, gq);
+    else C.template store<false>(P, q0, 0, gq);
+  }
   }
 }
 
@@ -594,8 +609,7 @@ extern "C" const char* sl_attention_mfma(
                max_pages, cu_q, positions, seq_begin, nh, nkv, page, scale, window, nsplit,
                (__bf16*)out, part_o, part_ml, part_row0, pair_tiles};
   const long long cols = (long long)max_q_len * g;
-  if (nsplit > 1) {
-    SL_CHECK(max_q_len == 1, "attention_mfma: the context is split for single tokens only");
+  if (nsplit > 1 && max_q_len == 1) {
     SL_CHECK(part_o != nullptr && part_ml != nullptr && part_rows == num_seqs,
              "attention_mfma: a split launch needs partial buffers for its rows");
     SL_CHECK(g <= 64, "attention_mfma: more than 64 query heads per kv head");
@@ -619,14 +633,26 @@ extern "C" const char* sl_attention_mfma(
   // the crossover.
   const long long tiles = (cols + 31) / 32;
   SL_CHECK(tiles <= 1 << 30, "attention_mfma: too many column tiles");
+  const bool shared = cols > 16 && SHARED_FITS && tiles * nkv * num_seqs >= shared_min_waves;
+  if (nsplit > 1) {
+    SL_CHECK(shared && !pair_tiles, "attention_mfma: prompt portions are split only as unpaired tiles through LDS");
+    SL_CHECK(nsplit <= 64 && part_o != nullptr && part_ml != nullptr && part_rows > 0,
+             "attention_mfma: a split launch needs partial buffers for its rows and at most 64 splits");
+  }
   if (cols <= 16) {
     attention_mfma_kernel<1, false><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);
-  } else if (!SHARED_FITS || tiles * nkv * num_seqs < shared_min_waves) {
+  } else if (!shared) {
     attention_mfma_kernel<2, false><<<dim3((unsigned)tiles, nkv, num_seqs), 64, 0, stream>>>(P);
   } else {
     const long long wg = (tiles + SHARED_WAVES - 1) / SHARED_WAVES;
-    attention_mfma_shared_kernel<<<dim3((unsigned)(pair_tiles ? (wg + 1) / 2 : wg), nkv, num_seqs),
+    attention_mfma_shared_kernel<<<dim3((unsigned)(pair_tiles ? (wg + 1) / 2 : wg * nsplit), nkv, num_seqs),
                                    64 * SHARED_WAVES, 0, stream>>>(P);
+    if (nsplit > 1) {
+      const char* e = sl_launch_status();
+      if (e) return e;
+      attention_combine_kernel<<<dim3(part_rows, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh,
+                                                                    part_row0, (__bf16*)out);
+    }
   }
   return sl_launch_status();
 }

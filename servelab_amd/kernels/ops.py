@@ -690,6 +690,11 @@ class HipOps:
     # 8,192: 737 against 1,125 us; eight prompts of 256: 23.5 against 21.6 us).
     SHARED_ATTENTION_MIN_WAVES = 1024
     SHARED_ATTENTION_MIN_CONTEXT = 1024
+    # ... and when such a launch has fewer workgroups than this and its tiles are unpaired (a portion deep
+    # in a long context), every tile is cut into shares of at least MIN_BLOCKS key blocks, at most MAX
+    PROMPT_SPLIT_WORKGROUPS = 4096
+    PROMPT_SPLIT_MIN_BLOCKS = 64
+    PROMPT_SPLIT_MAX = 8
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples
@@ -733,8 +738,17 @@ class HipOps:
             # tiles of a causal triangle differ in length and are paired; those of a portion
             # that starts deeper in its context than it is long do not
             pair = batch.max_ctx_len < 2 * batch.max_q_len
-            self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, 1,
-                       0 if shared else 1 << 30, int(pair), _p(out), None, None, 0, 0)
+            # few unpaired tiles over a long context: each is cut into shares of its keys
+            nsplit, part_o, part_ml = 1, None, None
+            if shared and not pair:
+                nsplit = max(1, min(self.PROMPT_SPLIT_MAX, batch.max_ctx_len // 32 // self.PROMPT_SPLIT_MIN_BLOCKS,
+                                    -(-self.PROMPT_SPLIT_WORKGROUPS // -(-waves // 4))))
+            if nsplit > 1:
+                part_o = self._new((n_pre_tok, nh, nsplit, D), torch.float32)
+                part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
+            self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
+                       0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
+                       n_pre_tok if nsplit > 1 else 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:

@@ -494,15 +494,23 @@ def test_paged_attention(both, nh, nkv, D, page, window):
 @pytest.mark.parametrize("nh,nkv,D,page", [(8, 1, 32, 16), (28, 4, 128, 16), (6, 2, 192, 64),
                                            (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16)])
 @pytest.mark.parametrize("window", [None, 16, 50])
-def test_prompt_attention_through_lds(nh, nkv, D, page, window):
+@pytest.mark.parametrize("form", ["paired", "unpaired", "shares"])
+def test_prompt_attention_through_lds(nh, nkv, D, page, window, form):
     """The prompt kernel whose wavefronts share each block of keys through LDS,
     forced at sizes far below its crossover: portions that end inside a
-    workgroup's 128 columns, that start deep in a context, and one-token rows."""
+    workgroup's 128 columns, that start deep in a context, and one-token rows;
+    whole prompts with late and early tiles paired in a workgroup; tiles cut
+    into shares of their keys (down to one block, some shares empty)."""
     from servelab_amd.kernels import HipOps
     dt = torch.bfloat16
     ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
     ops.SHARED_ATTENTION_MIN_CONTEXT = ops.SHARED_ATTENTION_MIN_WAVES = 0
-    seqs = [(130, 130), (277, 45), (64, 64), (200, 2), (333, 97), (16, 1), (145, 1)]
+    if form == "paired":
+        seqs = [(130, 130), (64, 64), (97, 97), (333, 333), (2, 2), (1, 1)]
+    else:
+        seqs = [(130, 130), (277, 45), (64, 64), (200, 2), (333, 97), (16, 1), (145, 1)]
+    if form == "shares":
+        ops.PROMPT_SPLIT_MIN_BLOCKS, ops.PROMPT_SPLIT_WORKGROUPS = 1, 1 << 20
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=5)
     scale = 1.0 / math.sqrt(D)
     got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
