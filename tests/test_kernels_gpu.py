@@ -156,10 +156,14 @@ def test_library_product_pads_its_rows_harmlessly():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 50, 64), (7, 1000, 3584), (16, 17, 96), (33, 200, 352), (64, 130, 1024)])
-def test_linear_skinny(M, N, K):
-    """The matrix-core few-rows kernel alone (bfloat16): ragged M and N."""
+@pytest.mark.parametrize("pairs", [False, True])
+def test_linear_skinny(M, N, K, pairs):
+    """The matrix-core few-rows kernel alone (bfloat16): ragged M and N; one
+    tile of W per workgroup (the rule's choice at these sizes) and two."""
     from servelab_amd.kernels import HipOps
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    if pairs:
+        ops._pair_tiles = lambda M, N, K: True
     x = randn(M, K, dtype=torch.bfloat16, seed=4)
     w = randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5)
     b = randn(N, seed=6)
@@ -259,10 +263,18 @@ def test_silu_mul(both):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 352, 128), (9, 192, 64), (40, 1000, 96), (70, 24, 32), (3, 12, 64)])
-def test_gated_linear(both, M, I, K):
+@pytest.mark.parametrize("pairs", [False, True])
+def test_gated_linear(both, M, I, K, pairs):
     """gate/up GEMM + silu-multiply: the fused few-rows kernel (bfloat16, blocks
-    of 8) and the two-kernel path, against the plain product with separate halves."""
+    of 8; one tile of W per workgroup and two) and the two-kernel path, against
+    the plain product with separate halves."""
     ops, emu, dt = both
+    if pairs:
+        if dt != torch.bfloat16:
+            pytest.skip("tiles of W are a matter of the bfloat16 kernels")
+        from servelab_amd.kernels import HipOps
+        ops = HipOps(dt, "cuda:0")
+        ops._pair_tiles = lambda M, N, K: True
     x = randn(M, K, dtype=dt, seed=1)
     gate, up = randn(I, K, dtype=dt, scale=0.2, seed=2), randn(I, K, dtype=dt, scale=0.2, seed=3)
     ref = emu.silu_mul(emu.linear(x, torch.cat([gate, up]), None))
@@ -277,14 +289,18 @@ def test_gated_linear(both, M, I, K):
 
 
 @pytest.mark.parametrize("M,H,N2", [(1, 64, 96), (8, 3584, 4608), (16, 200 * 32, 48), (5, 96, 1000)])
-def test_fused_add_norm_around_few_rows_products(M, H, N2):
+@pytest.mark.parametrize("pairs", [False, True])
+def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs):
     """A deferred product run by the norm that adds it (stream += x W1^T, rows
     left un-normalised, sums of squares by workgroup) and the products that
     read such rows (plain with bias, gated, float output with a row gather):
-    same results as product, add, norm and product one after the other."""
+    same results as product, add, norm and product one after the other; with
+    one tile of W per workgroup and with two."""
     from servelab_amd.kernels import HipOps
     from servelab_amd.kernels.ops import Deferred, ScaledRows
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    if pairs:
+        ops._pair_tiles = lambda M, N, K: True
     K1 = 128
     x = randn(M, K1, dtype=torch.bfloat16, seed=1)
     w1 = ops.prepare_weight(randn(H, K1, dtype=torch.bfloat16, scale=0.1, seed=2))
@@ -397,14 +413,18 @@ def test_rope_store_from_partial_sums(both, nh, nkv, D, page):
 
 @pytest.mark.parametrize("M", [1, 8, 16, 40])
 @pytest.mark.parametrize("nh,nkv,D,page,H", [(4, 2, 16, 16, 64), (28, 4, 128, 16, 256), (5, 1, 48, 32, 96)])
-def test_qkv_rope_store(M, nh, nkv, D, page, H):
+@pytest.mark.parametrize("pairs", [False, True])
+def test_qkv_rope_store(M, nh, nkv, D, page, H, pairs):
     """Product + rotation + cache write: the one fused kernel (at most 16 rows)
     and the product followed by rope_store give the same q, K pages and V
-    pages; also with un-normalised input rows and with no rotation or no write."""
+    pages; also with un-normalised input rows and with no rotation or no write;
+    with one tile of W per workgroup and with two."""
     from servelab_amd.kernels import HipOps
     from servelab_amd.kernels.ops import ScaledRows
     dt = torch.bfloat16
     ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+    if pairs:
+        ops._pair_tiles = lambda M, N, K: True
     N = (nh + 2 * nkv) * D
     x = randn(M, H, dtype=dt, seed=1)
     w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.1, seed=2))
