@@ -30,6 +30,7 @@ def parse_args(argv=None):
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--max-live", type=int, default=16, help="most requests live at a time")
     return ap.parse_args(argv)
 
 
@@ -41,7 +42,7 @@ def run(args, stdin=sys.stdin, stdout=sys.stdout, ops=None) -> int:
     _, model = load_model_on_device(args.model, args.dtype, args.device, ops=ops)
     page = args.block_size
     num_pages = max(1, -(-args.max_tokens // page))
-    runner = make_runner(model, num_pages, page, max_num_seqs=16)
+    runner = make_runner(model, num_pages, page, max_num_seqs=max(1, getattr(args, "max_live", 16)))
     for line in stdin:
         line = line.strip()
         if not line:

@@ -38,10 +38,10 @@ def tolerance(dtype, reference):
 
 
 def replay_in_process(folder, steps, out_dir, dtype, max_tokens, ops=None, device="cuda:0",
-                      block_size=16):
+                      block_size=16, max_live=16):
     from servelab_amd.replay import run
     args = argparse.Namespace(model=folder, dtype=dtype, out=out_dir, max_tokens=max_tokens,
-                              block_size=block_size, device=device)
+                              block_size=block_size, device=device, max_live=max_live)
     stdin = io.StringIO("".join(json.dumps(s) + "\n" for s in steps))
     stdout = io.StringIO()
     assert run(args, stdin, stdout, ops=ops) == 0

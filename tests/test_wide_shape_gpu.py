@@ -48,3 +48,53 @@ def test_wide_shape_matches_plain(tmp_path, wide, dtype):
     worst, where = compare(out, steps, reference, 152064)
     print(f"wide {dtype}: max abs err {worst:.3e} at {where}")
     assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
+
+
+@pytest.fixture(scope="module")
+def crowd(wide):
+    """One long request and 39 short ones, with the tokens they will be fed."""
+    folder, _, _ = wide
+    rng = random.Random(2)
+    decoded = {"L": 11}
+    decoded.update({f"s{i}": 8 if i < 7 else 5 if i < 15 else 2 for i in range(39)})
+    requests = {"L": [rng.randrange(152064) for _ in range(1400 + decoded["L"])]}
+    for i in range(39):
+        requests[f"s{i}"] = [rng.randrange(152064) for _ in range(4 + i % 5 + decoded[f"s{i}"])]
+    return folder, requests, decoded, plain_logits(folder, requests)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_wide_shape_long_prompt_and_growing_batches(tmp_path, crowd, dtype):
+    """What only serving sizes reach: a prompt of 1,400 tokens in one step (the
+    library products and the prompt attention that shares keys through LDS, in
+    bfloat16), then decode steps of 1, 8, 16 and 40 requests (every form of the
+    few-rows products, decode attention over a split context beside short
+    ones), with the newcomers' prompts beside the decoded tokens."""
+    folder, requests, decoded, reference = crowd
+    fed = {r: 0 for r in requests}
+    steps = []
+
+    def take(r, n):
+        toks = requests[r][fed[r]:fed[r] + n]
+        fed[r] += n
+        return {"id": r, "tokens": toks, "want": [n - 1]}
+
+    def step(entries):
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+
+    live = ["L"]
+    step([take("L", 1400)])
+    for newcomers in ([], [f"s{i}" for i in range(7)], [f"s{i}" for i in range(7, 15)],
+                      [f"s{i}" for i in range(15, 39)]):
+        if newcomers:
+            step([take(r, len(requests[r]) - decoded[r]) for r in newcomers] + [take(r, 1) for r in live])
+            live += newcomers
+        step([take(r, 1) for r in live])
+        step([take(r, 1) for r in live])
+    assert all(fed[r] == len(requests[r]) for r in requests)
+    steps[-1]["end"] = list(requests)
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, dtype, rs.max_tokens_needed(steps), max_live=40)
+    worst, where = compare(out, steps, reference, 152064)
+    print(f"wide, long prompt and batches, {dtype}: max abs err {worst:.3e} at {where}")
+    assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
