@@ -137,6 +137,179 @@ __global__ __launch_bounds__(64) void attention_general_combine_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Prompt portions, general sizes.  The kernel above gives a wavefront to every
+// (token, head) and lets it read its keys from the cache itself: for a prompt
+// of thousands of tokens every key row is fetched thousands of times.  Here a
+// workgroup of four wavefronts owns TILE_COLS columns, a column being a (token,
+// head of the group) pair of one sequence and one kv head, and walks the key
+// blocks its columns see: a block of KB keys and values is staged in LDS as
+// floats once and serves all columns; 16 lanes share a column, splitting a
+// block's keys for the scores and the head's channels for the output.  Float
+// FMAs only, running maximum and sum per column as above.
+// ---------------------------------------------------------------------------
+constexpr int TILE_COLS = 16;
+constexpr int TILE_THREADS = 256;
+
+template <int KB>
+__global__ __launch_bounds__(TILE_THREADS) void attention_general_tile_kernel(
+    const act_t* __restrict__ qkv, int row_stride, const act_t* __restrict__ kc,
+    const act_t* __restrict__ vc, const int* __restrict__ block_tables, int max_pages,
+    const int* __restrict__ cu_q, const int* __restrict__ positions, int nh, int nkv, int D,
+    int page, float scale, int window, act_t* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int KS = D + 4, VS = D + 1;                  // row strides: K rows are read 16 bytes at a time, by 16 rows at once
+  float* qs = lds;                                   // [TILE_COLS][D]
+  float* ks = qs + TILE_COLS * D;                    // [KB][KS]
+  float* vs = ks + KB * KS;                          // [KB][VS]
+  float* ps = vs + KB * VS;                          // [TILE_COLS][KB]
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int sub = lane & 15;                         // this lane's place among the 16 of its column
+  const int col = 4 * wave + (lane >> 4);            // column of the tile
+  const int seq = blockIdx.z, kvh = blockIdx.y;
+  const int g = nh / nkv;
+  const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0;
+  const int ncols = qlen * g;
+  const int c0 = blockIdx.x * TILE_COLS;
+  if (c0 >= ncols) return;
+  const int pos0 = positions[q0];
+  const int* table = block_tables + (size_t)seq * max_pages;
+
+  // the tile's columns and the keys any of them sees
+  const int c = c0 + col;
+  const bool live = c < ncols;
+  const int tok = live ? c / g : 0, head = kvh * g + (live ? c % g : 0);
+  const int pos_c = live ? pos0 + tok : -1;
+  const int lo_c = window > 0 && pos_c - window + 1 > 0 ? pos_c - window + 1 : 0;
+  const int tok_first = c0 / g;
+  const int c_last = c0 + TILE_COLS - 1 < ncols - 1 ? c0 + TILE_COLS - 1 : ncols - 1;
+  const int kmax = pos0 + c_last / g;
+  int kmin = 0;
+  if (window > 0 && pos0 + tok_first - window + 1 > 0) kmin = pos0 + tok_first - window + 1;
+
+  for (int idx = t; idx < TILE_COLS * D; idx += TILE_THREADS) {
+    const int cc = c0 + idx / D, d = idx % D;
+    qs[idx] = cc < ncols ? to_f(qkv[(size_t)(q0 + cc / g) * row_stride + (size_t)(kvh * g + cc % g) * D + d]) : 0.f;
+  }
+
+  float m = -INFINITY, l = 0.f;
+  float acc[MAX_D / 16];
+#pragma unroll
+  for (int j = 0; j < MAX_D / 16; ++j) acc[j] = 0.f;
+  const int nd16 = D / 16;
+
+  for (int kb = kmin / KB; kb <= kmax / KB; ++kb) {
+    const int kbase = kb * KB;
+    __syncthreads();                                 // the last block's readers are done (and qs is written)
+    for (int idx = t; idx < KB * D; idx += TILE_THREADS) {
+      {                                              // K: consecutive threads along a key's channels
+        const int key = kbase + idx / D, d = idx % D;
+        float v = 0.f;
+        if (key >= kmin && key <= kmax) {
+          const int pg = table[key / page];
+          v = to_f(kc[(((size_t)pg * nkv + kvh) * page + key % page) * D + d]);
+        }
+        ks[(idx / D) * KS + d] = v;
+      }
+      {                                              // V^T in the cache: consecutive threads along a channel's keys
+        const int kk = idx % KB, d = idx / KB, key = kbase + kk;
+        float v = 0.f;
+        if (key >= kmin && key <= kmax) {
+          const int pg = table[key / page];
+          v = to_f(vc[(((size_t)pg * nkv + kvh) * D + d) * page + key % page]);
+        }
+        vs[kk * VS + d] = v;
+      }
+    }
+    __syncthreads();
+    // scores of this lane's keys sub, sub + 16, ... of the block
+    float sc[KB / 16];
+#pragma unroll
+    for (int r = 0; r < KB / 16; ++r) sc[r] = 0.f;
+    const float* qrow = qs + col * D;
+    for (int d = 0; d < D; d += 4) {
+      const float4 q4 = *(const float4*)(qrow + d);
+#pragma unroll
+      for (int r = 0; r < KB / 16; ++r) {
+        const float4 k4 = *(const float4*)(ks + (sub + 16 * r) * KS + d);
+        sc[r] += q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < KB / 16; ++r) {
+      const int key = kbase + sub + 16 * r;
+      sc[r] = key >= lo_c && key <= pos_c ? sc[r] * scale : -INFINITY;
+      mx = fmaxf(mx, sc[r]);
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float mn = fmaxf(m, mx);
+    // a column that has seen no key yet keeps m = -inf: nothing to rescale, nothing to add
+    const float alpha = mn == -INFINITY ? 1.f : expf(m - mn);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < KB / 16; ++r) {
+      const float pr = sc[r] == -INFINITY ? 0.f : expf(sc[r] - mn);
+      psum += pr;
+      ps[col * KB + sub + 16 * r] = pr;
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) psum += __shfl_xor(psum, o, 64);
+    l = l * alpha + psum;
+    m = mn;
+    __syncthreads();                                 // ps is complete
+#pragma unroll
+    for (int j = 0; j < MAX_D / 16; ++j) acc[j] *= alpha;
+    const float* prow = ps + col * KB;
+    for (int kk = 0; kk < KB; ++kk) {
+      const float pk = prow[kk];
+      const float* vrow = vs + kk * VS + sub;
+#pragma unroll
+      for (int j = 0; j < MAX_D / 16; ++j)
+        if (j < nd16) acc[j] += pk * vrow[16 * j];
+    }
+  }
+  if (!live) return;
+  const float inv = 1.f / l;
+  act_t* o = out + ((size_t)(q0 + tok) * nh + head) * D + sub;
+#pragma unroll
+  for (int j = 0; j < MAX_D / 16; ++j)
+    if (j < nd16) o[16 * j] = from_f<act_t>(acc[j] * inv);
+}
+
+// Sequences [0, num_seqs) of the batch, prompt portions of at most max_q_len
+// tokens each (their tokens come first in the batch).  D % 16 == 0.
+extern "C" const char* sl_attention_general_tiles(
+    const void* qkv, int row_stride, const void* kc, const void* vc, const int* block_tables,
+    int max_pages, const int* cu_q, const int* positions, int num_seqs, int max_q_len, int nh,
+    int nkv, int D, int page, float scale, int window, void* out, hipStream_t stream) {
+  SL_CHECK(num_seqs >= 0 && max_q_len >= 1 && nh > 0 && nkv > 0 && nh % nkv == 0,
+           "attention tiles: heads must be a positive multiple of kv heads");
+  SL_CHECK(D > 0 && D <= MAX_D && D % 16 == 0, "attention tiles: head_dim must be a multiple of 16 up to 256");
+  SL_CHECK(page == 16 || page == 32 || page == 64, "attention tiles: page size must be 16, 32 or 64");
+  SL_CHECK(nkv <= 65535 && num_seqs <= 65535, "attention tiles: grid too large");
+  SL_CHECK(window >= 0, "attention tiles: window must be >= 0 (0 = none)");
+  if (num_seqs == 0) return nullptr;
+  const long long cols = (long long)max_q_len * (nh / nkv);
+  const long long tiles = (cols + TILE_COLS - 1) / TILE_COLS;
+  SL_CHECK(tiles <= 1 << 30, "attention tiles: too many column tiles");
+  const dim3 grid((unsigned)tiles, nkv, num_seqs);
+  const int KB = D <= 128 ? 32 : 16;
+  const size_t bytes = sizeof(float) * ((size_t)TILE_COLS * D + (size_t)KB * (D + 4) + (size_t)KB * (D + 1) +
+                                        (size_t)TILE_COLS * KB);
+  SL_CHECK(bytes <= 65536, "attention tiles: LDS need exceeds 64 KB");
+  if (KB == 32)
+    attention_general_tile_kernel<32><<<grid, TILE_THREADS, bytes, stream>>>(
+        (const act_t*)qkv, row_stride, (const act_t*)kc, (const act_t*)vc, block_tables, max_pages,
+        cu_q, positions, nh, nkv, D, page, scale, window, (act_t*)out);
+  else
+    attention_general_tile_kernel<16><<<grid, TILE_THREADS, bytes, stream>>>(
+        (const act_t*)qkv, row_stride, (const act_t*)kc, (const act_t*)vc, block_tables, max_pages,
+        cu_q, positions, nh, nkv, D, page, scale, window, (act_t*)out);
+  return sl_launch_status();
+}
+
 // nsplit > 1: part_o holds T * nh * nsplit * D floats, part_ml T * nh * nsplit * 2.
 extern "C" const char* sl_attention_general(
     const void* qkv, int row_stride, const void* kc, const void* vc, const int* block_tables,

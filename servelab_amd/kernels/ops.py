@@ -668,18 +668,34 @@ class HipOps:
             self._attention_mfma(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
                                  batch, scale, window, out)
             return out
+        stride = (nh + 2 * nkv) * D
+        first = 0                         # tokens before this one are done
+        n_pre, n_pre_tok = batch.num_prefill_seqs, batch.num_prefill_tokens
+        if n_pre and D % 16 == 0 and batch.max_q_len > 1:
+            # prompt portions (they come first in the batch): workgroups that stage each block of keys
+            # once for 16 columns, instead of a wavefront per (token, head) that reads its own
+            self._check(batch.cu_q, torch.int32, (batch.num_seqs + 1,), "cu_q")
+            self._call("attention", "sl_attention_general_tiles", _p(qkv), stride, _p(k_cache),
+                       _p(v_cache), _p(block_tables), max_pages, _p(batch.cu_q), _p(batch.positions),
+                       n_pre, batch.max_q_len, nh, nkv, D, page_size, _c_float(scale),
+                       int(window or 0), _p(out))
+            first = n_pre_tok
+        rest = T - first
+        if rest == 0:
+            return out
         # few tokens (a decode step): the keys of every (token, head) are shared out over several
         # wavefronts; the count depends on the number of tokens only, so that a captured step and an
         # eager one add up in the same order
-        nsplit = 1 if batch.max_q_len > 1 else max(1, min(64, self.GENERAL_ATTENTION_WAVES // (T * nh)))
+        single = first > 0 or batch.max_q_len == 1
+        nsplit = max(1, min(64, self.GENERAL_ATTENTION_WAVES // (rest * nh))) if single else 1
         part_o = part_ml = None
         if nsplit > 1:
-            part_o = self._new((T, nh, nsplit, D), torch.float32)
-            part_ml = self._new((T, nh, nsplit, 2), torch.float32)
-        self._call("attention", "sl_attention_general", _p(qkv), (nh + 2 * nkv) * D, _p(k_cache),
-                   _p(v_cache), _p(block_tables), max_pages, _p(batch.tok_seq),
-                   _p(batch.positions), T, nh, nkv, D, page_size, _c_float(scale),
-                   int(window or 0), _p(out), nsplit, _p(part_o), _p(part_ml))
+            part_o = self._new((rest, nh, nsplit, D), torch.float32)
+            part_ml = self._new((rest, nh, nsplit, 2), torch.float32)
+        self._call("attention", "sl_attention_general", _p(qkv[first:]), stride, _p(k_cache),
+                   _p(v_cache), _p(block_tables), max_pages, _p(batch.tok_seq[first:]),
+                   _p(batch.positions[first:]), rest, nh, nkv, D, page_size, _c_float(scale),
+                   int(window or 0), _p(out[first:]), nsplit, _p(part_o), _p(part_ml))
         return out
 
     GENERAL_ATTENTION_WAVES = 4096  # the general kernel's decode launches aim for this many wavefronts
