@@ -163,6 +163,117 @@ extern "C" const char* sl_gemm_tiled(const void* x, const void* w, const float* 
   return sl_launch_status();
 }
 
+// ------------------------------------- float32 products on the matrix cores
+#if defined(SL_F32)
+// y = x W^T in float32 for many rows: v_mfma_f32_32x32x2_f32 multiplies and adds
+// float32 values as they are (no reduced-precision inputs, float32 sums), at
+// twice the rate the vector ALU reaches without packed instructions.  A
+// workgroup of four wavefronts owns 128 rows of x by 128 rows of W, a wavefront
+// 64 x 64 of it as 2 x 2 tiles of 32 x 32; chunks of 16 values of k go through
+// double-buffered LDS (rows padded to 17 floats: the 32 rows one operand read
+// touches fall into 32 banks).  K % 16 == 0.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int FM = 128, FN = 128, FK = 16, FS = FK + 1;
+
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
+    float* __restrict__ y, int M, int N, int K) {
+  __shared__ float xs[2][FM * FS];
+  __shared__ float ws[2][FN * FS];
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * FM, n0 = blockIdx.x * FN;
+  // loader: thread t brings rows t / 4 and t / 4 + 64 of both tiles, 4 values of k from (t % 4) * 4;
+  // rows past the end load the last row (never stored)
+  const int lr = t >> 2, lk = (t & 3) * 4;
+  const float* xp[2];
+  const float* wp[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = m0 + lr + 64 * i < M ? m0 + lr + 64 * i : M - 1;
+    const int n = n0 + lr + 64 * i < N ? n0 + lr + 64 * i : N - 1;
+    xp[i] = x + (size_t)m * K + lk;
+    wp[i] = w + (size_t)n * K + lk;
+  }
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  float4 xr[2], wr[2];
+  auto load = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      xr[i] = *(const float4*)(xp[i] + k0);
+      wr[i] = *(const float4*)(wp[i] + k0);
+    }
+  };
+  auto store = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      float* xd = &xs[buf][(lr + 64 * i) * FS + lk];
+      float* wd = &ws[buf][(lr + 64 * i) * FS + lk];
+      xd[0] = xr[i].x; xd[1] = xr[i].y; xd[2] = xr[i].z; xd[3] = xr[i].w;
+      wd[0] = wr[i].x; wd[1] = wr[i].y; wd[2] = wr[i].z; wd[3] = wr[i].w;
+    }
+  };
+  const int nchunks = K / FK;
+  load(0);
+  store(0);
+  __syncthreads();
+  // operand element of this lane in a 32 x 2 step: row lane % 32, k lane / 32
+  const int orow = lane & 31, ok = lane >> 5;
+  for (int c = 0; c < nchunks; ++c) {
+    const int buf = c & 1;
+    if (c + 1 < nchunks) load((c + 1) * FK);
+    const float* xa = &xs[buf][(wm * 64 + orow) * FS + ok];
+    const float* wb = &ws[buf][(wn * 64 + orow) * FS + ok];
+#pragma unroll
+    for (int kk = 0; kk < FK; kk += 2) {
+      const float a0 = xa[kk], a1 = xa[32 * FS + kk];
+      const float b0 = wb[kk], b1 = wb[32 * FS + kk];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+    if (c + 1 < nchunks) store(buf ^ 1);
+    __syncthreads();
+  }
+  // element r of a tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn * 64 + 32 * j + (lane & 31);
+    if (n >= N) continue;
+    const float b = bias != nullptr ? bias[n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < M) y[(size_t)m * N + n] = acc[i][j][r] + b;
+      }
+  }
+}
+
+extern "C" const char* sl_gemm_f32_mfma(const void* x, const void* w, const float* bias, void* y,
+                                        int M, int N, int K, hipStream_t stream) {
+  SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_f32_mfma: sizes must be positive");
+  SL_CHECK(K % FK == 0, "gemm_f32_mfma: K must be a multiple of 16");
+  SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
+           "gemm_f32_mfma: x and W must be 16-byte aligned");
+  if (M == 0) return nullptr;
+  const dim3 grid((N + FN - 1) / FN, (M + FM - 1) / FM);
+  SL_CHECK(grid.y <= 65535, "gemm_f32_mfma: more than 65535 row tiles");
+  gemm_f32_mfma_kernel<<<grid, 256, 0, stream>>>((const float*)x, (const float*)w, bias, (float*)y,
+                                                 M, N, K);
+  return sl_launch_status();
+}
+#endif
+
 // ------------------------------------------------ few rows on the matrix cores
 #if !defined(SL_F32)
 // y[M, N] for M <= 64 in bfloat16: bound by streaming W from HBM once.

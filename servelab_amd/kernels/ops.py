@@ -342,6 +342,8 @@ class HipOps:
         if self.act_dtype == torch.float32:
             if K % 4 == 0 and M <= self.ROWS_KERNEL_MAX_M:
                 return self.linear_rows(x, weight.w, bias, out_f32)
+            if K % 16 == 0 and M >= self.F32_MFMA_MIN_M:
+                return self.linear_f32_mfma(x, weight.w, bias)
             return self.linear_tiled(x, weight.w, bias, out_f32)
         limit = self._few_rows_limit(weight)
         if (defer and self.fuse_norms and not out_f32 and self.WIDE_MIN_M <= M <= limit
@@ -498,6 +500,19 @@ class HipOps:
         if M >= self.LIBRARY_PADDED_MAX_M:
             return M
         return -(-M // self.LIBRARY_ROW_STEP) * self.LIBRARY_ROW_STEP
+
+    F32_MFMA_MIN_M = 33           # float32 products of this many rows or more run on the matrix cores
+
+    def linear_f32_mfma(self, x, w, bias):
+        """Float32 product by float32 matrix instructions (float32 inputs and sums,
+        no reduced-precision mode); K % 16 == 0."""
+        if self.act_dtype != torch.float32:
+            raise KernelError("linear_f32_mfma is for the float32 table only")
+        M, K = x.shape
+        N = w.shape[0]
+        y = self._new((M, N), torch.float32)
+        self._call("gemm", "sl_gemm_f32_mfma", _p(x), _p(w), _p(bias), _p(y), M, N, K)
+        return y
 
     def linear_library(self, x, w, bias):
         if self.act_dtype != torch.bfloat16:

@@ -766,3 +766,22 @@ def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
     many = randn(300, K, dtype=torch.bfloat16, seed=4)
     got = ops.linear(many, weight, b, out_f32=True)
     assert got.shape == (300, N) and rel_err(got, emu.linear(many, w, b, True)) < 2e-5
+
+
+@pytest.mark.parametrize("M,N,K", [(33, 200, 64), (128, 128, 16), (300, 1000, 352), (2048, 3584, 3584), (130, 70, 1024)])
+def test_float32_product_on_the_matrix_cores(M, N, K):
+    """Float32 products of many rows (v_mfma_f32_32x32x2_f32): against float64 as
+    exact as the plain FMA kernel's float32 sums of K terms (a reduced-precision
+    matrix mode would be a thousand times off); ragged edges of both tiles."""
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.float32, "cuda:0")
+    x, w, b = randn(M, K, seed=1), randn(N, K, scale=0.1, seed=2), randn(N, seed=3)
+    ref = (x.double() @ w.double().T + b.double())
+    for bias in (None, b):
+        got = ops.linear_f32_mfma(x, w, bias)
+        want = ref if bias is not None else ref - b.double()
+        assert got.dtype == torch.float32 and got.shape == (M, N)
+        err = ((got.double() - want).abs().max() / want.abs().max()).item()
+        plain = ((ops.linear_tiled(x, w, bias).double() - want).abs().max() / want.abs().max()).item()
+        assert err < max(1.5 * plain, 1e-6), (err, plain)
+        assert torch.equal(got, ops.linear(x, w, bias))          # the float32 table's choice at these sizes
