@@ -9,7 +9,8 @@ bounds can take the GPU down.
 Large bfloat16 matrix products (more rows than the hand-written few-rows
 kernel takes) go to the library GEMM behind ``torch.addmm`` — where the
 reference calls ``F.linear`` (servelab/parallel/layers.py:164-180).  The
-float32 table never does: its products are the hand-written FMA kernels.
+float32 table never does: its products are the hand-written float32 kernels
+(FMA, and float32 matrix instructions for many rows).
 """
 import contextlib
 import ctypes
