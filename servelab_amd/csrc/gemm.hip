@@ -168,56 +168,78 @@ extern "C" const char* sl_gemm_tiled(const void* x, const void* w, const float* 
 // y = x W^T in float32 for many rows: v_mfma_f32_32x32x2_f32 multiplies and adds
 // float32 values as they are (no reduced-precision inputs, float32 sums), at
 // twice the rate the vector ALU reaches without packed instructions.  A
-// workgroup of four wavefronts owns 128 rows of x by 128 rows of W, a wavefront
-// 64 x 64 of it as 2 x 2 tiles of 32 x 32; chunks of 16 values of k go through
+// workgroup of four wavefronts owns a tile of x rows by W rows, a wavefront its
+// part of it as tiles of 32 x 32; chunks of 16 values of k go through
 // double-buffered LDS (rows padded to 17 floats: the 32 rows one operand read
 // touches fall into 32 banks).  K % 16 == 0.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-constexpr int FM = 128, FN = 128, FK = 16, FS = FK + 1;
+constexpr int FK = 16, FS = FK + 1;
 
+// WM x WN wavefronts (four in all), each TI x TJ tiles of 32 x 32: a workgroup
+// owns 32 TI WM rows of x by 32 TJ WN rows of W.  <2, 2, 2, 2>: 128 x 128 for
+// many rows; <1, 1, 1, 4>: 32 x 128 up to 64 rows (7B shape, 64 rows: a decode
+// step of 95 ms against 129 ms with the large tiles and 175 ms with the FMA
+// tiles; at 8 rows the wavefront-per-column kernel is twice as fast as either:
+// 8 KB of W per barrier is too little in flight to stream it).
+template <int TI, int TJ, int WM, int WN>
 __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(
     const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
     float* __restrict__ y, int M, int N, int K) {
+  static_assert(WM * WN == 4, "four wavefronts");
+  constexpr int FM = 32 * TI * WM, FN = 32 * TJ * WN;
+  constexpr int XL = (FM * 4 + 255) / 256, WL = (FN * 4 + 255) / 256;    // 16-byte loads a thread makes per chunk
   __shared__ float xs[2][FM * FS];
   __shared__ float ws[2][FN * FS];
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int m0 = blockIdx.y * FM, n0 = blockIdx.x * FN;
-  // loader: thread t brings rows t / 4 and t / 4 + 64 of both tiles, 4 values of k from (t % 4) * 4;
+  // loader: 16-byte piece idx of a tile is row idx / 4, values of k from (idx % 4) * 4;
   // rows past the end load the last row (never stored)
-  const int lr = t >> 2, lk = (t & 3) * 4;
-  const float* xp[2];
-  const float* wp[2];
+  const float* xp[XL];
+  const float* wp[WL];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int m = m0 + lr + 64 * i < M ? m0 + lr + 64 * i : M - 1;
-    const int n = n0 + lr + 64 * i < N ? n0 + lr + 64 * i : N - 1;
-    xp[i] = x + (size_t)m * K + lk;
-    wp[i] = w + (size_t)n * K + lk;
+  for (int i = 0; i < XL; ++i) {
+    const int idx = t + 256 * i, r = idx / 4 < FM ? idx / 4 : FM - 1;
+    const int m = m0 + r < M ? m0 + r : M - 1;
+    xp[i] = x + (size_t)m * K + (idx & 3) * 4;
   }
-  f32x16 acc[2][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WL; ++i) {
+    const int idx = t + 256 * i, r = idx / 4 < FN ? idx / 4 : FN - 1;
+    const int n = n0 + r < N ? n0 + r : N - 1;
+    wp[i] = w + (size_t)n * K + (idx & 3) * 4;
+  }
+  f32x16 acc[TI][TJ];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-  float4 xr[2], wr[2];
+  float4 xr[XL], wr[WL];
   auto load = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      xr[i] = *(const float4*)(xp[i] + k0);
-      wr[i] = *(const float4*)(wp[i] + k0);
-    }
+    for (int i = 0; i < XL; ++i) xr[i] = *(const float4*)(xp[i] + k0);
+#pragma unroll
+    for (int i = 0; i < WL; ++i) wr[i] = *(const float4*)(wp[i] + k0);
   };
   auto store = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      float* xd = &xs[buf][(lr + 64 * i) * FS + lk];
-      float* wd = &ws[buf][(lr + 64 * i) * FS + lk];
-      xd[0] = xr[i].x; xd[1] = xr[i].y; xd[2] = xr[i].z; xd[3] = xr[i].w;
-      wd[0] = wr[i].x; wd[1] = wr[i].y; wd[2] = wr[i].z; wd[3] = wr[i].w;
+    for (int i = 0; i < XL; ++i) {
+      const int idx = t + 256 * i;
+      if (idx < FM * 4) {
+        float* d = &xs[buf][(idx / 4) * FS + (idx & 3) * 4];
+        d[0] = xr[i].x; d[1] = xr[i].y; d[2] = xr[i].z; d[3] = xr[i].w;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {
+      const int idx = t + 256 * i;
+      if (idx < FN * 4) {
+        float* d = &ws[buf][(idx / 4) * FS + (idx & 3) * 4];
+        d[0] = wr[i].x; d[1] = wr[i].y; d[2] = wr[i].z; d[3] = wr[i].w;
+      }
     }
   };
   const int nchunks = K / FK;
@@ -229,32 +251,36 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(
   for (int c = 0; c < nchunks; ++c) {
     const int buf = c & 1;
     if (c + 1 < nchunks) load((c + 1) * FK);
-    const float* xa = &xs[buf][(wm * 64 + orow) * FS + ok];
-    const float* wb = &ws[buf][(wn * 64 + orow) * FS + ok];
+    const float* xa = &xs[buf][(wm * 32 * TI + orow) * FS + ok];
+    const float* wb = &ws[buf][(wn * 32 * TJ + orow) * FS + ok];
 #pragma unroll
     for (int kk = 0; kk < FK; kk += 2) {
-      const float a0 = xa[kk], a1 = xa[32 * FS + kk];
-      const float b0 = wb[kk], b1 = wb[32 * FS + kk];
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+      float a[TI], b[TJ];
+#pragma unroll
+      for (int i = 0; i < TI; ++i) a[i] = xa[32 * i * FS + kk];
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) b[j] = wb[32 * j * FS + kk];
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
     }
     if (c + 1 < nchunks) store(buf ^ 1);
     __syncthreads();
   }
   // element r of a tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn * 64 + 32 * j + (lane & 31);
+  for (int j = 0; j < TJ; ++j) {
+    const int n = n0 + (wn * TJ + j) * 32 + (lane & 31);
     if (n >= N) continue;
-    const float b = bias != nullptr ? bias[n] : 0.f;
+    const float bv = bias != nullptr ? bias[n] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m < M) y[(size_t)m * N + n] = acc[i][j][r] + b;
+        const int m = m0 + (wm * TI + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < M) y[(size_t)m * N + n] = acc[i][j][r] + bv;
       }
   }
 }
@@ -266,10 +292,15 @@ extern "C" const char* sl_gemm_f32_mfma(const void* x, const void* w, const floa
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
            "gemm_f32_mfma: x and W must be 16-byte aligned");
   if (M == 0) return nullptr;
-  const dim3 grid((N + FN - 1) / FN, (M + FM - 1) / FM);
+  const int rows = M <= 64 ? 32 : 128;
+  const dim3 grid((N + 127) / 128, (M + rows - 1) / rows);
   SL_CHECK(grid.y <= 65535, "gemm_f32_mfma: more than 65535 row tiles");
-  gemm_f32_mfma_kernel<<<grid, 256, 0, stream>>>((const float*)x, (const float*)w, bias, (float*)y,
-                                                 M, N, K);
+  if (M <= 64)
+    gemm_f32_mfma_kernel<1, 1, 1, 4><<<grid, 256, 0, stream>>>((const float*)x, (const float*)w, bias,
+                                                              (float*)y, M, N, K);
+  else
+    gemm_f32_mfma_kernel<2, 2, 2, 2><<<grid, 256, 0, stream>>>((const float*)x, (const float*)w, bias,
+                                                              (float*)y, M, N, K);
   return sl_launch_status();
 }
 #endif

@@ -502,7 +502,7 @@ class HipOps:
             return M
         return -(-M // self.LIBRARY_ROW_STEP) * self.LIBRARY_ROW_STEP
 
-    F32_MFMA_MIN_M = 33           # float32 products of this many rows or more run on the matrix cores
+    F32_MFMA_MIN_M = 17           # float32 products of this many rows or more run on the matrix cores
 
     def linear_f32_mfma(self, x, w, bias):
         """Float32 product by float32 matrix instructions (float32 inputs and sums,

@@ -768,7 +768,8 @@ def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
     assert got.shape == (300, N) and rel_err(got, emu.linear(many, w, b, True)) < 2e-5
 
 
-@pytest.mark.parametrize("M,N,K", [(33, 200, 64), (128, 128, 16), (300, 1000, 352), (2048, 3584, 3584), (130, 70, 1024)])
+@pytest.mark.parametrize("M,N,K", [(2, 130, 48), (8, 3584, 3584), (33, 200, 64), (64, 100, 96), (65, 100, 96),
+                                   (128, 128, 16), (300, 1000, 352), (2048, 3584, 3584), (130, 70, 1024)])
 def test_float32_product_on_the_matrix_cores(M, N, K):
     """Float32 products of many rows (v_mfma_f32_32x32x2_f32): against float64 as
     exact as the plain FMA kernel's float32 sums of K terms (a reduced-precision
@@ -784,4 +785,5 @@ def test_float32_product_on_the_matrix_cores(M, N, K):
         err = ((got.double() - want).abs().max() / want.abs().max()).item()
         plain = ((ops.linear_tiled(x, w, bias).double() - want).abs().max() / want.abs().max()).item()
         assert err < max(1.5 * plain, 1e-6), (err, plain)
-        assert torch.equal(got, ops.linear(x, w, bias))          # the float32 table's choice at these sizes
+        if M >= ops.F32_MFMA_MIN_M:
+            assert torch.equal(got, ops.linear(x, w, bias))      # the float32 table's choice at these sizes
