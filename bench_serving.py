@@ -132,6 +132,7 @@ def summarise(done: list, elapsed: float, ttft_slo_ms: float, tpot_slo_ms: float
 
 def build_engine(args):
     from servelab_amd import CacheConfig, LLMEngine, SchedulerConfig, load_config
+    from servelab_amd.cli import tune_option
     cache = CacheConfig(block_size=args.block_size, num_blocks=args.num_blocks or None,
                         gpu_memory_utilization=args.gpu_memory_utilization)
     sched = SchedulerConfig(max_num_seqs=args.max_num_seqs,
@@ -140,11 +141,11 @@ def build_engine(args):
                             policy=args.scheduler_policy)
     if args.model:
         cfg = load_config(args.model)
-        return cfg, LLMEngine(cfg, cache, sched, dtype=args.dtype, tune_products=args.tune_products)
+        return cfg, LLMEngine(cfg, cache, sched, dtype=args.dtype, tune_products=tune_option(args))
     import bench                                     # random weights of a named shape, made on the device
     cfg, model, _ = bench.build(argparse.Namespace(shape=args.shape, layers=args.layers,
                                                    dtype=args.dtype, seed=args.seed))
-    return cfg, LLMEngine(cfg, cache, sched, model=model, tune_products=args.tune_products)
+    return cfg, LLMEngine(cfg, cache, sched, model=model, tune_products=tune_option(args))
 
 
 def run(args) -> dict:
@@ -209,6 +210,7 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--warmup-requests", type=int, default=4,
                     help="short requests run before the clock starts (0 = none)")
     ap.add_argument("--tune-products", action="store_true")
+    ap.add_argument("--tune-rows", default="", help="further step sizes (rows) to tune the library products for")
     return ap
 
 

@@ -45,7 +45,16 @@ def build_parser():
     ap.add_argument("--tune-products", action="store_true",
                     help="at start-up, time the library's matrix kernels for a full-budget step "
                          "and keep the fastest (bfloat16 only)")
+    ap.add_argument("--tune-rows", default="",
+                    help="comma-separated further step sizes (rows) to time them for, e.g. typical "
+                         "prompt lengths; implies --tune-products")
     return ap
+
+
+def tune_option(args):
+    """What ``LLMEngine(tune_products=...)`` takes: False, True, or the further row counts."""
+    rows = [int(n) for n in args.tune_rows.split(",") if n.strip()] if getattr(args, "tune_rows", "") else []
+    return rows if rows else bool(args.tune_products)
 
 
 def main(argv=None) -> int:
@@ -84,7 +93,7 @@ def main(argv=None) -> int:
         mc, CacheConfig(block_size=args.block_size, num_blocks=args.num_blocks or None),
         SchedulerConfig(max_num_seqs=args.max_num_seqs,
                         max_num_batched_tokens=args.max_batched_tokens),
-        seed=args.seed, tokenizer=tokenizer, dtype=args.dtype, tune_products=args.tune_products)
+        seed=args.seed, tokenizer=tokenizer, dtype=args.dtype, tune_products=tune_option(args))
     if args.prompt_ids:
         prompts = [[int(t) for t in args.prompt_ids.split(",")]]
     elif tokenizer is not None:

@@ -48,4 +48,4 @@ class EngineConfig:
     seed: int = 1234
     dtype: str = "auto"                    # auto (config.json's torch_dtype) | bfloat16 | float32
     device: str = "cuda:0"
-    tune_products: bool = False            # time the library's kernels for full-budget steps at start-up
+    tune_products: object = False          # True, or further row counts: time the library's kernels at start-up

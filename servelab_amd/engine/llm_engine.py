@@ -24,10 +24,11 @@ class LLMEngine:
                  scheduler_config: Optional[SchedulerConfig] = None, seed: int = 1234,
                  device: str = "cuda:0", tokenizer=None,
                  clock: Optional[Callable[[], float]] = None, dtype: str = "auto",
-                 model=None, ops=None, tune_products: bool = False):
+                 model=None, ops=None, tune_products=False):
         """``model_config.path`` names the model folder (as in the reference,
         servelab/engine/engine.py:86-87); ``model`` may pass an already loaded
-        DecoderModel instead."""
+        DecoderModel instead.  ``tune_products``: True, or a list of further
+        step sizes (rows) to time the library's matrix kernels for."""
         self.model_config = model_config
         self.cache_config = cache_config or CacheConfig()
         self.scheduler_config = scheduler_config or SchedulerConfig()
@@ -53,6 +54,10 @@ class LLMEngine:
             # a step that uses its whole token budget is the common large step under load;
             # decode steps of more requests than the few-rows kernels take are library products too
             rows = [self.scheduler_config.max_num_batched_tokens]
+            if not isinstance(tune_products, bool):
+                # further row counts the caller expects often (typical prompt lengths): the
+                # library's choices hold for exactly the shapes that were timed
+                rows += [int(n) for n in tune_products]
             library_rows = getattr(model.rt.ops, "library_rows", None)
             if library_rows is not None:
                 first = model.rt.ops.SKINNY_MAX_M + 1
