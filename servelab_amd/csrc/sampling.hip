@@ -238,7 +238,7 @@ constexpr int CUT_MAX_CHUNKS = 64;
 
 struct CutState {                          // what the rounds so far know of a row's cut
   uint64_t mass_above;                     // mass of the logits above every pattern that begins with `prefix`
-  uint64_t target;                         // top-p: top_p * the row's whole mass (known after round 0)
+  uint64_t target;                         // top-p: top_p * the row's whole mass (known once the first digit is counted)
   uint32_t prefix;                         // the leading bytes of the cut's pattern
   uint32_t count_above;
   float xmax;
