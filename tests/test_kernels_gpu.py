@@ -787,3 +787,30 @@ def test_float32_product_on_the_matrix_cores(M, N, K):
         assert err < max(1.5 * plain, 1e-6), (err, plain)
         if M >= ops.F32_MFMA_MIN_M:
             assert torch.equal(got, ops.linear(x, w, bias))      # the float32 table's choice at these sizes
+
+
+@pytest.mark.parametrize("N,K", [(200, 96), (1000, 352), (2560, 3584)])
+def test_products_at_every_boundary_of_the_row_counts(N, K):
+    """ops.linear / gated_linear / deferred products at each row count where the
+    bfloat16 table changes kernels (few-rows, wide, LDS-staged, padded library),
+    for a small, a medium and a large matrix: always the plain product."""
+    from servelab_amd.kernels import HipOps
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    w = randn(N, K, dtype=torch.bfloat16, scale=0.05, seed=2)
+    weight, b = ops.prepare_weight(w), randn(N, seed=3)
+    gain = 1 + 0.1 * randn(N, seed=4)
+    for M in (1, 8, 9, 16, 17, 32, 33, 64, 65, 96, 97, 128, 129, 160, 511, 512, 513):
+        x = randn(M, K, dtype=torch.bfloat16, seed=M)
+        ref = emu.linear(x, w, b, True)
+        assert rel_err(ops.linear(x, weight, b), ref) < 2 ** -7, M
+        assert rel_err(ops.linear(x, weight, b, out_f32=True), ref) < 2 ** -7, M
+        assert rel_err(ops.materialize(ops.linear(x, weight, b, defer=True)), ref) < 2 ** -7, M
+        if N % 16 == 0:
+            assert rel_err(ops.gated_linear(x, weight, 8), emu.silu_mul(emu.linear(x, w, None), 8)) < 2 ** -6, M
+        # a deferred product through the norm that adds it
+        resid = randn(M, N, seed=5)
+        want = resid + ref
+        got = ops.add_rmsnorm(resid, ops.linear(x, weight, b, defer=True), gain, 1e-6)
+        assert rel_err(resid, want) < 2 ** -7, M
+        normed = want * torch.rsqrt(want.pow(2).mean(-1, keepdim=True) + 1e-6) * gain
+        assert rel_err(got, normed) < 2 ** -6, M
