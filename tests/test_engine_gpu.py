@@ -254,3 +254,38 @@ def test_decode_graphs_of_a_hundred_requests():
     for i in range(4):
         alone = runner.step([StepEntry("solo", [(7 * i + 17) % 4096], [0])])[0]
         assert (alone - runs[True][i, 17]).abs().max().item() < 0.05 * alone.abs().max().item()
+
+
+def test_many_requests_under_three_regimes_generate_the_same_tokens(tmp_path):
+    """Sixty requests of random lengths, float32, greedy: with room for all, with
+    a fifth of the pages (preemption and recomputation) and with few requests
+    and small portions at a time, every request generates the same tokens; no
+    page is left held."""
+    folder = make_folder(tmp_path, "B", seed=41)
+    vocab = TINY["B"]["vocab_size"]
+    rng = random.Random(12)
+    prompts = [[rng.randrange(vocab) for _ in range(max(1, int(rng.gauss(60, 35))))] for _ in range(60)]
+    lengths = [max(1, int(rng.gauss(20, 9))) for _ in prompts]
+    need = sum(-(-(len(p) + n) // 16) for p, n in zip(prompts, lengths))
+    results = {}
+    for name, seqs, budget, blocks in (("roomy", 32, 512, need + 8), ("tight", 32, 128, need // 5),
+                                       ("narrow", 4, 24, need // 3)):
+        eng = LLMEngine(load_config(folder), CacheConfig(num_blocks=blocks),
+                        SchedulerConfig(max_num_seqs=seqs, max_num_batched_tokens=budget), dtype="float32")
+        ids = [eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(n))
+               for p, n in zip(prompts, lengths)]
+        done = {}
+        while eng.has_unfinished():
+            for o in eng.step():
+                done[o.request_id] = o
+        eng.runner.manager.check()
+        stats = eng.stats()
+        assert set(stats["pages_in_use"]) == {0}
+        results[name] = [done[i].outputs[0].token_ids for i in ids]
+        # EOS may end a request early; otherwise it has its number of tokens
+        assert all(len(t) == n or done[i].outputs[0].finish_reason == "eos"
+                   for t, n, i in zip(results[name], lengths, ids))
+        if name == "tight":
+            assert stats["num_preemptions_total"] > 0
+    assert results["tight"] == results["roomy"]
+    assert results["narrow"] == results["roomy"]
