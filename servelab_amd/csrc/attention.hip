@@ -111,6 +111,120 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
   }
 }
 
+// The same for up to GROUP_HEADS query heads of one kv head at a time: a decode
+// row's heads of a group read the same keys and values, so one wavefront takes
+// them together and every key row and value column is fetched once for all of
+// them (the kernel above fetches it once per head).
+constexpr int GROUP_HEADS = 8;
+
+__global__ __launch_bounds__(64) void attention_general_group_kernel(
+    const act_t* __restrict__ qkv, int row_stride, const act_t* __restrict__ kc,
+    const act_t* __restrict__ vc, const int* __restrict__ block_tables, int max_pages,
+    const int* __restrict__ tok_seq, const int* __restrict__ positions, int nh, int nkv, int D,
+    int page, float scale, int window, act_t* __restrict__ out, int nsplit,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+  __shared__ float qs[GROUP_HEADS][MAX_D];
+  __shared__ float ps[GROUP_HEADS][64];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const int g = nh / nkv, chunks = (g + GROUP_HEADS - 1) / GROUP_HEADS;
+  const int kvh = blockIdx.y / chunks, h0 = kvh * g + (blockIdx.y % chunks) * GROUP_HEADS;
+  const int nheads = kvh * g + g - h0 < GROUP_HEADS ? kvh * g + g - h0 : GROUP_HEADS;
+  const int s = tok_seq[t], p = positions[t];
+  const int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  const int* table = block_tables + (size_t)s * max_pages;
+  for (int idx = lane; idx < GROUP_HEADS * D; idx += 64)      // rows past nheads: zeros, results never stored
+    qs[idx / D][idx % D] = idx / D < nheads
+        ? to_f(qkv[(size_t)t * row_stride + (size_t)(h0 + idx / D) * D + idx % D]) : 0.f;
+  __syncthreads();
+
+  float m[GROUP_HEADS], l[GROUP_HEADS], acc[GROUP_HEADS][MAX_D / 64];
+#pragma unroll
+  for (int h = 0; h < GROUP_HEADS; ++h) {
+    m[h] = -INFINITY;
+    l[h] = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAX_D / 64; ++i) acc[h][i] = 0.f;
+  }
+  const int first = lo / 64, nblk = p / 64 + 1 - first;
+  const int b0 = first + (int)((long long)nblk * blockIdx.z / nsplit);
+  const int b1 = first + (int)((long long)nblk * (blockIdx.z + 1) / nsplit);
+  for (int kb = b0 * 64; kb < b1 * 64; kb += 64) {
+    const int r = kb + lane;
+    const bool valid = r >= lo && r <= p;
+    float dot[GROUP_HEADS];
+#pragma unroll
+    for (int h = 0; h < GROUP_HEADS; ++h) dot[h] = 0.f;
+    if (valid) {
+      const int pg = table[r / page];
+      const act_t* kr = kc + (((size_t)pg * nkv + kvh) * page + r % page) * D;
+      for (int d = 0; d < D; ++d) {
+        const float kv = to_f(kr[d]);
+#pragma unroll
+        for (int h = 0; h < GROUP_HEADS; ++h) dot[h] += qs[h][d] * kv;
+      }
+    }
+    float alpha[GROUP_HEADS];
+#pragma unroll
+    for (int h = 0; h < GROUP_HEADS; ++h) {
+      const float sc = valid ? dot[h] * scale : -INFINITY;
+      const float mn = fmaxf(m[h], wave_max(sc));  // every block holds a visible key
+      alpha[h] = expf(m[h] - mn);                  // exp(-inf) = 0 on the first block
+      const float pr = valid ? expf(sc - mn) : 0.f;
+      l[h] = l[h] * alpha[h] + wave_sum(pr);
+      m[h] = mn;
+      ps[h][lane] = pr;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < GROUP_HEADS; ++h)
+#pragma unroll
+      for (int i = 0; i < MAX_D / 64; ++i) acc[h][i] *= alpha[h];
+    for (int pb = 0; pb < 64; pb += page) {
+      const int r0 = kb + pb;
+      if (r0 > p) break;
+      if (r0 + page <= lo) continue;               // wholly before the window: may be released
+      const int pg = table[r0 / page];
+      const act_t* vbase = vc + ((size_t)pg * nkv + kvh) * D * page;
+#pragma unroll
+      for (int i = 0; i < MAX_D / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) {
+          const act_t* vr = vbase + (size_t)d * page;
+          for (int j = 0; j < page; ++j) {
+            const float v = to_f(vr[j]);
+#pragma unroll
+            for (int h = 0; h < GROUP_HEADS; ++h) acc[h][i] += ps[h][pb + j] * v;
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int h = 0; h < GROUP_HEADS; ++h) {
+    if (h >= nheads) break;
+    const size_t row = (size_t)t * nh + h0 + h;
+    if (nsplit > 1) {
+#pragma unroll
+      for (int i = 0; i < MAX_D / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) part_o[(row * nsplit + blockIdx.z) * D + d] = acc[h][i];
+      }
+      if (lane == 0) {
+        part_ml[(row * nsplit + blockIdx.z) * 2] = m[h];
+        part_ml[(row * nsplit + blockIdx.z) * 2 + 1] = l[h];
+      }
+    } else {
+      const float inv = 1.f / l[h];
+#pragma unroll
+      for (int i = 0; i < MAX_D / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) out[row * D + d] = from_f<act_t>(acc[h][i] * inv);
+      }
+    }
+  }
+}
+
 // out[t, h, :] = sum_j w_j o_j / sum_j w_j l_j,  w_j = exp(m_j - max m); a share
 // without keys has m = -inf and l = 0 and drops out.  One wavefront per (t, h).
 __global__ __launch_bounds__(64) void attention_general_combine_kernel(
@@ -326,9 +440,17 @@ extern "C" const char* sl_attention_general(
   SL_CHECK(nsplit == 1 || (part_o != nullptr && part_ml != nullptr),
            "attention: shares of the keys need the partial buffers");
   if (T == 0) return nullptr;
-  attention_general_kernel<<<dim3(T, nh, nsplit), 64, 0, stream>>>(
-      (const act_t*)qkv, row_stride, (const act_t*)kc, (const act_t*)vc, block_tables, max_pages,
-      tok_seq, positions, nh, nkv, D, page, scale, window, (act_t*)out, nsplit, part_o, part_ml);
+  const int g = nh / nkv;
+  if (g > 1) {                                       // the heads of a group together
+    const int chunks = (g + GROUP_HEADS - 1) / GROUP_HEADS;
+    attention_general_group_kernel<<<dim3(T, nkv * chunks, nsplit), 64, 0, stream>>>(
+        (const act_t*)qkv, row_stride, (const act_t*)kc, (const act_t*)vc, block_tables, max_pages,
+        tok_seq, positions, nh, nkv, D, page, scale, window, (act_t*)out, nsplit, part_o, part_ml);
+  } else {
+    attention_general_kernel<<<dim3(T, nh, nsplit), 64, 0, stream>>>(
+        (const act_t*)qkv, row_stride, (const act_t*)kc, (const act_t*)vc, block_tables, max_pages,
+        tok_seq, positions, nh, nkv, D, page, scale, window, (act_t*)out, nsplit, part_o, part_ml);
+  }
   const char* e = sl_launch_status();
   if (e || nsplit == 1) return e;
   attention_general_combine_kernel<<<dim3(T, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh, D,

@@ -703,7 +703,9 @@ class HipOps:
         # wavefronts; the count depends on the number of tokens only, so that a captured step and an
         # eager one add up in the same order
         single = first > 0 or batch.max_q_len == 1
-        nsplit = max(1, min(64, self.GENERAL_ATTENTION_WAVES // (rest * nh))) if single else 1
+        group = nh // nkv                 # a wavefront takes up to 8 heads of a group together
+        per_token = nkv * -(-group // 8) if group > 1 else nh
+        nsplit = max(1, min(64, self.GENERAL_ATTENTION_WAVES // (rest * per_token))) if single else 1
         part_o = part_ml = None
         if nsplit > 1:
             part_o = self._new((rest, nh, nsplit, D), torch.float32)
