@@ -582,6 +582,8 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
 }
 
 extern "C" int sl_attention_mfma_head_dim() { return D; }
+// whether this head size has the prompt kernel that shares keys through LDS (its buffers fit)
+extern "C" int sl_attention_mfma_shares_keys() { return SHARED_FITS ? 1 : 0; }
 
 // One launch over sequences [seq_begin, seq_begin + num_seqs), all with at
 // most max_q_len tokens.  nsplit > 1 needs part_o / part_ml for the rows

@@ -768,7 +768,8 @@ class HipOps:
         if n_pre:
             waves = -(-batch.max_q_len * (nh // nkv) // 32) * nkv * n_pre
             shared = (waves >= self.SHARED_ATTENTION_MIN_WAVES and
-                      batch.max_ctx_len >= self.SHARED_ATTENTION_MIN_CONTEXT)
+                      batch.max_ctx_len >= self.SHARED_ATTENTION_MIN_CONTEXT and
+                      bool(self._lib[lib].sl_attention_mfma_shares_keys()))
             # tiles of a causal triangle differ in length and are paired; those of a portion
             # that starts deeper in its context than it is long do not
             pair = batch.max_ctx_len < 2 * batch.max_q_len

@@ -513,7 +513,8 @@ def test_paged_attention(both, nh, nkv, D, page, window):
 
 
 @pytest.mark.parametrize("nh,nkv,D,page", [(8, 1, 32, 16), (28, 4, 128, 16), (6, 2, 192, 64),
-                                           (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16)])
+                                           (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16),
+                                           (4, 2, 256, 16)])     # 256: no LDS form; the same calls take the other kernel
 @pytest.mark.parametrize("window", [None, 16, 50])
 @pytest.mark.parametrize("form", ["paired", "unpaired", "shares"])
 def test_prompt_attention_through_lds(nh, nkv, D, page, window, form):
