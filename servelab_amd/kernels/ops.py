@@ -729,6 +729,7 @@ class HipOps:
     PROMPT_SPLIT_WORKGROUPS = 4096
     PROMPT_SPLIT_MIN_BLOCKS = 64
     PROMPT_SPLIT_MAX = 8
+    PROMPT_SPLIT_BYTES = 512 << 20   # ... and no more shares than keep the partial outputs below this
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples
@@ -777,7 +778,8 @@ class HipOps:
             nsplit, part_o, part_ml = 1, None, None
             if shared and not pair:
                 nsplit = max(1, min(self.PROMPT_SPLIT_MAX, batch.max_ctx_len // 32 // self.PROMPT_SPLIT_MIN_BLOCKS,
-                                    -(-self.PROMPT_SPLIT_WORKGROUPS // -(-waves // 4))))
+                                    -(-self.PROMPT_SPLIT_WORKGROUPS // -(-waves // 4)),
+                                    self.PROMPT_SPLIT_BYTES // (n_pre_tok * nh * D * 4)))
             if nsplit > 1:
                 part_o = self._new((n_pre_tok, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
