@@ -12,10 +12,10 @@ import torch
 from ..config import CacheConfig, SchedulerConfig
 from ..sampling import Sampler
 from .batch import StepEntry
-from .output import RequestOutput
+from .output import RequestOutput, result_of
 from .sampling_params import SamplingParams
 from .scheduler import Scheduler
-from .sequence import Sequence
+from .request import Request
 from .session import load_model_on_device, make_runner
 
 
@@ -68,8 +68,7 @@ class LLMEngine:
                                    eos_token_id=model.spec.eos_token_id,
                                    max_positions=model.spec.max_position_embeddings)
         self.sampler = Sampler(model.rt.ops, self.device, seed)
-        self._req_counter = 0
-        self._draws: Dict[str, int] = {}
+        self._submitted = 0
         self.num_steps = 0
 
     # -------------------------------------------------------------- intake
@@ -86,11 +85,11 @@ class LLMEngine:
         bad = [t for t in prompt_token_ids if not 0 <= int(t) < vocab]
         if bad:
             raise ValueError(f"token id {bad[0]} is outside the vocabulary of {vocab}")
-        self._req_counter += 1
-        request_id = request_id or f"req-{self._req_counter}"
-        seq = Sequence(request_id, list(prompt_token_ids), sampling_params or SamplingParams(),
-                       priority=priority, arrival_time=self.clock(), number=self._req_counter)
-        self.scheduler.add_request(seq)
+        self._submitted += 1
+        request_id = request_id or f"req-{self._submitted}"
+        self.scheduler.add_request(Request(
+            request_id, prompt_token_ids, sampling_params or SamplingParams(), priority=priority,
+            arrived=self.clock(), number=self._submitted))
         return request_id
 
     def abort_request(self, request_id: str) -> bool:
@@ -105,59 +104,51 @@ class LLMEngine:
         requests that finished (or were aborted) in this step
         (servelab/engine/engine.py:169-241)."""
         plan = self.scheduler.schedule()
-        outputs = [RequestOutput.from_sequence(s, self._detokenize) for s in plan.aborted]
+        outputs = [result_of(r, self._to_text) for r in plan.aborted]
         if plan.is_empty():
             if not outputs and self.scheduler.has_unfinished():
                 raise RuntimeError("nothing can be scheduled although requests are unfinished")
             return outputs
-        entries: List[StepEntry] = []
-        sampling: List[Sequence] = []
-        for ps in plan.prefills:                 # prompt portions first, then decode tokens
-            seq, start, n = ps.seq, ps.num_computed, ps.num_new_tokens
-            last = start + n == seq.prefill_target
-            entries.append(StepEntry(seq.request_id, seq.token_ids[start:start + n],
-                                     [n - 1] if last else []))
-            if last:
-                sampling.append(seq)
-            seq.num_computed_tokens = start + n
-        for seq in plan.decodes:
-            entries.append(StepEntry(seq.request_id, [seq.token_ids[-1]], [0]))
-            sampling.append(seq)
-            seq.num_computed_tokens = seq.get_len()      # this token's cache is written below
+        items = plan.items()                     # portions first, then single tokens
+        entries = [StepEntry(it.request.request_id, it.token_ids,
+                             [it.count - 1] if it.samples else []) for it in items]
+        drawing = [it.request for it in items if it.samples]
         logits = self.runner.step(entries)
-        tokens = self.sampler.sample(
-            logits, [s.sampling_params for s in sampling], [s.number for s in sampling],
-            [s.num_output_tokens for s in sampling])
-        sampled = {s.request_id: t for s, t in zip(sampling, tokens)}
-        finished = self.scheduler.update_after_exec(sampled, now=self.clock())
+        tokens = self.sampler.sample(logits, [r.params for r in drawing],
+                                     [r.number for r in drawing], [r.num_output for r in drawing])
+        finished = self.scheduler.complete(
+            plan, {r.request_id: t for r, t in zip(drawing, tokens)}, now=self.clock())
         self.num_steps += 1
-        return outputs + [RequestOutput.from_sequence(s, self._detokenize) for s in finished]
+        return outputs + [result_of(r, self._to_text) for r in finished]
 
-    def _detokenize(self, token_ids: List[int]) -> str:
-        return "" if self.tokenizer is None else self.tokenizer.decode(token_ids)
+    @property
+    def _to_text(self):
+        return self.tokenizer.decode if self.tokenizer is not None else None
 
     # ------------------------------------------------------------ generate
+    def run(self, on_step: Optional[Callable[[dict], None]] = None):
+        """Steps until nothing is unfinished, yielding each result as its
+        request ends; ``on_step`` is called with ``stats()`` after every step."""
+        while self.has_unfinished():
+            yield from self.step()
+            if on_step is not None:
+                on_step(self.stats())
+
     def generate(self, prompts: List, sampling_params: Optional[SamplingParams] = None,
                  verbose: bool = False) -> List[RequestOutput]:
-        """Offline generation; prompts are strings (needs a tokenizer) or lists
-        of token ids; outputs come back in input order
-        (servelab/engine/engine.py:249-270)."""
+        """Offline generation of a batch of prompts — strings (needs a tokenizer)
+        or lists of token ids — all with the same parameters; results in the
+        order of the prompts (the call of servelab/engine/engine.py:249-270).
+        ``verbose`` prints a line of queue and cache figures per step."""
         params = sampling_params or SamplingParams()
-        ids = []
-        for p in prompts:
-            ids.append(self.add_request(
-                prompt=p if isinstance(p, str) else None,
-                prompt_token_ids=None if isinstance(p, str) else list(p),
-                sampling_params=params))
-        results: Dict[str, RequestOutput] = {}
-        while self.has_unfinished():
-            for out in self.step():
-                results[out.request_id] = out
-            if verbose:
-                st = self.scheduler.stats()
-                print(f"[step] running={st['running']} waiting={st['waiting']} "
-                      f"cache={st['gpu_cache_usage']:.0%}")
-        return [results.get(i) for i in ids]
+        order = [self.add_request(p, params) if isinstance(p, str)
+                 else self.add_request(None, params, prompt_token_ids=list(p)) for p in prompts]
+
+        def line(st):
+            print(f"[step {st['steps']}] running={st['running']} waiting={st['waiting']} "
+                  f"cache={st['gpu_cache_usage']:.0%}", flush=True)
+        done = {out.request_id: out for out in self.run(line if verbose else None)}
+        return [done.get(rid) for rid in order]
 
     def stats(self) -> dict:
         return {**self.scheduler.stats(), **self.runner.manager.stats(),

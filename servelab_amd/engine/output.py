@@ -1,8 +1,7 @@
-"""Result records (servelab/engine/output.py:9-41)."""
+"""Result records (servelab/engine/output.py:9-41): the field names callers of
+the reference read."""
 from dataclasses import dataclass, field
-from typing import List, Optional
-
-from .sequence import Sequence
+from typing import Callable, List, Optional
 
 
 @dataclass
@@ -22,11 +21,11 @@ class RequestOutput:
     finished: bool = False
     metrics: Optional[dict] = None
 
-    @classmethod
-    def from_sequence(cls, seq: Sequence, detokenize=None) -> "RequestOutput":
-        reason = seq.status.value.replace("FINISHED_", "").lower() if seq.is_finished() else None
-        out = CompletionOutput(index=0, token_ids=list(seq.output_token_ids), finish_reason=reason)
-        if detokenize is not None:
-            out.text = detokenize(out.token_ids)
-        return cls(request_id=seq.request_id, prompt_token_ids=list(seq.prompt_token_ids),
-                   outputs=[out], finished=seq.is_finished(), metrics=seq.metrics.to_dict())
+
+def result_of(req, to_text: Optional[Callable[[List[int]], str]] = None) -> RequestOutput:
+    """The record of a request as it stands (usually: finished)."""
+    generated = list(req.output)
+    completion = CompletionOutput(token_ids=generated, finish_reason=req.finish_reason,
+                                  text=to_text(generated) if to_text else "")
+    return RequestOutput(req.request_id, prompt_token_ids=list(req.prompt), outputs=[completion],
+                         finished=req.done, metrics=req.times.report())

@@ -1,5 +1,6 @@
-"""Sampling parameters of a request: the reference's names, meanings, defaults
-and validation (servelab/engine/sampling_params.py:6-28)."""
+"""How a request's tokens are drawn.  Field names, meanings and defaults are
+the reference's (servelab/engine/sampling_params.py:6-14); every field is
+checked at construction and all faults are reported in one message."""
 from dataclasses import dataclass
 from typing import Tuple
 
@@ -15,15 +16,15 @@ class SamplingParams:
     stop_token_ids: Tuple[int, ...] = ()
 
     def __post_init__(self):
-        if self.temperature < 0.0:
-            raise ValueError("temperature must be >= 0")
-        if not 0.0 < self.top_p <= 1.0:
-            raise ValueError("top_p must be in (0, 1]")
-        if self.top_k != -1 and self.top_k < 1:
-            raise ValueError("top_k must be -1 or >= 1")
-        if self.max_tokens < 1:
-            raise ValueError("max_tokens must be >= 1")
-        self.stop_token_ids = tuple(self.stop_token_ids)
+        self.stop_token_ids = tuple(int(t) for t in self.stop_token_ids)
+        faults = [f"{name}={value!r} ({rule})" for name, value, ok, rule in (
+            ("temperature", self.temperature, self.temperature >= 0.0, "negative"),
+            ("top_p", self.top_p, 0.0 < self.top_p <= 1.0, "outside (0, 1]"),
+            ("top_k", self.top_k, self.top_k == -1 or self.top_k >= 1, "neither -1 nor positive"),
+            ("max_tokens", self.max_tokens, self.max_tokens >= 1, "below 1"),
+        ) if not ok]
+        if faults:
+            raise ValueError("SamplingParams: " + "; ".join(faults))
 
     @staticmethod
     def greedy(max_tokens: int = 16) -> "SamplingParams":

@@ -1,70 +1,91 @@
 """Continuous batching with chunked prefill and recompute preemption (no tensors).
 
 Reference: ``Scheduler`` (servelab/engine/scheduler.py:107-369).  One pass per
-step under a token budget: first one decode token for every running request
-whose prompt is cached (:176-188), then the next portion of prompts that are
-part-way (:190-198), then admission from the waiting queue in policy order
-until a request does not fit (:201-241).  Pages are reserved while planning.
+step under a token budget: one token for every active request that is owed
+only its newest token (:176-188), then the next portion of requests that are
+owed more (:190-198), then admission from the queue in policy order until a
+request does not fit (:201-241).  Pages are reserved while planning, and the
+scheduler itself books the outcome of the step (``complete``): how much more
+of each request is cached, the sampled tokens, who is finished.
 
 What happens when pages run out (reference :276-316, with these decisions):
-  * a running request that cannot grow takes the pages of the request that the
+  * an active request that cannot grow takes the pages of the request that the
     policy would schedule last and that has nothing planned in this step; the
-    victim's cache is dropped, it returns to the front of the waiting queue and
-    is computed again from its first token (generated tokens included).  The
-    reference preempts one victim and leaves the failing request out of the
-    step; here the request tries again until it fits or no victim is left.
+    victim's cache is dropped, it returns to the front of the queue and is owed
+    everything it holds (generated tokens included).  The reference preempts
+    one victim and leaves the failing request out of the step; here the request
+    tries again until it fits or no victim is left.
   * with no victim left the request preempts itself.
-  * a waiting request never evicts a running one: admission simply stops
+  * a queued request never evicts an active one: admission simply stops
     (head-of-line blocking, reference :231-237).
   * a request that could not fit in the whole pool, or is longer than the
     model's positions, is aborted at admission (reference :211-215) and — unlike
     there — is reported with finish reason "aborted".
+  * with ``chunked_prefill`` off, whole prompts go before decode tokens
+    (reference :177), but only while a prompt can in fact be admitted: when
+    every slot is taken or the head of the queue does not fit, the active
+    requests decode on, which is what frees the room.  (The reference plans
+    nothing in that case and stops for good.)
 """
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional
 
 from ..config import SchedulerConfig
-from .sequence import Sequence, SequenceStatus
+from .request import ACTIVE, QUEUED, Request
 
 
 # ------------------------------------------------------------------ policies
-def fcfs_key(seq: Sequence):
+def fcfs_key(req: Request):
     """First come first served (servelab/engine/scheduler.py:37-41); ties by
     submission number rather than by the id string."""
-    return (seq.arrival_time, seq.number)
+    return (req.times.arrived, req.number)
 
 
-def priority_key(seq: Sequence):
+def priority_key(req: Request):
     """Smaller priority value first (servelab/engine/scheduler.py:44-48)."""
-    return (seq.priority, seq.arrival_time, seq.number)
+    return (req.priority, req.times.arrived, req.number)
 
 
 POLICIES = {"fcfs": fcfs_key, "priority": priority_key}
 
 
 @dataclass
-class PrefillSched:
-    seq: Sequence
-    num_new_tokens: int          # portion size
-    num_computed: int            # tokens cached before this portion
+class Planned:
+    """``count`` tokens of ``request`` from position ``start`` on run in this step."""
+    request: Request
+    start: int
+    count: int
+
+    @property
+    def samples(self) -> bool:
+        """Whether the step's last logits of this request are its next token."""
+        return self.start + self.count == len(self.request.tokens)
+
+    @property
+    def token_ids(self) -> List[int]:
+        return self.request.tokens[self.start:self.start + self.count]
 
 
 @dataclass
-class SchedulerOutput:
-    prefills: List[PrefillSched] = field(default_factory=list)
-    decodes: List[Sequence] = field(default_factory=list)
+class Plan:
+    portions: List[Planned] = field(default_factory=list)     # requests owed more than a token
+    decodes: List[Planned] = field(default_factory=list)      # one token each
     preempted: List[str] = field(default_factory=list)
-    aborted: List[Sequence] = field(default_factory=list)
+    aborted: List[Request] = field(default_factory=list)
 
     def is_empty(self) -> bool:
-        return not self.prefills and not self.decodes
+        return not self.portions and not self.decodes
 
     @property
-    def num_batched_tokens(self) -> int:
-        return sum(p.num_new_tokens for p in self.prefills) + len(self.decodes)
+    def num_tokens(self) -> int:
+        return sum(p.count for p in self.portions) + len(self.decodes)
+
+    def items(self) -> List[Planned]:
+        """Everything that runs, in the order the step function wants it."""
+        return self.portions + self.decodes
 
     def planned_ids(self):
-        return {p.seq.request_id for p in self.prefills} | {s.request_id for s in self.decodes}
+        return {p.request.request_id for p in self.items()}
 
 
 class Scheduler:
@@ -76,150 +97,161 @@ class Scheduler:
         self.eos_token_id = eos_token_id
         self.max_positions = max_positions
         self.key = POLICIES[config.policy]
-        self.waiting: List[Sequence] = []
-        self.running: List[Sequence] = []
+        self.queue: List[Request] = []
+        self.active: List[Request] = []
         self.num_preemptions = 0
 
     # -------------------------------------------------------------- intake
-    def add_request(self, seq: Sequence) -> None:
-        self.waiting.append(seq)
+    def add_request(self, req: Request) -> None:
+        self.queue.append(req)
 
     def abort_request(self, request_id: str) -> bool:
         """servelab/engine/scheduler.py:132-144."""
-        for queue in (self.waiting, self.running):
-            for i, s in enumerate(queue):
-                if s.request_id == request_id:
-                    queue.pop(i)
+        for held in (self.queue, self.active):
+            for i, r in enumerate(held):
+                if r.request_id == request_id:
+                    held.pop(i)
                     self.manager.close(request_id)
-                    s.status = SequenceStatus.FINISHED_ABORTED
+                    r.finish("aborted", self.clock())
                     return True
         return False
 
     def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.queue or self.active)
 
     # ------------------------------------------------------------ schedule
-    def schedule(self) -> SchedulerOutput:
+    def schedule(self) -> Plan:
         now = self.clock()
-        out = SchedulerOutput()
+        plan = Plan()
         budget = self.cfg.max_num_batched_tokens
+        prompts_first = not self.cfg.chunked_prefill and bool(self.queue)
+        if not prompts_first:
+            budget = self._plan_decodes(plan, budget)
+        budget = self._plan_portions(plan, budget)
+        budget = self._admit(plan, budget, now)
+        if prompts_first and not plan.portions:
+            self._plan_decodes(plan, budget)
+        return plan
 
-        # 1) one token for every running request whose prompt is cached
-        if self.cfg.chunked_prefill or not self.waiting:
-            for seq in list(self.running):
-                if not seq.is_prefill_done():
-                    continue
-                if len(out.decodes) >= self.cfg.max_num_seqs or budget < 1:
-                    break
-                if seq not in self.running:
-                    continue                     # preempted earlier in this pass
-                if self._reserve(seq, seq.num_computed_tokens + 1, out):
-                    out.decodes.append(seq)
-                    budget -= 1
+    def _plan_decodes(self, plan: Plan, budget: int) -> int:
+        for req in list(self.active):
+            if not req.decoding:
+                continue
+            if len(plan.decodes) >= self.cfg.max_num_seqs or budget < 1:
+                break
+            if req.phase != ACTIVE:
+                continue                         # preempted earlier in this pass
+            if self._reserve(req, req.cached + 1, plan):
+                plan.decodes.append(Planned(req, req.cached, 1))
+                budget -= 1
+        return budget
 
-        # 2) prompts that are part-way, in policy order
-        for seq in sorted((s for s in self.running if not s.is_prefill_done()), key=self.key):
+    def _plan_portions(self, plan: Plan, budget: int) -> int:
+        for req in sorted((r for r in self.active if not r.decoding), key=self.key):
             if budget <= 0:
                 break
-            if seq not in self.running:
+            if req.phase != ACTIVE:
                 continue
-            chunk = self._portion(seq, budget)
-            if self._reserve(seq, seq.num_computed_tokens + chunk, out):
-                out.prefills.append(PrefillSched(seq, chunk, seq.num_computed_tokens))
-                budget -= chunk
+            count = self._portion(req, budget)
+            if self._reserve(req, req.cached + count, plan):
+                plan.portions.append(Planned(req, req.cached, count))
+                budget -= count
+        return budget
 
-        # 3) admission
-        self.waiting.sort(key=self.key)
-        while self.waiting and len(self.running) < self.cfg.max_num_seqs and budget > 0:
-            seq = self.waiting[0]
-            too_long = self.max_positions is not None and seq.get_len() > self.max_positions
-            if too_long or not self.manager.can_ever_hold(seq.get_len()):
-                self.waiting.pop(0)
-                seq.status = SequenceStatus.FINISHED_ABORTED
-                seq.metrics.finished_time = now
-                out.aborted.append(seq)
+    def _admit(self, plan: Plan, budget: int, now: float) -> int:
+        self.queue.sort(key=self.key)
+        while self.queue and len(self.active) < self.cfg.max_num_seqs and budget > 0:
+            req = self.queue[0]
+            too_long = self.max_positions is not None and len(req.tokens) > self.max_positions
+            if too_long or not self.manager.can_ever_hold(len(req.tokens)):
+                self.queue.pop(0)
+                req.finish("aborted", now)
+                plan.aborted.append(req)
                 continue
-            if not self.manager.open(seq.request_id):
+            if not self.manager.open(req.request_id):
                 break                            # no state slot free
-            chunk = self._portion(seq, budget)
-            if not self.manager.grow(seq.request_id, seq.num_computed_tokens + chunk):
-                self.manager.close(seq.request_id)
+            count = self._portion(req, budget)
+            if not self.manager.grow(req.request_id, req.cached + count):
+                self.manager.close(req.request_id)
                 break                            # head-of-line blocking
-            seq.metrics.first_scheduled_time = seq.metrics.first_scheduled_time or now
-            self.waiting.pop(0)
-            seq.status = SequenceStatus.RUNNING
-            self.running.append(seq)
-            out.prefills.append(PrefillSched(seq, chunk, seq.num_computed_tokens))
-            budget -= chunk
-        return out
+            if req.times.admitted is None:
+                req.times.admitted = now
+            self.queue.pop(0)
+            req.phase = ACTIVE
+            self.active.append(req)
+            plan.portions.append(Planned(req, req.cached, count))
+            budget -= count
+        return budget
 
     # ------------------------------------------------------------- helpers
-    def _portion(self, seq: Sequence, budget: int) -> int:
-        """Next portion of a prompt: what the budget leaves, at least one token;
-        the whole rest when chunking is off (servelab/engine/scheduler.py:254-258)."""
-        remaining = seq.remaining_prefill_tokens()
+    def _portion(self, req: Request, budget: int) -> int:
+        """Next portion of what a request is owed: what the budget leaves, at
+        least one token; all of it when chunking is off
+        (servelab/engine/scheduler.py:254-258)."""
         if self.cfg.chunked_prefill:
-            return max(1, min(remaining, budget))
-        return max(1, remaining)
+            return max(1, min(req.owed, budget))
+        return req.owed
 
-    def _reserve(self, seq: Sequence, total_tokens: int, out: SchedulerOutput) -> bool:
-        """Pages for ``total_tokens`` of a running request, preempting others
+    def _reserve(self, req: Request, total_tokens: int, plan: Plan) -> bool:
+        """Pages for ``total_tokens`` of an active request, preempting others
         while none are free.  False when the request itself had to go."""
-        while not self.manager.grow(seq.request_id, total_tokens):
-            planned = out.planned_ids()
+        while not self.manager.grow(req.request_id, total_tokens):
+            planned = plan.planned_ids()
             victim = None
-            for cand in sorted(self.running, key=self.key, reverse=True):
-                if cand is not seq and cand.request_id not in planned:
+            for cand in sorted(self.active, key=self.key, reverse=True):
+                if cand is not req and cand.request_id not in planned:
                     victim = cand
                     break
             if victim is None:
-                self._preempt(seq, out)
+                self._preempt(req, plan)
                 return False
-            self._preempt(victim, out)
+            self._preempt(victim, plan)
         return True
 
-    def _preempt(self, seq: Sequence, out: SchedulerOutput) -> None:
+    def _preempt(self, req: Request, plan: Plan) -> None:
         """Recompute preemption (servelab/engine/scheduler.py:300-316)."""
-        self.running.remove(seq)
-        self.manager.close(seq.request_id)
-        seq.on_preempt_recompute()
-        self.waiting.insert(0, seq)
-        out.preempted.append(seq.request_id)
+        self.active.remove(req)
+        self.manager.close(req.request_id)
+        req.lost_cache()
+        self.queue.insert(0, req)
+        plan.preempted.append(req.request_id)
         self.num_preemptions += 1
 
     # ------------------------------------------------------ after the step
-    def update_after_exec(self, sampled: Dict[str, int], now: Optional[float] = None) -> List[Sequence]:
-        """Append sampled tokens, apply the stop conditions, free what finished
+    def complete(self, plan: Plan, sampled: Dict[str, int],
+                 now: Optional[float] = None) -> List[Request]:
+        """Book a step that ran ``plan``: every planned request has that much
+        more cached; those whose step ended at their newest token take their
+        sampled token from ``sampled`` and meet the stop conditions
         (servelab/engine/scheduler.py:319-349).  Returns the requests that
-        finished in this step."""
+        finished in this step; their pages are free again."""
         now = self.clock() if now is None else now
-        by_id = {s.request_id: s for s in self.running}
-        finished: List[Sequence] = []
-        for request_id, token in sampled.items():
-            seq = by_id.get(request_id)
-            if seq is None:
+        finished: List[Request] = []
+        for item in plan.items():
+            req = item.request
+            if req.phase != ACTIVE:
+                continue                         # aborted while the step ran
+            if not req.ran(item.count):
                 continue
-            seq.append_token(token)
-            if seq.metrics.first_token_time == 0.0:
-                seq.metrics.first_token_time = now
-            sp = seq.sampling_params
-            is_stop = token == self.eos_token_id or token in sp.stop_token_ids
-            if is_stop and not sp.ignore_eos:
-                seq.status = SequenceStatus.FINISHED_EOS          # the stop token stays in the output
-            elif seq.num_output_tokens >= sp.max_tokens:
-                seq.status = SequenceStatus.FINISHED_LENGTH
-            elif self.max_positions is not None and seq.get_len() >= self.max_positions:
-                seq.status = SequenceStatus.FINISHED_LENGTH       # no position left for another token
-            if seq.is_finished():
-                finished.append(seq)
-        for seq in finished:
-            self.running.remove(seq)
-            self.manager.close(seq.request_id)
-            seq.metrics.finished_time = now
+            token = int(sampled[req.request_id])
+            req.sampled(token, now)
+            sp = req.params
+            stops = token == self.eos_token_id or token in sp.stop_token_ids
+            if stops and not sp.ignore_eos:
+                req.finish("eos", now)           # the stop token stays in the output
+            elif req.num_output >= sp.max_tokens:
+                req.finish("length", now)
+            elif self.max_positions is not None and len(req.tokens) >= self.max_positions:
+                req.finish("length", now)        # no position left for another token
+            if req.done:
+                finished.append(req)
+        for req in finished:
+            self.active.remove(req)
+            self.manager.close(req.request_id)
         return finished
 
     def stats(self) -> dict:
         """servelab/engine/scheduler.py:358-369, without the prefix cache."""
-        return {"waiting": len(self.waiting), "running": len(self.running),
+        return {"waiting": len(self.queue), "running": len(self.active),
                 "gpu_cache_usage": round(self.manager.usage(), 4),
                 "num_preemptions_total": self.num_preemptions}

@@ -13,9 +13,11 @@ from servelab_amd.engine.session import load_model_on_device
 from tiny_configs import make_folder
 
 
-def make_engine(folder, num_blocks=64, max_batched=256, max_seqs=8, block_size=16):
+def make_engine(folder, num_blocks=64, max_batched=256, max_seqs=8, block_size=16, chunked=True,
+                policy="fcfs"):
     return LLMEngine(load_config(folder), CacheConfig(block_size=block_size, num_blocks=num_blocks),
-                     SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched),
+                     SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched,
+                                     chunked_prefill=chunked, policy=policy),
                      device="cpu", dtype="float32", ops=EmulatedOps())
 
 
@@ -64,10 +66,35 @@ def test_running_requests_keep_the_invariant(folder_and_plain):
         eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(5))
     while eng.has_unfinished():
         eng.step()
-        for s in eng.scheduler.running:               # tests/test_engine_smoke.py:113-127
-            if s.is_prefill_done():
-                assert s.num_computed_tokens == s.get_len() - 1
-            assert eng.runner.manager.length(s.request_id) == s.num_computed_tokens
+        for r in eng.scheduler.active:                # tests/test_engine_smoke.py:113-127
+            assert r.owed >= 1 and eng.runner.manager.length(r.request_id) == r.cached
+
+
+@pytest.mark.parametrize("max_seqs,num_blocks", [(2, 64), (8, 9)])
+def test_whole_prompts_mode_finishes_under_full_slots_and_a_tight_pool(folder_and_plain, max_seqs,
+                                                                       num_blocks):
+    """chunked_prefill off with more requests than slots, and with a pool that cannot hold them
+    all: prompts run whole, decoding goes on while nothing can be admitted, tokens are plain's."""
+    folder, want = folder_and_plain
+    eng = make_engine(folder, chunked=False, max_seqs=max_seqs, num_blocks=num_blocks, max_batched=32)
+    outs = eng.generate(PROMPTS, SamplingParams.greedy(12))
+    assert [o.outputs[0].token_ids for o in outs] == want
+    eng.runner.manager.check()
+    assert eng.runner.manager.num_free_pages() == num_blocks
+
+
+def test_priority_policy_serves_the_smaller_value_first(folder_and_plain):
+    folder, want = folder_and_plain
+    eng = make_engine(folder, policy="priority", max_seqs=1)
+    ids = [eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(12),
+                           priority=pr) for p, pr in zip(PROMPTS, (3, 0, 2, 1))]
+    order, done = [], {}
+    while eng.has_unfinished():
+        for out in eng.step():
+            order.append(out.request_id)
+            done[out.request_id] = out.outputs[0].token_ids
+    assert order == [ids[1], ids[3], ids[2], ids[0]]
+    assert [done[i] for i in ids] == want
 
 
 def test_eos_stops_and_stays_in_the_output(folder_and_plain):

@@ -4,7 +4,7 @@ import pytest
 
 from servelab_amd.cache import CacheManager
 from servelab_amd.config import SchedulerConfig
-from servelab_amd.engine import SamplingParams, Scheduler, Sequence, SequenceStatus
+from servelab_amd.engine import Request, SamplingParams, Scheduler
 from servelab_amd.parts import PagedKVSpec
 
 
@@ -36,37 +36,33 @@ class Driver:
 
     def submit(self, rid, prompt_len, output_len, priority=0, ignore_eos=True):
         self.n += 1
-        seq = Sequence(rid, list(range(1000, 1000 + prompt_len)),
-                       SamplingParams(max_tokens=output_len, ignore_eos=ignore_eos),
-                       priority=priority, arrival_time=self.clock.t, number=self.n)
-        self.scheduler.add_request(seq)
-        return seq
+        req = Request(rid, list(range(1000, 1000 + prompt_len)),
+                      SamplingParams(max_tokens=output_len, ignore_eos=ignore_eos),
+                      priority=priority, arrived=self.clock.t, number=self.n)
+        self.scheduler.add_request(req)
+        return req
 
     def step(self):
         out = self.scheduler.schedule()
         self.plans.append(out)
         sampled = {}
-        assert out.num_batched_tokens <= max(self.scheduler.cfg.max_num_batched_tokens, 1) \
+        assert out.num_tokens <= max(self.scheduler.cfg.max_num_batched_tokens, 1) \
             or not self.scheduler.cfg.chunked_prefill
-        for ps in out.prefills:
-            assert ps.num_computed == ps.seq.num_computed_tokens
-            ps.seq.num_computed_tokens += ps.num_new_tokens
-            self.manager.commit(ps.seq.request_id, ps.seq.num_computed_tokens)
-            if ps.seq.is_prefill_done():
-                sampled[ps.seq.request_id] = self.token
-        for seq in out.decodes:
-            seq.num_computed_tokens = seq.get_len()
-            self.manager.commit(seq.request_id, seq.num_computed_tokens)
-            sampled[seq.request_id] = self.token
+        for item in out.items():
+            assert item.start == item.request.cached and 1 <= item.count <= item.request.owed
+            self.manager.commit(item.request.request_id, item.start + item.count)
+            if item.samples:
+                sampled[item.request.request_id] = self.token
+        assert all(d.count == 1 and d.samples for d in out.decodes)
         self.clock.t += 0.01
-        self.finished += self.scheduler.update_after_exec(sampled)
+        self.finished += self.scheduler.complete(out, sampled)
         self.aborted += out.aborted
         self.manager.check()
-        # servelab's invariant (tests/test_engine_smoke.py:113-127)
-        for s in self.scheduler.running:
-            if s.is_prefill_done():
-                assert s.num_computed_tokens == s.get_len() - 1
-        assert set(self.manager.lengths) == {s.request_id for s in self.scheduler.running}
+        # servelab's invariant (tests/test_engine_smoke.py:113-127): between steps an active
+        # request has everything cached but what it is owed, and it is owed at least a token
+        for r in self.scheduler.active:
+            assert r.owed >= 1 and self.manager.lengths[r.request_id] == r.cached
+        assert set(self.manager.lengths) == {r.request_id for r in self.scheduler.active}
         return out
 
     def run(self, max_steps=2000):
@@ -85,16 +81,16 @@ def test_all_finish_with_exact_counts():
     for i in range(5):
         d.submit(f"r{i}", 10, 5)
     d.run()
-    assert {s.request_id: s.num_output_tokens for s in d.finished} == {f"r{i}": 5 for i in range(5)}
-    assert all(s.status == SequenceStatus.FINISHED_LENGTH for s in d.finished)
+    assert {s.request_id: s.num_output for s in d.finished} == {f"r{i}": 5 for i in range(5)}
+    assert all(s.finish_reason == "length" for s in d.finished)
 
 
 def test_portions_respect_the_budget():
     d = Driver(max_batched=8)
     d.submit("big", 40, 1)
     out = d.scheduler.schedule()
-    assert len(out.prefills) == 1 and out.prefills[0].num_new_tokens == 8
-    assert out.prefills[0].num_computed == 0
+    assert len(out.portions) == 1 and out.portions[0].count == 8
+    assert out.portions[0].start == 0
 
 
 def test_decodes_first_then_portions_share_the_budget():
@@ -103,10 +99,10 @@ def test_decodes_first_then_portions_share_the_budget():
     d.step()                               # a: whole prompt, first token sampled
     d.submit("b", 40, 2)
     out = d.step()
-    assert [s.request_id for s in out.decodes] == ["a"]
-    assert out.prefills[0].seq.request_id == "b" and out.prefills[0].num_new_tokens == 15
+    assert [d.request.request_id for d in out.decodes] == ["a"]
+    assert out.portions[0].request.request_id == "b" and out.portions[0].count == 15
     out = d.step()
-    assert out.prefills[0].num_computed == 15 and out.prefills[0].num_new_tokens == 15
+    assert out.portions[0].start == 15 and out.portions[0].count == 15
 
 
 def test_several_prompts_are_cut_in_one_step():
@@ -114,25 +110,25 @@ def test_several_prompts_are_cut_in_one_step():
     d.submit("a", 12, 1)
     d.submit("b", 12, 1)
     out = d.scheduler.schedule()
-    assert [(p.seq.request_id, p.num_new_tokens) for p in out.prefills] == [("a", 12), ("b", 8)]
+    assert [(p.request.request_id, p.count) for p in out.portions] == [("a", 12), ("b", 8)]
 
 
 def test_fcfs_and_priority_order():
     d = Driver(max_batched=12)
     for i in range(4):
         d.submit(f"r{i}", 20, 1)
-    assert d.scheduler.schedule().prefills[0].seq.request_id == "r0"
+    assert d.scheduler.schedule().portions[0].request.request_id == "r0"
     d = Driver(max_batched=12, policy="priority")
     d.submit("low", 20, 1, priority=5)
     d.submit("high", 20, 1, priority=0)
-    assert d.scheduler.schedule().prefills[0].seq.request_id == "high"
+    assert d.scheduler.schedule().portions[0].request.request_id == "high"
 
 
 def test_request_numbers_not_id_strings_break_ties():
     d = Driver(max_batched=4)
     d.submit("req-10", 4, 1)
     d.submit("req-2", 4, 1)
-    assert d.scheduler.schedule().prefills[0].seq.request_id == "req-10"
+    assert d.scheduler.schedule().portions[0].request.request_id == "req-10"
 
 
 def test_preemption_when_pages_run_out():
@@ -141,9 +137,9 @@ def test_preemption_when_pages_run_out():
     seqs = [d.submit(f"r{i}", 8, 10) for i in range(4)]
     d.run()
     assert len(d.finished) == 4
-    assert sum(s.metrics.num_preemptions for s in d.finished) > 0
+    assert sum(s.times.preemptions for s in d.finished) > 0
     # outputs survive a preemption: ten tokens each, the prompt untouched
-    assert all(s.num_output_tokens == 10 and s.num_prompt_tokens == 8 for s in seqs)
+    assert all(s.num_output == 10 and s.prompt_len == 8 for s in seqs)
     # the victim is the request that came last, and it goes to the front of the queue
     first = next(p for p in d.plans if p.preempted)
     assert first.preempted[0] == "r3" or first.preempted[0] == "r2"
@@ -156,19 +152,19 @@ def test_the_victim_is_the_last_in_policy_order_and_requeues_first():
     d.step()                         # both prompts (2 pages each), first tokens
     d.step()                         # position 7 still fits the second page
     out = d.step()                   # a needs position 8 -> a third page: b is evicted
-    assert out.preempted == ["b"] and [s.request_id for s in out.decodes] == ["a"]
-    assert b.status == SequenceStatus.WAITING and d.scheduler.waiting[0] is b
-    assert b.num_computed_tokens == 0 and b.prefill_target == 9 and b.num_prompt_tokens == 7
+    assert out.preempted == ["b"] and [d.request.request_id for d in out.decodes] == ["a"]
+    assert b.phase == "queued" and d.scheduler.queue[0] is b
+    assert b.cached == 0 and b.owed == 9 and b.prompt_len == 7 and b.num_output == 2
     d.run()
-    assert a.num_output_tokens == 8 and b.num_output_tokens == 8
+    assert a.num_output == 8 and b.num_output == 8
 
 
 def test_a_single_request_too_big_for_what_is_left_preempts_itself_then_aborts_or_finishes():
     d = Driver(num_pages=3, page_size=4, max_batched=64, max_seqs=2)
     s = d.submit("a", 10, 8)         # grows to 18 tokens > 12
     d.run()
-    assert s.status == SequenceStatus.FINISHED_ABORTED and d.aborted == [s]
-    assert s.metrics.num_preemptions == 1
+    assert s.finish_reason == "aborted" and d.aborted == [s]
+    assert s.times.preemptions == 1
 
 
 def test_oversize_and_overlong_requests_abort_at_admission():
@@ -176,13 +172,13 @@ def test_oversize_and_overlong_requests_abort_at_admission():
     big = d.submit("big", 17, 2)
     ok = d.submit("ok", 8, 2)
     out = d.step()
-    assert out.aborted == [big] and big.status == SequenceStatus.FINISHED_ABORTED
-    assert out.prefills[0].seq is ok
+    assert out.aborted == [big] and big.finish_reason == "aborted" and big.done
+    assert out.portions[0].request is ok
     d = Driver(num_pages=64, page_size=4, max_positions=12)
     assert d.submit("long", 13, 1) and d.step().aborted[0].request_id == "long"
     s = d.submit("edge", 10, 20)
     d.run()
-    assert s.get_len() == 12 and s.status == SequenceStatus.FINISHED_LENGTH
+    assert len(s.tokens) == 12 and s.finish_reason == "length"
 
 
 def test_head_of_line_blocking_and_max_num_seqs():
@@ -191,11 +187,11 @@ def test_head_of_line_blocking_and_max_num_seqs():
     d.submit("b", 12, 1)             # does not fit beside a
     d.submit("c", 2, 1)              # would fit, but waits behind b
     out = d.scheduler.schedule()
-    assert [p.seq.request_id for p in out.prefills] == ["a"]
+    assert [p.request.request_id for p in out.portions] == ["a"]
     d = Driver(max_seqs=2, max_batched=64)
     for i in range(5):
         d.submit(f"r{i}", 4, 3)
-    assert len(d.scheduler.schedule().prefills) == 2
+    assert len(d.scheduler.schedule().portions) == 2
     d.run()
 
 
@@ -204,8 +200,8 @@ def test_eos_and_stop_tokens():
     s = d.submit("a", 4, 10, ignore_eos=False)
     t = d.submit("b", 4, 3, ignore_eos=True)
     d.run()
-    assert s.status == SequenceStatus.FINISHED_EOS and s.output_token_ids == [7]
-    assert t.status == SequenceStatus.FINISHED_LENGTH and t.num_output_tokens == 3
+    assert s.finish_reason == "eos" and s.output == [7]
+    assert t.finish_reason == "length" and t.num_output == 3
 
 
 def test_abort():
@@ -220,22 +216,41 @@ def test_abort():
     assert d.manager.num_free_pages() == 16
 
 
-def test_unchunked_mode_runs_whole_prompts_and_holds_decodes_while_any_waits():
-    d = Driver(chunked=False, max_batched=8, num_pages=64, max_seqs=1)
+def test_unchunked_mode_runs_whole_prompts_before_decode_tokens():
+    d = Driver(chunked=False, max_batched=8, num_pages=64, max_seqs=2)
     d.submit("a", 20, 3)
-    d.submit("b", 20, 2)
     out = d.step()
-    assert out.prefills[0].num_new_tokens == 20
-    out = d.scheduler.schedule()
-    assert out.is_empty()            # b waits, max_seqs is 1: servelab/engine/scheduler.py:177
-    d.scheduler.abort_request("b")
+    assert out.portions[0].count == 20         # the whole prompt, beyond the token budget
+    d.submit("b", 20, 2)
+    out = d.step()                             # b can be admitted: it goes first, a holds
+    assert [p.request.request_id for p in out.portions] == ["b"] and not out.decodes
+    out = d.step()
+    assert sorted(x.request.request_id for x in out.decodes) == ["a", "b"]
     d.run()
+
+
+def test_unchunked_mode_decodes_on_when_nothing_can_be_admitted():
+    # every slot taken: the reference plans nothing here (servelab/engine/scheduler.py:177) and
+    # stops for good; the active request has to go on, since that is what frees the slot
+    d = Driver(chunked=False, max_batched=8, num_pages=64, max_seqs=1)
+    a = d.submit("a", 20, 3)
+    b = d.submit("b", 20, 2)
+    d.step()
+    out = d.step()
+    assert [x.request.request_id for x in out.decodes] == ["a"] and not out.portions
+    d.run()
+    assert a.num_output == 3 and b.num_output == 2
+    # the head of the queue does not fit beside what is active (tight pool): same decision
+    d = Driver(chunked=False, max_batched=64, num_pages=8, page_size=4, max_seqs=4)
+    reqs = [d.submit(f"r{i}", 14, 6) for i in range(3)]
+    d.run()
+    assert all(r.num_output == 6 and r.finish_reason == "length" for r in reqs)
 
 
 def test_window_groups_keep_few_pages_during_long_decoding():
     d = Driver(num_pages=12, page_size=4, max_batched=64, window=8)
     s = d.submit("a", 6, 40)
     d.run()
-    assert s.num_output_tokens == 40
+    assert s.num_output == 40
     assert d.manager.page_groups[1].allocator.high_water <= 4
     assert d.manager.page_groups[0].allocator.high_water == 12
