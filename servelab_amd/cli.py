@@ -6,13 +6,15 @@ and --kv-cache-dtype are accepted for compatibility: this engine has no prefix
 cache and keeps the cache in the compute dtype), the same fixed
 max_num_seqs=16 / max_num_batched_tokens=1024 defaults, temperature 1.0
 sampling unless told otherwise, the same printed lines.  Without --model a
-tiny random model is written to a temporary folder and used, as there.
+tiny random model is used, as there; here its weights (and those of any
+``--config`` with ``--random-weights SEED``) are drawn on the device, so a
+configuration of any size starts at once and no folder is written, unless
+--model names one to write.
 """
 import argparse
 import json
 import os
 import sys
-import tempfile
 
 TINY_DEFAULT = dict(
     architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=96, hidden_size=32,
@@ -34,7 +36,8 @@ def build_parser():
     ap.add_argument("--dtype", default="auto", choices=["auto", "bfloat16", "bf16", "float32", "fp32"])
     ap.add_argument("--config", default="", help="config.json for --random-weights")
     ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
-                    help="write seeded random weights for --config (or the tiny default) and use them")
+                    help="seeded random weights for --config (or the tiny default), made on the "
+                         "device; with --model DIR they are written there as a model folder first")
     ap.add_argument("--prompt-ids", default="", help="comma-separated token ids instead of --prompt")
     ap.add_argument("--temperature", type=float, default=1.0)
     ap.add_argument("--top-k", type=int, default=-1)
@@ -66,17 +69,17 @@ def main(argv=None) -> int:
                    write_random_model)
     from .config import resolve_architecture
 
-    tmp = None
     tokenizer = None
+    seed = None
     if args.model and args.random_weights is None:
-        folder = args.model
-        has_files = any(os.path.exists(os.path.join(folder, f))
+        mc = load_config(args.model)
+        has_files = any(os.path.exists(os.path.join(args.model, f))
                         for f in ("tokenizer.json", "tokenizer_config.json", "tokenizer.model"))
         try:
             if not has_files:
                 raise FileNotFoundError("no tokenizer files in the model folder")
             from transformers import AutoTokenizer          # tokenizer files only, optional
-            tokenizer = AutoTokenizer.from_pretrained(folder)
+            tokenizer = AutoTokenizer.from_pretrained(args.model)
         except Exception as e:                              # noqa: BLE001
             print(f"[warn] no tokenizer: {e}")
     else:
@@ -84,16 +87,17 @@ def main(argv=None) -> int:
         if args.config:
             with open(args.config, encoding="utf-8") as f:
                 raw = json.load(f)
-        cfg = resolve_architecture(raw).config_from_hf(raw, "")
-        tmp = tempfile.TemporaryDirectory()
-        folder = args.model or os.path.join(tmp.name, "random-model")
-        write_random_model(cfg, folder, seed=args.random_weights or 0)
-    mc = load_config(folder)
+        mc = resolve_architecture(raw).config_from_hf(raw, "")
+        seed = args.random_weights or 0
+        if args.model:                                      # keep the model: a folder, made on the host
+            write_random_model(mc, args.model, seed=seed)
+            mc, seed = load_config(args.model), None
     engine = LLMEngine(
         mc, CacheConfig(block_size=args.block_size, num_blocks=args.num_blocks or None),
         SchedulerConfig(max_num_seqs=args.max_num_seqs,
                         max_num_batched_tokens=args.max_batched_tokens),
-        seed=args.seed, tokenizer=tokenizer, dtype=args.dtype, tune_products=tune_option(args))
+        seed=args.seed, tokenizer=tokenizer, dtype=args.dtype, tune_products=tune_option(args),
+        random_weights=seed)
     if args.prompt_ids:
         prompts = [[int(t) for t in args.prompt_ids.split(",")]]
     elif tokenizer is not None:
@@ -108,8 +112,6 @@ def main(argv=None) -> int:
         text = comp.text if comp.text else str(comp.token_ids)
         print(f"[{out.request_id}] finish={comp.finish_reason} -> {text}")
     print("stats:", engine.stats())
-    if tmp is not None:
-        tmp.cleanup()
     return 0
 
 

@@ -16,7 +16,7 @@ from .output import RequestOutput, result_of
 from .sampling_params import SamplingParams
 from .scheduler import Scheduler
 from .request import Request
-from .session import load_model_on_device, make_runner
+from .session import load_model_on_device, make_runner, random_model_on_device
 
 
 class LLMEngine:
@@ -24,10 +24,12 @@ class LLMEngine:
                  scheduler_config: Optional[SchedulerConfig] = None, seed: int = 1234,
                  device: str = "cuda:0", tokenizer=None,
                  clock: Optional[Callable[[], float]] = None, dtype: str = "auto",
-                 model=None, ops=None, tune_products=False):
+                 model=None, ops=None, tune_products=False, random_weights: Optional[int] = None):
         """``model_config.path`` names the model folder (as in the reference,
         servelab/engine/engine.py:86-87); ``model`` may pass an already loaded
-        DecoderModel instead.  ``tune_products``: True, or a list of further
+        DecoderModel instead, and ``random_weights`` a seed: the model of
+        ``model_config`` then gets seeded random weights made on the device and
+        no folder is read.  ``tune_products``: True, or a list of further
         step sizes (rows) to time the library's matrix kernels for."""
         self.model_config = model_config
         self.cache_config = cache_config or CacheConfig()
@@ -36,10 +38,12 @@ class LLMEngine:
         self.clock = clock or time.monotonic
         if device == "auto":
             device = "cuda:0"
+        if model is None and random_weights is not None:
+            model = random_model_on_device(model_config, random_weights, dtype, device, ops=ops)
         if model is None:
             if not getattr(model_config, "path", ""):
-                raise ValueError("model_config.path must name a model folder "
-                                 "(write_random_model makes one from a configuration and a seed)")
+                raise ValueError("model_config.path must name a model folder (or pass "
+                                 "random_weights=SEED; write_random_model writes such a folder)")
             _, model = load_model_on_device(model_config.path, dtype, device, ops=ops,
                                             config=model_config)
         self.model = model
@@ -153,5 +157,7 @@ class LLMEngine:
     def stats(self) -> dict:
         return {**self.scheduler.stats(), **self.runner.manager.stats(),
                 "num_blocks": self.num_blocks, "block_size": self.cache_config.block_size,
-                "dtype": str(self.dtype).replace("torch.", ""), "device": str(self.device),
+                "dtype": str(self.dtype).replace("torch.", ""),
+                "checkpoint_dtype": getattr(self.model_config, "dtype", None),
+                "device": str(self.device),
                 "steps": self.num_steps}

@@ -4,6 +4,7 @@ Reference: the first half of ``LLMEngine.__init__``
 (servelab/engine/engine.py:84-111): resolve the dtype, build the model, load
 the checkpoint, size and allocate the cache pool.
 """
+import sys
 from typing import Optional
 
 import torch
@@ -12,21 +13,32 @@ from ..cache import CachePool
 from ..parts.base import Runtime
 from ..parts.model import DecoderModel, build_model_spec
 from ..weights.loader import Checkpoint, load_config
+from ..weights.random_init import RandomCheckpoint
 from .runner import ModelRunner
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
            "float32": torch.float32, "fp32": torch.float32}
 
 
+FLOAT16_NOTICE = ("config.json says torch_dtype float16: this engine has bfloat16 and float32 kernels "
+                  "only; the weights are converted and served in bfloat16 (8 bits of mantissa instead "
+                  "of 11, a wider exponent), so logits differ from a float16 run by rounding. "
+                  "Pass dtype float32 for the exact path.")
+
+
 def resolve_dtype(name: str, config=None) -> torch.dtype:
-    """'auto' takes config.json's torch_dtype; float16 checkpoints are served
-    in bfloat16 (weights are kept in bfloat16)."""
+    """'auto' takes config.json's torch_dtype.  There are no float16 kernels: a
+    float16 checkpoint under 'auto' is served in bfloat16 and says so on
+    standard error (the reference serves it as float16,
+    servelab/engine/engine.py:35-39); float16 asked for by name is refused."""
     if name in (None, "auto"):
         name = getattr(config, "dtype", "bfloat16")
-        if name == "float16":
+        if name in ("float16", "fp16", "half"):
+            print(f"[servelab_amd] {FLOAT16_NOTICE}", file=sys.stderr, flush=True)
             name = "bfloat16"
     if name not in _DTYPES:
-        raise ValueError(f"dtype must be bfloat16 or float32, is {name!r}")
+        raise ValueError(f"dtype must be bfloat16 or float32 (or auto), is {name!r}: "
+                         "there are no kernels for other types")
     return _DTYPES[name]
 
 
@@ -44,6 +56,16 @@ def load_model_on_device(folder: str, dtype="auto", device="cuda:0", ops=None, c
     model = DecoderModel(build_model_spec(config), rt)
     model.load(Checkpoint(folder))
     return config, model
+
+
+def random_model_on_device(config, seed: int, dtype="auto", device="cuda:0", ops=None) -> DecoderModel:
+    """A DecoderModel of ``config`` with seeded random weights drawn on the
+    device, tensor by tensor as the parts load them; no folder is written
+    (examples/run_engine.py:21-24 makes its tiny default model on the host)."""
+    rt = make_runtime(resolve_dtype(dtype, config), device, ops)
+    model = DecoderModel(build_model_spec(config), rt)
+    model.load(RandomCheckpoint(model.spec.param_specs(), seed, rt.device, rt.act_dtype))
+    return model
 
 
 def default_num_pages(model: DecoderModel, page_size: int, utilization: float) -> int:

@@ -121,11 +121,15 @@ def decoder_layer(cfg, w, i, h, positions):
     eps = cfg["rms_norm_eps"]
     T = h.shape[0]
 
+    def project(name, heads):
+        y = x @ w[p + f"self_attn.{name}.weight"].T
+        if cfg.get("attention_bias", True):           # servelab/parallel/tp_model.py:48-50 (qkv_bias)
+            y = y + w[p + f"self_attn.{name}.bias"]
+        return y.view(T, heads, D)
+
     x = rms_norm(h, w[p + "input_layernorm.weight"], eps)
-    q = (x @ w[p + "self_attn.q_proj.weight"].T + w[p + "self_attn.q_proj.bias"]).view(T, nh, D)
-    k = (x @ w[p + "self_attn.k_proj.weight"].T + w[p + "self_attn.k_proj.bias"]).view(T, nkv, D)
-    v = (x @ w[p + "self_attn.v_proj.weight"].T + w[p + "self_attn.v_proj.bias"]).view(T, nkv, D)
-    inv_freq = rope_inv_freq(cfg.get("rope_theta", 1e6), D, dtype=h.dtype)
+    q, k, v = project("q_proj", nh), project("k_proj", nkv), project("v_proj", nkv)
+    inv_freq = rope_inv_freq(cfg.get("rope_theta", 1e6), D, dtype=h.dtype).to(h.device)
     q = apply_rope(q, positions, inv_freq)
     k = apply_rope(k, positions, inv_freq)
     o = attention(q, k, v, 1.0 / math.sqrt(D), positions, positions,
@@ -146,8 +150,9 @@ def forward(cfg, weights, token_ids, dtype=torch.float32, start_position=0):
     position.
     """
     w = {k: v.to(dtype) for k, v in weights.items()}
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
-    positions = torch.arange(start_position, start_position + len(ids))
+    device = w["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
+    positions = torch.arange(start_position, start_position + len(ids), device=device)
     h = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
         h = decoder_layer(cfg, w, i, h, positions)

@@ -153,3 +153,13 @@ def test_cli_smoke(folder_and_plain, capsys, monkeypatch):
                      "--num-blocks", "32"]) == 0
     printed = capsys.readouterr().out
     assert f"[req-1] finish=length -> {want[0]}" in printed and "stats:" in printed
+
+
+def test_float16_checkpoints_are_served_in_bfloat16_and_say_so(tmp_path, capsys):
+    from servelab_amd.engine.session import resolve_dtype
+    cfg = load_config(make_folder(tmp_path, "A", seed=1, torch_dtype="float16"))
+    assert resolve_dtype("auto", cfg) == torch.bfloat16
+    assert "served in bfloat16" in capsys.readouterr().err
+    with pytest.raises(ValueError, match="no kernels"):
+        resolve_dtype("float16", cfg)
+    assert resolve_dtype("float32", cfg) == torch.float32 and capsys.readouterr().err == ""

@@ -59,6 +59,34 @@ def test_rope_properties():
     assert torch.allclose(big[..., 1:half], x[..., 1:half], atol=1e-3)       # theta -> inf: identity
 
 
+def test_rope_is_a_complex_multiplication():
+    """The rotation as a library routine: the pair (x[j], x[j + D/2]) read as the complex number
+    x[j] + i x[j + D/2] is multiplied by exp(+i pos inv_freq[j]).  A flipped sign (the conjugate)
+    or interleaved pairs (x[2j], x[2j + 1]) fail this."""
+    D = 24
+    inv = plain.rope_inv_freq(1e6, D)
+    x = torch.randn(7, 3, D, dtype=torch.float64)
+    pos = torch.tensor([0, 1, 3, 4, 50, 51, 64])        # float32 angles: small positions keep 1e-5
+    z = torch.complex(x[..., :D // 2], x[..., D // 2:])
+    angle = pos.double()[:, None, None] * inv.double()
+    want = z * torch.polar(torch.ones_like(angle), angle)
+    got = plain.apply_rope(x.float(), pos, inv)
+    assert torch.allclose(got[..., :D // 2].double(), want.real, atol=1e-5)
+    assert torch.allclose(got[..., D // 2:].double(), want.imag, atol=1e-5)
+    flipped = z * torch.polar(torch.ones_like(angle), -angle)
+    assert not torch.allclose(got[..., D // 2:].double(), flipped.imag, atol=1e-2)
+    # hence q_m . k_n = Re(sum_j q_j conj(k_j) exp(i (m - n) theta_j)): distances only
+    q, k = torch.randn(1, 1, D), torch.randn(1, 1, D)
+    zq = torch.complex(q[..., :D // 2], q[..., D // 2:]).to(torch.complex128)
+    zk = torch.complex(k[..., :D // 2], k[..., D // 2:]).to(torch.complex128)
+    m, n = 40, 33
+    want_score = (zq * zk.conj() * torch.polar(torch.ones(D // 2, dtype=torch.float64),
+                                               (m - n) * inv.double())).real.sum()
+    got_score = (plain.apply_rope(q, torch.tensor([m]), inv) *
+                 plain.apply_rope(k, torch.tensor([n]), inv)).sum()
+    assert abs(float(got_score) - float(want_score)) < 1e-4
+
+
 def test_attention_reduces_to_the_library_routine():
     T, nh, nkv, D = 9, 4, 2, 8
     q, k, v = torch.randn(T, nh, D), torch.randn(T, nkv, D), torch.randn(T, nkv, D)

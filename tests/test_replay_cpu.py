@@ -38,3 +38,19 @@ def test_replay_matches_plain(tmp_path, which, schedule):
                       ops=EmulatedOps(torch.float32), device="cpu")
     worst, where = compare(out, steps, reference, vocab)
     assert worst < 1e-4, f"max abs err {worst} at {where}"
+
+
+@pytest.mark.parametrize("page", [16, 32, 64])
+def test_replay_of_the_probe_model_at_every_page_size(tmp_path, page):
+    import probe_model as pm
+    from replay_harness import probe_score
+    folder = pm.write_probe_model(str(tmp_path / "probe"))
+    vocab = pm.PROBE["vocab_size"]
+    requests = make_requests(vocab, [150, 61, 333, 97, 260, 48, 129], seed=8)
+    reference = plain_logits(folder, requests)
+    steps = rs.mixed(requests, {r: max(2, len(t) - 32) for r, t in requests.items()})
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, "float32", rs.max_tokens_needed(steps, max(64, page)),
+                      ops=EmulatedOps(torch.float32), device="cpu", block_size=page)
+    worst, where = compare(out, steps, reference, vocab, score=probe_score)
+    assert worst <= 0.02, f"score {worst} at {where}"

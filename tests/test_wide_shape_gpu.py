@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import replay_schedules as rs
-from replay_harness import compare, plain_logits, replay_in_process, tolerance
+from replay_harness import bfloat16_bar, compare, plain_logits, replay_in_process, tolerance
 from servelab_amd import Qwen2Config, write_random_model
 
 pytestmark = pytest.mark.gpu
@@ -46,8 +46,10 @@ def test_wide_shape_matches_plain(tmp_path, wide, dtype):
     out = str(tmp_path / "out")
     replay_in_process(folder, steps, out, dtype, rs.max_tokens_needed(steps))
     worst, where = compare(out, steps, reference, 152064)
-    print(f"wide {dtype}: max abs err {worst:.3e} at {where}")
-    assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
+    bar = tolerance(dtype, reference) if dtype == "float32" else \
+        bfloat16_bar(folder, requests, reference, 152064, "wide")
+    print(f"wide {dtype}: max abs err {worst:.3e} at {where}, bar {bar:.3e}")
+    assert worst < bar, f"max abs err {worst} at {where}"
 
 
 @pytest.fixture(scope="module")
@@ -98,3 +100,42 @@ def test_wide_shape_long_prompt_and_growing_batches(tmp_path, crowd, dtype):
     worst, where = compare(out, steps, reference, 152064)
     print(f"wide, long prompt and batches, {dtype}: max abs err {worst:.3e} at {where}")
     assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
+
+
+def test_float32_error_at_depth():
+    """The float32 path against a float64 run of the plain implementation at 2, 4, 8 and all 28
+    layers of the 7B widths (vocabulary cut to 4,099 rows: depth is what is looked at).  The weights are made
+    on the device and shared by both sides; the plain implementation runs on the device in float64
+    and in float32 (library products, no reduced-precision mode), the latter to show what float32
+    arithmetic itself costs at that depth.  Prompt of 48 tokens, then 16 tokens one by one.
+    Up to 8 layers the error stays below 1e-4; at every depth it stays within 1.5 times what the
+    plain implementation loses by computing in float32 itself (it grows like the square root of
+    the depth for both)."""
+    import plain_qwen2 as plain
+    from servelab_amd.engine import ModelRunner, StepEntry
+    from servelab_amd.engine.session import random_model_on_device
+    torch.backends.cuda.matmul.allow_tf32 = False
+    rng = random.Random(4)
+    toks = [rng.randrange(4099) for _ in range(64)]
+    report = {}
+    for layers in (2, 4, 8, 28):
+        raw = dict(WIDE, num_hidden_layers=layers, vocab_size=4099, eos_token_id=4098)
+        cfg = Qwen2Config.from_hf(raw)
+        model = random_model_on_device(cfg, 7, "float32")
+        from servelab_amd.weights import RandomCheckpoint
+        weights = RandomCheckpoint(model.spec.param_specs(), 7, "cuda:0", torch.float32).state_dict()
+        exact = plain.forward(raw, weights, toks, dtype=torch.float64)
+        plain32 = plain.forward(raw, weights, toks, dtype=torch.float32).double()
+        runner = ModelRunner(model, 8, 16)
+        rows = [runner.step([StepEntry("a", toks[:48], list(range(48)))])]
+        rows += [runner.step([StepEntry("a", [t], [0])]).clone() for t in toks[48:]]
+        got = torch.cat(rows).double()
+        report[layers] = ((got - exact).abs().max().item(), (plain32 - exact).abs().max().item(),
+                          exact.abs().max().item())
+        del model, runner, weights
+        torch.cuda.empty_cache()
+    for layers, (engine, arithmetic, top) in report.items():
+        print(f"float32 at {layers} layers of the 7B widths: engine {engine:.2e}, plain float32 "
+              f"{arithmetic:.2e} off the float64 logits (largest {top:.2f})")
+    assert all(report[layers][0] <= 1e-4 for layers in (2, 4, 8)), report
+    assert all(engine <= 1.5 * arithmetic for engine, arithmetic, _ in report.values()), report
