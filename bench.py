@@ -46,43 +46,18 @@ SHAPES = {"7b": ("Qwen2.5-7B shape", QWEN25_7B), "32b": ("Qwen2.5-32B shape", QW
           "72b": ("Qwen2.5-72B shape", QWEN25_72B)}
 
 
-class RandomCheckpoint:
-    """Seeded random tensors made on the device when a part asks for them, so
-    that a 15 GB model needs no file: N(0, 0.02), norm gains 1 + N(0, 0.05)."""
-
-    def __init__(self, specs, seed, device, dtype):
-        self.specs, self.seed, self.device, self.dtype = specs, seed, device, dtype
-        self.order = {n: i for i, n in enumerate(specs)}
-
-    def shapes(self):
-        return {n: s.shape for n, s in self.specs.items()}
-
-    def get(self, name):
-        import torch
-        spec = self.specs[name]
-        gen = torch.Generator(device=self.device)
-        gen.manual_seed(self.seed * 100003 + self.order[name])
-        t = torch.randn(spec.shape, generator=gen, device=self.device, dtype=torch.float32)
-        t = 1.0 + 0.05 * t if spec.init == "gain" else 0.02 * t
-        return t.to(self.dtype) if len(spec.shape) > 1 else t
-
-
 def build(args):
     import torch
     import servelab_amd  # noqa: F401
     from servelab_amd import Qwen2Config
-    from servelab_amd.engine.session import make_runtime, resolve_dtype
-    from servelab_amd.parts import DecoderModel, build_model_spec
+    from servelab_amd.engine.session import random_model_on_device
 
     raw = dict(SHAPES[args.shape][1])
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_hf(raw)
-    dtype = resolve_dtype(args.dtype)
-    rt = make_runtime(dtype, "cuda:0")
-    model = DecoderModel(build_model_spec(cfg), rt)
-    model.load(RandomCheckpoint(model.spec.param_specs(), args.seed, rt.device, dtype))
+    model = random_model_on_device(cfg, args.seed, args.dtype, "cuda:0")
     torch.cuda.synchronize()
     return cfg, model, full_layers
 

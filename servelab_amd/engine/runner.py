@@ -7,6 +7,7 @@ selected rows, float32 logits.  Here that is a function of its own below the
 scheduler, so that trace replay, the benchmark and the engine drive the same
 code.  It runs only the tokens it is given, from the cache earlier steps left.
 """
+from collections import OrderedDict
 from typing import Dict, Hashable, List, Optional
 
 import torch
@@ -24,6 +25,12 @@ class OutOfPages(RuntimeError):
 class ModelRunner:
     GRAPH_MAX_SEQS = 64
     GRAPH_MIN_CONTEXT = 512
+    # Captured decode graphs keep their outputs (float32 logits [requests, vocabulary]) and metadata
+    # buffers for as long as they live; their intermediates share one memory pool.  What they keep
+    # is bounded: at most this share of the device memory that is free once the cache pool stands,
+    # and at most GRAPH_MEMORY_MAX bytes; the graph used longest ago goes first.
+    GRAPH_MEMORY_SHARE = 0.25
+    GRAPH_MEMORY_MAX = 4 << 30
 
     def __init__(self, model: DecoderModel, num_pages: int, page_size: int,
                  max_num_seqs: int = 64, use_graphs: bool = True):
@@ -40,8 +47,15 @@ class ModelRunner:
         # table says itself up to how many rows its products stay clear of library calls
         self.use_graphs = (use_graphs and self.rt.device.type == "cuda" and model.spec.graph_safe)
         self.graph_max_seqs = int(getattr(self.rt.ops, "graph_rows_limit", self.GRAPH_MAX_SEQS))
-        self._graphs = {}
+        self._graphs: "OrderedDict[tuple, tuple]" = OrderedDict()     # least recently used first
+        self._graph_pool = None           # one memory pool for the intermediates of all captures
+        self._graph_bytes = 0
+        self.graph_memory_limit = self.GRAPH_MEMORY_MAX
+        if self.use_graphs:
+            free, _ = torch.cuda.mem_get_info(self.rt.device)
+            self.graph_memory_limit = min(self.GRAPH_MEMORY_MAX, int(free * self.GRAPH_MEMORY_SHARE))
         self.graph_replays = 0
+        self.graph_evictions = 0
         self._decoding = None         # the last graph step, for the next one to continue from
 
     # ------------------------------------------------------------ requests
@@ -127,6 +141,7 @@ class ModelRunner:
         host = torch.from_numpy(arr.flat)
         entry = self._graphs.get(key)
         if entry is not None:
+            self._graphs.move_to_end(key)
             graph, dev, staging, logits, copied = entry
             copied.synchronize()              # the last copy out of the staging buffer is done
             staging.copy_(host)
@@ -145,14 +160,40 @@ class ModelRunner:
         with torch.cuda.stream(side):
             eager = self.model.forward(batch, self.bindings)
         torch.cuda.current_stream().wait_stream(side)
+        need = self._entry_bytes(dev, B)
+        self._make_room(need)
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, pool=self._graph_pool):
             logits = self.model.forward(batch, self.bindings)
         copied = torch.cuda.Event()
         copied.record()
         self._graphs[key] = (graph, dev, staging, logits, copied)
+        self._graph_bytes += need
         self._decoding = (key, arr)
         return eager
+
+    def _entry_bytes(self, dev, B) -> int:
+        """What a captured graph keeps alive beside the shared pool of
+        intermediates: its logits and its metadata buffer."""
+        return B * self.model.spec.vocab_size * 4 + dev.numel() * dev.element_size()
+
+    def _make_room(self, need: int) -> None:
+        """Drop the graphs used longest ago until ``need`` more bytes fit the
+        limit (a single graph larger than the limit is still kept alone).
+        The device is idle for this: a graph's memory must not return to the
+        pool while a replay of it is still running."""
+        if not self._graphs or self._graph_bytes + need <= self.graph_memory_limit:
+            return
+        torch.cuda.synchronize(self.rt.device)
+        while self._graphs and self._graph_bytes + need > self.graph_memory_limit:
+            old_key, (graph, dev, staging, logits, copied) = self._graphs.popitem(last=False)
+            self._graph_bytes -= self._entry_bytes(dev, old_key[0])
+            self.graph_evictions += 1
+            if self._decoding is not None and self._decoding[0] == old_key:
+                self._decoding = None
+            del graph, dev, staging, logits, copied
 
     def _continue_decoding(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
         """The common decode step — the same requests as the last graph step,
@@ -195,6 +236,7 @@ class ModelRunner:
                 if p % bs == 0:
                     flat[tables_at + i * pages + p // bs] = page
         arr.starts = starts
+        self._graphs.move_to_end(key)
         graph, dev, staging, logits, copied = self._graphs[key]
         copied.synchronize()
         staging.copy_(torch.from_numpy(flat))
@@ -238,7 +280,8 @@ class ModelRunner:
 
     def step(self, entries: List[StepEntry]) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of
-        the entries and of their ``want``."""
+        the entries and of their ``want``.  The tensor may be a captured graph's
+        output buffer: it is valid until the next call of ``step``."""
         if not entries:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32,
                                device=self.rt.device)

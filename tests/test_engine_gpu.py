@@ -124,6 +124,48 @@ def test_graph_replay_equals_eager(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_graphs_are_bounded(tmp_path, dtype, monkeypatch):
+    """More graph keys (requests x context capacity) than the memory limit holds: the graphs used
+    longest ago are dropped and captured again when their shape returns; logits equal those of a
+    runner without graphs throughout, and device memory does not grow from one round to the next."""
+    monkeypatch.setattr(ModelRunner, "GRAPH_MIN_CONTEXT", 32)
+    folder = make_folder(tmp_path, "B", seed=28)
+    _, model = load_model_on_device(folder, dtype)
+    vocab = TINY["B"]["vocab_size"]
+    eager = ModelRunner(model, 64, 16, use_graphs=False)
+    graphs = ModelRunner(model, 64, 16, use_graphs=True)
+    per_graph = vocab * 4 * 3 + 4096
+    graphs.graph_memory_limit = 3 * per_graph            # the six keys together need four times a graph of 3
+    rng = random.Random(5)
+
+    def one_round(tag):
+        worst = 0.0
+        for batch in (1, 2, 3, 2, 1, 3):                  # with two context capacities each: 6 keys
+            ids = [f"{tag}{batch}_{i}" for i in range(batch)]
+            prompt = [[rng.randrange(vocab) for _ in range(20 + 3 * i)] for i in range(batch)]
+            for r in (eager, graphs):
+                r.step([StepEntry(i, p, []) for i, p in zip(ids, prompt)])
+            for _ in range(16):                           # contexts cross 32: a second capacity
+                toks = [rng.randrange(vocab) for _ in ids]
+                a = eager.step([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)])
+                b = graphs.step([StepEntry(i, [t], [0]) for i, t in zip(ids, toks)])
+                worst = max(worst, (a - b).abs().max().item())
+            for i in ids:
+                eager.close(i), graphs.close(i)
+        return worst
+
+    assert one_round("a") <= (0.0 if dtype == "float32" else 1e-2)
+    torch.cuda.synchronize()
+    held, evicted = torch.cuda.memory_allocated(), graphs.graph_evictions
+    assert evicted > 0 and len(graphs._graphs) < 6 and graphs._graph_bytes <= graphs.graph_memory_limit
+    assert one_round("b") <= (0.0 if dtype == "float32" else 1e-2)
+    torch.cuda.synchronize()
+    assert graphs.graph_evictions > evicted and graphs._graph_bytes <= graphs.graph_memory_limit
+    assert torch.cuda.memory_allocated() <= held + (1 << 20)
+    assert graphs.graph_replays > 100
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("which", ["A", "B"])
 def test_first_tokens_of_a_sequence(tmp_path, which, dtype):
     """Position 0 alone, then 1, 2, 3...: a prompt of one token, portions of one."""
@@ -227,19 +269,13 @@ def test_decode_graphs_of_a_hundred_requests():
     """With matrices large enough for the LDS-staged kernel, decode steps of 65
     to 128 requests hold no library product and replay a graph: same logits as
     the eager steps, and as each request stepped alone."""
-    import os
-    import sys
-    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-    import bench
     from servelab_amd import Qwen2Config
-    from servelab_amd.engine.session import make_runtime
-    from servelab_amd.parts import DecoderModel, build_model_spec
-    raw = dict(bench.QWEN25_7B, num_hidden_layers=1, hidden_size=3072, num_attention_heads=24,
-               num_key_value_heads=4, intermediate_size=3072, vocab_size=4096)
-    rt = make_runtime(torch.bfloat16, "cuda:0")
-    model = DecoderModel(build_model_spec(Qwen2Config.from_hf(raw)), rt)
-    model.load(bench.RandomCheckpoint(model.spec.param_specs(), 5, rt.device, torch.bfloat16))
-    assert rt.ops.graph_rows_limit == 128
+    from servelab_amd.engine.session import random_model_on_device
+    raw = dict(TINY["B"], num_hidden_layers=1, hidden_size=3072, num_attention_heads=24,
+               num_key_value_heads=4, head_dim=128, intermediate_size=3072, vocab_size=4096,
+               use_sliding_window=False, max_position_embeddings=4096)
+    model = random_model_on_device(Qwen2Config.from_hf(raw), 5, "bfloat16")
+    assert model.rt.ops.graph_rows_limit == 128
     B = 100
     rng = random.Random(9)
     prompts = {f"r{i}": [rng.randrange(4096) for _ in range(3 + i % 5)] for i in range(B)}
@@ -296,3 +332,33 @@ def test_many_requests_under_three_regimes_generate_the_same_tokens(tmp_path):
             assert stats["num_preemptions_total"] > 0
     assert results["tight"] == results["roomy"]
     assert results["narrow"] == results["roomy"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_command_line_generates_the_plain_tokens(dtype, capsys):
+    """``run_engine`` itself on the GPU, on its tiny default model with random weights made on the
+    device (examples/run_engine.py:27-72): the printed tokens are the plain implementation's."""
+    import re
+    import servelab_amd.cli as cli
+    from servelab_amd import Qwen2Config
+    from servelab_amd.parts import build_model_spec
+    from servelab_amd.weights import RandomCheckpoint
+    assert cli.main(["--random-weights", "3", "--temperature", "0", "--max-tokens", "10",
+                     "--dtype", dtype, "--num-blocks", "32"]) == 0
+    printed = capsys.readouterr().out
+    got = [int(t) for t in re.search(r"\[req-1\] finish=(\w+) -> \[([0-9, ]+)\]", printed).group(2).split(",")]
+    raw = dict(cli.TINY_DEFAULT)
+    spec = build_model_spec(Qwen2Config.from_hf(raw))
+    weights = {n: t.float().cpu() for n, t in RandomCheckpoint(
+        spec.param_specs(), 3, "cuda:0",
+        torch.float32 if dtype == "float32" else torch.bfloat16).state_dict().items()}
+    prompt = [t % raw["vocab_size"] for t in range(10, 40)]
+    assert "stats:" in printed and "[step 1]" in printed
+    if dtype == "float32":
+        want = plain.greedy_generate(raw, weights, prompt, 10)
+        assert got == want[:len(got)] and (len(got) == 10 or got[-1] == raw["eos_token_id"])
+    else:
+        logits = plain.forward(raw, weights, prompt + got)
+        for i, t in enumerate(got):
+            row = logits[len(prompt) - 1 + i]
+            assert row[t] >= row.max() - 0.02 * row.abs().max(), f"token {i}"

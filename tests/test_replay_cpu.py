@@ -54,3 +54,18 @@ def test_replay_of_the_probe_model_at_every_page_size(tmp_path, page):
                       ops=EmulatedOps(torch.float32), device="cpu", block_size=page)
     worst, where = compare(out, steps, reference, vocab, score=probe_score)
     assert worst <= 0.02, f"score {worst} at {where}"
+
+
+def test_replay_without_attention_bias(tmp_path):
+    folder = make_folder(tmp_path, "B", seed=13, attention_bias=False)
+    from safetensors import safe_open
+    with safe_open(folder + "/model.safetensors", "pt") as f:
+        assert not any(name.endswith("_proj.bias") for name in f.keys())
+    requests = make_requests(TINY["B"]["vocab_size"], [50, 35, 81], seed=9)
+    reference = plain_logits(folder, requests)
+    steps = rs.mixed(requests, {r: len(t) - 8 for r, t in requests.items()}, max_live=2)
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, "float32", rs.max_tokens_needed(steps),
+                      ops=EmulatedOps(torch.float32), device="cpu")
+    worst, where = compare(out, steps, reference, TINY["B"]["vocab_size"])
+    assert worst < 1e-4, f"max abs err {worst} at {where}"

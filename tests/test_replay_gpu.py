@@ -99,3 +99,19 @@ def test_trace_run_program(tmp_path, dtype):
     replay_program(folder, steps, out, dtype, rs.max_tokens_needed(steps))
     worst, where = compare(out, steps, reference, vocab)
     assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_without_attention_bias(tmp_path, dtype):
+    """``attention_bias: false``: q, k and v have no bias tensors at all."""
+    folder = make_folder(tmp_path, "B", seed=13, attention_bias=False)
+    vocab = TINY["B"]["vocab_size"]
+    requests = make_requests(vocab, [50, 35, 81, 120], seed=9)
+    reference = plain_logits(folder, requests)
+    steps = rs.mixed(requests, {r: len(t) - 8 for r, t in requests.items()}, max_live=3)
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, dtype, rs.max_tokens_needed(steps))
+    worst, where = compare(out, steps, reference, vocab)
+    bar = tolerance(dtype, reference) if dtype == "float32" else \
+        bfloat16_bar(folder, requests, reference, vocab, "nobias")
+    assert worst < bar, f"max abs err {worst} at {where}"
