@@ -13,6 +13,8 @@
 // seed and how many tokens it has drawn, not on the batch it is in.  The
 // reference draws from a host generator instead (sampler.py:11-13).
 #include "common.h"
+#include "sampling_api.h"
+#include <mutex>
 
 struct Best { float v; int i; };
 
@@ -546,4 +548,55 @@ extern "C" const char* sl_sample(const float* logits, int R, int V, const float*
   if (e) return e;
   argmax_final_kernel<<<R, 64, 0, stream>>>((const Best*)work, chunks, out);
   return sl_launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// The entry point that allocates nothing (declared and described in
+// sampling_api.h).  `scratch` is a host-side stand-in in host code, not a device
+// address: the address of each GPU's copy is looked up once per device, with
+// that device current, and only that address is ever handed to a kernel.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[SL_SAMPLE_STATIC_BYTES];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static void* scratch_address[STATIC_MAX_DEVICES];     // by device ordinal; nullptr: not looked up yet
+static std::mutex scratch_mutex;
+
+static const char* scratch_of_current_device(void** address) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess) return "sample_static: no current device";
+  SL_CHECK(device >= 0 && device < STATIC_MAX_DEVICES, "sample_static: device ordinal beyond 63");
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_address[device] == nullptr) {
+    void* found = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hipGetErrorString(e);
+    SL_CHECK(found != nullptr, "sample_static: the scratch array has no address on this device");
+    scratch_address[device] = found;
+  }
+  *address = scratch_address[device];
+  return nullptr;
+}
+
+extern "C" const char* sl_sample_static(const float* logits, int R, int V, const float* temperature,
+                                        const int* top_k, const float* top_p, const int64_t* seeds,
+                                        const int64_t* draws, int* out, hipStream_t stream) {
+  SL_CHECK(R >= 0 && V > 0, "sample_static: sizes must be positive");
+  SL_CHECK((top_k == nullptr) == (top_p == nullptr), "sample_static: top_k and top_p go together");
+  if (R == 0) return nullptr;
+  const bool cuts = top_k != nullptr;
+  // slices of about 2,048 logits (4,096 when cuts are searched: every workgroup
+  // adds up the tables of all slices of its row), as the callers of sl_sample choose
+  int chunks = cuts ? V / 4096 : V / 2048;
+  const int most = cuts ? 16 : 64;
+  chunks = chunks < 1 ? 1 : chunks > most ? most : chunks;
+  void* work = nullptr;
+  if (!(cuts && chunks < 2)) {             // (short rows with cuts take one workgroup a row, no scratch)
+    SL_CHECK(sl_sample_workspace(R, chunks, cuts) <= (size_t)SL_SAMPLE_STATIC_BYTES,
+             "sample_static: these rows need more scratch than the static 8 MiB array holds "
+             "(rows x slices x 6,160 bytes with cuts, x 8 without); use sl_sample with a workspace");
+    const char* e = scratch_of_current_device(&work);
+    if (e) return e;
+  }
+  return sl_sample(logits, R, V, temperature, top_k, top_p, seeds, draws, chunks, work, out, stream);
 }

@@ -5,7 +5,7 @@ Each source is a unit of its own: ``hipcc -shared -fPIC`` turns it into one
 dtype (and per the sizes a source takes as macros, such as the head size of the
 matrix-core attention kernels), so the first call for a model compiles what
 that model needs and nothing else.  Libraries are kept beside the sources in
-``csrc/_build/`` under a name that carries a hash of the source, the header and
+``csrc/_build/`` under a name that carries a hash of the source, the headers and
 the flags, so a stale library is never loaded.
 """
 import ctypes
@@ -65,7 +65,8 @@ def build_dir() -> str:
 
 def _digest(u: Unit) -> str:
     h = hashlib.sha256()
-    for name in (u[0] + ".hip", "common.h"):
+    headers = sorted(n for n in os.listdir(CSRC) if n.endswith(".h"))
+    for name in [u[0] + ".hip"] + headers:
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
     h.update(" ".join(BASE_FLAGS + list(u[1])).encode())

@@ -845,3 +845,26 @@ class HipOps:
         self._call("sampling", "sl_sample", _p(logits), R, V, _p(temperature), _p(top_k),
                    _p(top_p), _p(seeds), _p(draws), chunks, _p(work), _p(out))
         return out
+
+    def sample_static(self, logits, temperature=None, top_k=None, top_p=None, seeds=None, draws=None):
+        """``sample`` (or ``argmax`` when ``temperature`` is None) through the
+        library's entry point that allocates nothing: its scratch is a static
+        device array of 8 MiB inside the library, shared by all calls on this
+        GPU, so calls must not overlap on two streams.  Only the result tensor
+        is allocated here; sizes whose scratch would not fit are refused."""
+        R, V = logits.shape
+        self._check(logits, torch.float32, None, "logits")
+        if temperature is not None:
+            self._check(temperature, torch.float32, (R,), "temperature")
+            self._check(seeds, torch.int64, (R,), "seeds")
+            self._check(draws, torch.int64, (R,), "draws")
+        if (top_k is None) != (top_p is None) or (top_k is not None and temperature is None):
+            raise KernelError("sample_static: top_k and top_p go together and need temperatures")
+        if top_k is not None:
+            self._check(top_k, torch.int32, (R,), "top_k")
+            self._check(top_p, torch.float32, (R,), "top_p")
+        out = self._new((R,), torch.int32)
+        self._call("sampling", "sl_sample_static", _p(logits), R, V, _p(temperature), _p(top_k),
+                   _p(top_p), _p(seeds), _p(draws), _p(out))
+        return out
+
