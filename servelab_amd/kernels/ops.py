@@ -120,7 +120,6 @@ class HipOps:
         self._lib = {stem: build.load(build.unit(stem, self.dtype_name))
                      for stem in build.DEFAULT_STEMS}
         self._fn = {}
-        self._bias_cache = {}
         self.use_mfma_attention = True
         self._num_cus = max(1, torch.cuda.get_device_properties(self.device).multi_processor_count)
         self.fuse_norms = act_dtype == torch.bfloat16
@@ -515,24 +514,31 @@ class HipOps:
         self._call("gemm", "sl_gemm_f32_mfma", _p(x), _p(w), _p(bias), _p(y), M, N, K)
         return y
 
-    def linear_library(self, x, w, bias):
+    def library_sums(self, x, w, out_dtype=None):
+        """x w^T by the library, in bfloat16 or (``out_dtype`` float32) with the
+        float32 sums kept.  Fewer than LIBRARY_PADDED_MAX_M rows are padded to a
+        multiple of LIBRARY_ROW_STEP; the rows beyond M hold whatever the buffer
+        held: a row of a product depends on its own row of x only (the library
+        splits no K across rows), and they are cut off."""
         if self.act_dtype != torch.bfloat16:
             raise KernelError("the library GEMM is for the bfloat16 table only")
         M = x.shape[0]
         rows = self.library_rows(M)
         if rows != M:
-            # the rows beyond M hold whatever the buffer held: every row of a
-            # product depends on its own row of x only, and they are cut off below
             padded = self._new((rows, x.shape[1]))
             padded[:M].copy_(x)
             x = padded
-        if bias is None:
+        if out_dtype is None:
             return torch.mm(x, w.t())[:M]
-        entry = self._bias_cache.get(id(bias))       # (the float bias itself, its bfloat16 copy)
-        if entry is None or entry[0] is not bias:
-            entry = (bias, bias.to(torch.bfloat16))
-            self._bias_cache[id(bias)] = entry
-        return torch.addmm(entry[1], x, w.t())[:M]
+        return torch.mm(x, w.t(), out_dtype=out_dtype)[:M]
+
+    def linear_library(self, x, w, bias):
+        """Many rows: the library's product.  A bias is added to the float32
+        sums before the one rounding to bfloat16, as the few-rows kernels do, so
+        that a row gives the same values whichever path its step takes."""
+        if bias is None:
+            return self.library_sums(x, w)
+        return self.library_sums(x, w, torch.float32).add_(bias).to(torch.bfloat16)
 
     @contextlib.contextmanager
     def library_tuning(self, max_ms: int = 30, results_file: Optional[str] = None):
@@ -643,6 +649,16 @@ class HipOps:
                                     True, split=product)
                     return qkv
                 qkv = product
+            elif (self.act_dtype == torch.bfloat16 and not isinstance(x, ScaledRows)
+                    and M > self._few_rows_limit(weight)):
+                # many rows: the library keeps the float32 sums, and the rotation kernel adds the
+                # float32 bias, rotates and rounds once, exactly as the fused few-rows kernel does
+                self._check(x, self.act_dtype, (M, K), "x")
+                sums = self.library_sums(x, self.rows_of(weight), torch.float32)
+                qkv = self._new((M, N))
+                self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                                True, split=PartialSums(sums.unsqueeze(0), bias))
+                return qkv
             else:
                 qkv = self.linear(x, weight, bias)
             self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True)

@@ -460,6 +460,47 @@ def test_qkv_rope_store(M, nh, nkv, D, page, H, pairs):
             assert rel_err(g, r) < 2 ** -5
 
 
+def test_a_row_gives_the_same_keys_whichever_path_its_step_takes():
+    """q/k/v with a bias that bfloat16 cannot hold, for the same 300 rows in one step (library
+    product) and in steps of 8 and of 40 rows (few-rows kernels): every route adds the float32
+    bias to float32 sums and rounds once, so q and the cached K and V agree except where the
+    order of a sum moves a value across a rounding boundary (a fraction of a per cent of the
+    entries, by one step of bfloat16).  Rounding the bias to bfloat16 first, or rounding the
+    product before the bias is added, changes a quarter of the entries."""
+    from servelab_amd.kernels import HipOps
+    dt = torch.bfloat16
+    ops = HipOps(dt, "cuda:0")
+    nh, nkv, D, page, H, M = 8, 2, 64, 16, 3072, 300       # 768 x 3072 = 2.4 M elements: library above 64 rows
+    N = (nh + 2 * nkv) * D
+    x = randn(M, H, dtype=dt, seed=1)
+    w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.02, seed=2))
+    bias = (randn(N, scale=2.0, seed=3) * 1.001).contiguous()
+    assert (bias.bfloat16().float() != bias).float().mean() > 0.9
+    inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
+    emu = EmulatedOps(dt)
+    cos, sin = emu.rope_tables(torch.arange(M, dtype=torch.int32).cuda(), inv)
+    pages = -(-M // page)
+    slots = torch.randperm(pages * page)[:M].to(torch.int32).cuda()
+
+    def run(rows_per_step):
+        kc = torch.zeros(pages, nkv, page, D, dtype=dt, device="cuda")
+        vc = torch.zeros(pages, nkv, D, page, dtype=dt, device="cuda")
+        q = []
+        for a in range(0, M, rows_per_step):
+            b = min(M, a + rows_per_step)
+            qkv = ops.qkv_rope_store(x[a:b].contiguous(), w, bias, nh, nkv, D, cos[a:b].contiguous(),
+                                     sin[a:b].contiguous(), slots[a:b].contiguous(), kc, vc, page)
+            q.append(qkv[:, :nh * D].float())
+        return torch.cat(q), kc.float(), vc.float()
+    assert ops._few_rows_limit(w) == 64
+    whole, by8, by40 = run(M), run(8), run(40)
+    for other in (by8, by40):
+        for a, b in zip(whole, other):
+            differ = (a != b).float().mean().item()
+            assert differ < 0.01, differ
+            assert ((a - b).abs() <= 2 ** -7 * a.abs().clamp_min(2 ** -6)).all()
+
+
 def make_attention_case(dt, nh, nkv, D, page, seqs, seed=0):
     """``seqs``: list of (context length after the step, query length).  Builds
     a cache with shuffled pages and garbage in unused rows."""
