@@ -118,16 +118,17 @@ extern "C" const char* sl_rope_tables(const int* pos, const float* inv_freq, flo
 }
 
 // ------------------------------------------------- rotary + write to pages
-// qkv rows are [q heads | k heads | v heads], head-major.  q and k are rotated
-// in place with pairs (j, j + D/2) (servelab/parallel/tp_model.py:128); the
+// qkv rows are [q heads | k heads | v heads], head-major.  The first `rot`
+// channels of every q and k head are rotated in place with pairs (j, j + rot/2)
+// (rot = D: servelab/parallel/tp_model.py:128; tables [T, rot/2]); the
 // rotated k and the v of each token go to its cache row (:129,
 // servelab/kv_cache/pool.py:68-78): K pages [page, nkv, page_size, D], V pages
 // [page, nkv, D, page_size].  One block per (token, head).
 //
 // pairs8: the channels of every q and k head come in the order the fused
-// few-rows product wants them (gemm.hip): blocks of 16 that hold channels
-// 8b..8b+7 followed by their partners D/2+8b..D/2+8b+7, so that pair j sits at
-// 16 (j / 8) + j % 8 and 8 further.  Scores do not depend on the order of the
+// few-rows product wants them (gemm.hip): the rotated channels in blocks of 16
+// that hold channels 8b..8b+7 followed by their partners rot/2+8b..rot/2+8b+7,
+// so that pair j sits at 16 (j / 8) + j % 8 and 8 further; then the rest.  Scores do not depend on the order of the
 // channels as long as q and the cached k agree; v keeps its order.
 // The float partial sums of a q/k/v product whose K was split over workgroups
 // ([nparts][T][N], bias not yet added): the kernel below then reads its input
@@ -144,9 +145,9 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const SplitProduct sp
                                   const float* __restrict__ cosv,
                                   const float* __restrict__ sinv, const int* __restrict__ slots,
                                   act_t* __restrict__ kc, act_t* __restrict__ vc, int nh, int nkv,
-                                  int D, int page, int pairs8) {
+                                  int D, int rot, int page, int pairs8) {
   const int t = blockIdx.x, hd = blockIdx.y;
-  const int half = D / 2;
+  const int half = rot / 2;
   const size_t row = ((size_t)t * (nh + 2 * nkv) + hd) * D;
   act_t* x = qkv + row;
   auto input = [&](int c) {
@@ -181,6 +182,11 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const SplitProduct sp
         dst[p2] = from_f<act_t>(x2);
       }
     }
+    for (int c = rot + threadIdx.x; c < D; c += blockDim.x) {       // channels beyond the rotated ones pass
+      const float v = input(c);
+      if (sp.parts != nullptr && hd < nh) x[c] = from_f<act_t>(v);
+      if (dst != nullptr) dst[c] = from_f<act_t>(v);
+    }
   } else if (vc != nullptr) {
     const int slot = slots[t];
     act_t* dst = vc + ((size_t)(slot / page) * nkv + (hd - nh - nkv)) * D * page + slot % page;
@@ -201,16 +207,18 @@ struct __attribute__((aligned(16))) F4 { float v[4]; };
 // one token and writes them back, k also to its cache row.
 __global__ __launch_bounds__(256) void rope_store_qk_kernel(
     act_t* __restrict__ qkv, const float* __restrict__ cosv, const float* __restrict__ sinv,
-    const int* __restrict__ slots, act_t* __restrict__ kc, int nh, int nkv, int D, int page,
-    int pairs8) {
-  const int t = blockIdx.x, half = D / 2, chunks = half / 8;
+    const int* __restrict__ slots, act_t* __restrict__ kc, int nh, int nkv, int D, int rot,
+    int page, int pairs8) {
+  const int t = blockIdx.x, half = rot / 2, chunks = D / 16, rotated = rot / 16;
   const int items = (nh + nkv) * chunks;
   for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < items; w += gridDim.y * blockDim.x) {
     const int hd = w / chunks, c = w % chunks;
-    const int p1 = pairs8 ? 16 * c : 8 * c, p2 = pairs8 ? p1 + 8 : p1 + half;
+    // chunks below `rotated` hold 8 pairs; the others 16 channels that pass unrotated
+    const bool turn = c < rotated;
+    const int p1 = !turn || pairs8 ? 16 * c : 8 * c, p2 = !turn || pairs8 ? p1 + 8 : p1 + half;
     act_t* x = qkv + ((size_t)t * (nh + 2 * nkv) + hd) * D;
     Act8 a = *(const Act8*)(x + p1), b = *(const Act8*)(x + p2);
-    if (cosv != nullptr) {
+    if (cosv != nullptr && turn) {
       const float* cp = cosv + (size_t)t * half + 8 * c;
       const float* sp = sinv + (size_t)t * half + 8 * c;
       const F4 c0 = *(const F4*)cp, c1 = *(const F4*)(cp + 4);
@@ -263,11 +271,13 @@ __global__ __launch_bounds__(256) void store_v_kernel(
 // [nparts][T][N] plus bias; q is then written to qkv, k and v only to the pages.
 extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* sinv,
                                      const int* slots, void* kc, void* vc, int T, int nh, int nkv,
-                                     int D, int page, int pairs8, const float* parts, int nparts,
-                                     const float* bias, hipStream_t stream) {
+                                     int D, int rot, int page, int pairs8, const float* parts,
+                                     int nparts, const float* bias, hipStream_t stream) {
   SL_CHECK(T >= 0 && nh > 0 && nkv > 0, "rope_store: sizes must be positive");
-  SL_CHECK(D > 0 && D % 2 == 0, "rope_store: head_dim must be even");
-  SL_CHECK(!pairs8 || D % 16 == 0, "rope_store: the blocked pair order needs head_dim % 16 == 0");
+  SL_CHECK(D > 0 && rot >= 0 && rot <= D && rot % 2 == 0,
+           "rope_store: the rotated width must be even and at most head_dim");
+  SL_CHECK(cosv == nullptr || rot > 0, "rope_store: tables given but no channel is rotated");
+  SL_CHECK(!pairs8 || rot % 16 == 0, "rope_store: the blocked pair order needs a rotated width % 16 == 0");
   SL_CHECK((cosv == nullptr) == (sinv == nullptr), "rope_store: cos and sin go together");
   SL_CHECK((kc == nullptr) == (vc == nullptr), "rope_store: k and v pages go together");
   SL_CHECK(kc == nullptr || (slots != nullptr && page > 0), "rope_store: pages need slots");
@@ -279,10 +289,11 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
   if (cosv == nullptr && kc == nullptr && parts == nullptr) return nullptr;
   const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kc % 16) == 0 &&
                        ((uintptr_t)cosv % 16) == 0 && ((uintptr_t)sinv % 16) == 0;
-  if (parts == nullptr && T >= VECTOR_MIN_TOKENS && D % 16 == 0 && D <= 256 && aligned && nkv <= 65535) {
+  if (parts == nullptr && T >= VECTOR_MIN_TOKENS && D % 16 == 0 && rot % 16 == 0 && D <= 256 && aligned &&
+      nkv <= 65535) {
     const int items = (nh + nkv) * (D / 16);
     rope_store_qk_kernel<<<dim3(T, (items + 255) / 256 < 64 ? (items + 255) / 256 : 64), 256, 0, stream>>>(
-        (act_t*)qkv, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, page, pairs8);
+        (act_t*)qkv, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, rot, page, pairs8);
     const char* e = sl_launch_status();
     if (e || vc == nullptr) return e;
     store_v_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>((const act_t*)qkv, slots, (act_t*)vc, T,
@@ -290,6 +301,6 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
     return sl_launch_status();
   }
   rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, sp, cosv, sinv, slots, (act_t*)kc,
-                                                       (act_t*)vc, nh, nkv, D, page, pairs8);
+                                                       (act_t*)vc, nh, nkv, D, rot, page, pairs8);
   return sl_launch_status();
 }

@@ -356,18 +356,20 @@ struct NormFusion {
 
 // Rotary embedding and the write to the cache pages fused into the q/k/v
 // product (ROPE): the rows of W are ordered so that a tile of 16 result columns
-// of a q or k head holds channels 8b..8b+7 and their partners D/2+8b..D/2+8b+7;
+// of a q or k head holds channels 8b..8b+7 and their partners rot/2+8b..rot/2+8b+7
+// (rot: the rotated width, the whole head for Qwen2; tiles beyond it pass unrotated);
 // the epilogue rotates each pair, writes q into the result buffer and the
 // rotated k and the v of token m into the cache row slots[m]
 // (servelab/parallel/tp_model.py:128-129).  q and the cached k keep that
 // channel order (scores do not depend on it); v is in its own order.
 struct RopeStore {
-  const float* cosv;         // [M, D / 2] or nullptr (no rotation)
+  const float* cosv;         // [M, rot / 2] or nullptr (no rotation)
   const float* sinv;
   const int* slots;          // [M] cache rows, or nullptr (nothing is written)
   __bf16* kc;                // [pages, nkv, page, D]
   __bf16* vc;                // [pages, nkv, D, page]
   int nh, nkv, D, page;
+  int rot;                   // the first rot channels of a head are rotated (rot % 16 == 0), the rest pass
 };
 
 // NT tiles (16 columns of y each) per workgroup share every load of x: with 8
@@ -519,8 +521,8 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
         const int hd = n / R.D, p = n % R.D;
         if (hd < R.nh + R.nkv) {
           float val = s;
-          if (R.cosv != nullptr) {
-            const int j = 8 * (p / 16) + p % 8, half = R.D / 2;
+          if (R.cosv != nullptr && p < R.rot) {
+            const int j = 8 * (p / 16) + p % 8, half = R.rot / 2;
             const float c = R.cosv[(size_t)m * half + j], sn = R.sinv[(size_t)m * half + j];
             val = p % 16 < 8 ? s * c - partner * sn : s * c + partner * sn;
           }
@@ -592,6 +594,8 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
     SL_CHECK(R.D % 16 == 0 && R.nh > 0 && R.nkv > 0 && N == (R.nh + 2 * R.nkv) * R.D,
              "gemm_skinny: q/k/v columns must be (heads + 2 kv heads) * head_dim, head_dim % 16 == 0");
     SL_CHECK((R.cosv == nullptr) == (R.sinv == nullptr), "gemm_skinny: cos and sin go together");
+    SL_CHECK(R.rot >= 0 && R.rot <= R.D && R.rot % 16 == 0 && (R.cosv == nullptr || R.rot > 0),
+             "gemm_skinny: the rotated width must be a multiple of 16, at most head_dim");
     SL_CHECK(R.slots == nullptr || (R.kc != nullptr && R.vc != nullptr && R.page > 0),
              "gemm_skinny: cache rows need the pages");
     const dim3 grid2(((N + 15) / 16 + 1) / 2);

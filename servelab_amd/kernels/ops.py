@@ -40,7 +40,22 @@ def _ptr(t: Optional[torch.Tensor]):
 class _RopeStore(ctypes.Structure):
     """``RopeStore`` of gemm.hip."""
     _fields_ = [("cosv", _c_void_p), ("sinv", _c_void_p), ("slots", _c_void_p), ("kc", _c_void_p),
-                ("vc", _c_void_p), ("nh", _c_int), ("nkv", _c_int), ("D", _c_int), ("page", _c_int)]
+                ("vc", _c_void_p), ("nh", _c_int), ("nkv", _c_int), ("D", _c_int), ("page", _c_int),
+                ("rot", _c_int)]
+
+
+class RotationPlan:
+    """How the kernels of this table want the q and k channels of a head laid
+    out for a position encoding, decided once at load (``plan_rotation``):
+    ``order`` is the permutation the mixer applies to the rows of its q and k
+    matrices and biases (new channel i is old channel ``order[i]``; None: as
+    they are), ``rot_dim`` how many leading channels are rotated, ``blocked``
+    whether the rotated channels lie in blocks of 8 followed by their 8
+    partners (what the fused q/k/v kernel rotates) or as first and second half."""
+    __slots__ = ("order", "rot_dim", "blocked")
+
+    def __init__(self, order, rot_dim, blocked):
+        self.order, self.rot_dim, self.blocked = order, int(rot_dim), bool(blocked)
 
 
 class LinearWeight:
@@ -598,14 +613,19 @@ class HipOps:
         return pages
 
     def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                   pairs8=False, split=None):
+                   pairs8=False, split=None, rot_dim=None):
         """Rotate q and k of ``qkv`` in place (``cos`` None: no rotation) and write
-        k and v to their cache rows (``k_cache`` None: no write).  ``pairs8``:
-        the channels of q and k heads come in blocks of 8 channels and their 8
-        partners (the order ``qkv_rope_store`` uses), else first and second half.
+        k and v to their cache rows (``k_cache`` None: no write).  The first
+        ``rot_dim`` channels of a head are rotated (default: all), pair j being
+        (j, j + rot_dim / 2); ``pairs8``: they come in blocks of 8 channels and
+        their 8 partners (the order ``qkv_rope_store`` uses) instead.
         ``split``: the product arrives as ``PartialSums``; ``qkv`` is then only
         written (its q columns)."""
         T = qkv.shape[0]
+        rot = D if rot_dim is None else int(rot_dim)
+        if rot % 2 or not 0 <= rot <= D or (pairs8 and rot % 16) or (cos is not None and rot == 0):
+            raise KernelError(f"rope_store: cannot rotate {rot} of {D} channels"
+                              + (" in blocks of 8 pairs" if pairs8 else ""))
         self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
         parts = bias = None
         if split is not None:
@@ -614,17 +634,17 @@ class HipOps:
             if bias is not None:
                 self._check(bias, torch.float32, ((nh + 2 * nkv) * D,), "bias")
         if cos is not None:
-            self._check(cos, torch.float32, (T, D // 2), "cos")
-            self._check(sin, torch.float32, (T, D // 2), "sin")
+            self._check(cos, torch.float32, (T, rot // 2), "cos")
+            self._check(sin, torch.float32, (T, rot // 2), "sin")
         if k_cache is not None:
             self._check_pages(k_cache, v_cache, nkv, D, page_size)
             self._check(slots, torch.int32, (T,), "slots")
         self._call("elementwise", "sl_rope_store", _p(qkv), _p(cos), _p(sin), _p(slots),
-                   _p(k_cache), _p(v_cache), T, nh, nkv, D, page_size, int(pairs8),
+                   _p(k_cache), _p(v_cache), T, nh, nkv, D, rot, page_size, int(pairs8),
                    _p(parts), parts.shape[0] if parts is not None else 0, _p(bias))
 
     def qkv_rope_store(self, x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
-                       page_size):
+                       page_size, rot_dim=None):
         """q/k/v product, rotation and cache write.  The rows of ``weight`` (and
         ``bias``) hold every q and k head in the blocked pair order (``pairs8``
         above).  Returns the [T, (nh + 2 nkv) D] buffer whose q columns the
@@ -634,8 +654,10 @@ class HipOps:
             weight = LinearWeight(weight)
         M, K = x.shape
         N = weight.shape[0]
-        if N != (nh + 2 * nkv) * D or D % 16:
-            raise KernelError("qkv_rope_store: weight rows must be (nh + 2 nkv) * D with D % 16 == 0")
+        rot = D if rot_dim is None else int(rot_dim)
+        if N != (nh + 2 * nkv) * D or D % 16 or rot % 16 or not 0 <= rot <= D:
+            raise KernelError("qkv_rope_store: weight rows must be (nh + 2 nkv) * D with D % 16 == 0, "
+                              "the rotated width a multiple of 16")
         fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
                  and weight.tiled is not None and weight.shape == (N, K))
         if not fused:
@@ -646,7 +668,7 @@ class HipOps:
                 if isinstance(product, PartialSums):
                     qkv = self._new((M, N))
                     self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                                    True, split=product)
+                                    True, split=product, rot_dim=rot)
                     return qkv
                 qkv = product
             elif (self.act_dtype == torch.bfloat16 and not isinstance(x, ScaledRows)
@@ -657,11 +679,12 @@ class HipOps:
                 sums = self.library_sums(x, self.rows_of(weight), torch.float32)
                 qkv = self._new((M, N))
                 self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                                True, split=PartialSums(sums.unsqueeze(0), bias))
+                                True, split=PartialSums(sums.unsqueeze(0), bias), rot_dim=rot)
                 return qkv
             else:
                 qkv = self.linear(x, weight, bias)
-            self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True)
+            self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True,
+                            rot_dim=rot)
             return qkv
         scaled = x if isinstance(x, ScaledRows) else None
         if scaled is None:
@@ -669,16 +692,68 @@ class HipOps:
         if bias is not None:
             self._check(bias, torch.float32, (N,), "bias")
         if cos is not None:
-            self._check(cos, torch.float32, (M, D // 2), "cos")
-            self._check(sin, torch.float32, (M, D // 2), "sin")
+            self._check(cos, torch.float32, (M, rot // 2), "cos")
+            self._check(sin, torch.float32, (M, rot // 2), "sin")
         if k_cache is not None:
             self._check_pages(k_cache, v_cache, nkv, D, page_size)
             self._check(slots, torch.int32, (M,), "slots")
         rope = _RopeStore(_ptr(cos), _ptr(sin), _ptr(slots if k_cache is not None else None),
-                          _ptr(k_cache), _ptr(v_cache), nh, nkv, D, page_size)
+                          _ptr(k_cache), _ptr(v_cache), nh, nkv, D, page_size, rot)
         qkv = self._new((M, N))
         self._skinny(scaled.x if scaled is not None else x, weight, bias, qkv, M, N, K,
                      scaled=scaled, rope=rope)
+        return qkv
+
+    # --------------------------------------------- position encodings of a mixer
+    def plan_rotation(self, head_dim, layout) -> RotationPlan:
+        """The channel order of q and k heads for a position encoding whose
+        ``layout`` is None (nothing is rotated) or says ``rot_dim`` (the leading
+        channels that are rotated) and ``pairing``: "half" pairs channel j with
+        j + rot_dim / 2, "interleaved" 2j with 2j + 1.  Scores do not depend on
+        the order of the channels as long as q and the cached k agree, so an
+        interleaved pairing is turned into halves by the order alone, and the
+        rotated channels are laid out in blocks of 8 and their 8 partners where
+        the fused q/k/v kernel can take them (head size and rotated width
+        multiples of 16)."""
+        D = int(head_dim)
+        rot = 0 if layout is None else int(layout.rot_dim)
+        pairing = "half" if layout is None else layout.pairing
+        if rot % 2 or not 0 <= rot <= D:
+            raise KernelError(f"a rotation of {rot} of {D} channels has no kernel: the width must be even")
+        if pairing not in ("half", "interleaved"):
+            raise KernelError(f"pairing '{pairing}' has no kernel (half or interleaved)")
+        order = list(range(D))
+        if pairing == "interleaved":
+            order[:rot] = list(range(0, rot, 2)) + list(range(1, rot, 2))
+        blocked = D % 16 == 0 and rot % 16 == 0
+        if blocked and rot:
+            halves = order[:rot]
+            order[:rot] = [halves[(i % 16 >= 8) * (rot // 2) + 8 * (i // 16) + i % 8] for i in range(rot)]
+        plain = order == list(range(D))
+        return RotationPlan(None if plain else torch.tensor(order, dtype=torch.long), rot, blocked)
+
+    def project_qkv(self, x, weight, bias, nh, nkv, D, plan, tables, slots, k_cache, v_cache,
+                    page_size):
+        """What a mixer calls: the q/k/v product of ``x`` (rows of ``weight`` in
+        the order of ``plan``), the position encoding's work on q and k for this
+        step's ``tables`` (whatever the encoding's ``tables()`` returned: None,
+        or an object with ``cos`` and ``sin`` [T, rot_dim / 2]) and the write of
+        k and v into the cache.  Returns [T, (nh + 2 nkv) D] whose q columns the
+        attention reads."""
+        cos = sin = None
+        if tables is not None:
+            cos, sin = getattr(tables, "cos", None), getattr(tables, "sin", None)
+            if cos is None or sin is None:
+                raise KernelError(f"position tables of type {type(tables).__name__} have no kernel: "
+                                  "this table rotates channel pairs by cos and sin and nothing else")
+            if plan.rot_dim == 0:
+                raise KernelError("the position encoding gives tables but its layout rotates nothing")
+        if plan.blocked:
+            return self.qkv_rope_store(x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
+                                       page_size, rot_dim=plan.rot_dim)
+        qkv = self.linear(x, weight, bias)
+        self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                        rot_dim=plan.rot_dim)
         return qkv
 
     # ------------------------------------------------------------ attention

@@ -1,5 +1,5 @@
 from .base import (Block, FeedForward, Mixer, Norm, PagedKVSpec, ParamSpec, Part,
-                   PositionEncoding, Runtime, StateSpec, prefixed)
+                   PositionEncoding, RotaryLayout, RotaryTables, Runtime, StateSpec, prefixed)
 from .norm import RMSNorm
 from .position import NoPosition, RotaryPosition
 from .attention import PagedAttention

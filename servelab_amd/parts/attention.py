@@ -5,7 +5,8 @@ Reference math: q/k/v projections with optional bias, head-major views
 (:128-129); per sequence scores * 1/sqrt(D), causal mask, softmax and PV in
 float32 with kv head = head // g (:136-157).  The reference runs three GEMMs
 and a Python loop over sequences; here q, k and v come from one GEMM over the
-row-concatenated weight, one kernel rotates and writes the pages, and one call
+row-concatenated weight, the kernel table applies the position encoding (a
+parameter this mixer never looks inside) and writes the pages, and one call
 attends for all sequences of the batch through their block tables.  The
 window (keys p - W < r <= p) is this build's own.
 """
@@ -54,19 +55,17 @@ class PagedAttention(Mixer):
     def load(self, tensors, rt):
         self.rt = rt
         self.position.load(tensors, rt)
-        # [Wq; Wk; Wv] -> one [(nh + 2 nkv) D, H] matrix, one GEMM.  When the head
-        # size allows, the channels of every q and k head are reordered into
-        # blocks of 8 channels followed by their 8 rotation partners (what the
-        # fused product + rotation + cache write of the kernel table wants);
-        # q . k does not depend on the order, v keeps its own.
-        self.pairs8 = self.head_dim % 16 == 0 and hasattr(rt.ops, "qkv_rope_store")
-        d, half = self.head_dim, self.head_dim // 2
+        # [Wq; Wk; Wv] -> one [(nh + 2 nkv) D, H] matrix, one GEMM.  The kernel table says in
+        # which order it wants the channels of every q and k head for this position encoding
+        # (q . k does not depend on the order as long as both agree); v keeps its own.
+        self.rotation = rt.ops.plan_rotation(self.head_dim, self.position.layout())
+        order = self.rotation.order
 
         def reorder(t, heads):
-            if not self.pairs8:
+            if order is None:
                 return t
-            blocks = t.reshape(heads, 2, half // 8, 8, *t.shape[1:])      # [head, half, block, 8, ...]
-            return blocks.transpose(1, 2).reshape(t.shape)               # [head, block, half, 8, ...]
+            by_head = t.reshape(heads, self.head_dim, *t.shape[1:])
+            return by_head[:, order.to(t.device)].reshape(t.shape)
         self.w_qkv = rt.linear_weight(torch.cat(
             [reorder(tensors("q_proj.weight"), self.num_heads),
              reorder(tensors("k_proj.weight"), self.num_kv_heads), tensors("v_proj.weight")], 0))
@@ -81,17 +80,11 @@ class PagedAttention(Mixer):
     # ---- compute
     def forward(self, x, batch, cache, shared):
         ops = self.rt.ops
-        tables = self.position.tables(batch, shared)
-        cos, sin = tables if tables is not None else (None, None)
         group = batch.groups[cache.group]
         slots, kc, vc = (group.slots, cache.k, cache.v) if cache.write else (None, None, None)
-        if self.pairs8:
-            qkv = ops.qkv_rope_store(x, self.w_qkv, self.b_qkv, self.num_heads, self.num_kv_heads,
-                                     self.head_dim, cos, sin, slots, kc, vc, cache.page_size)
-        else:
-            qkv = ops.linear(x, self.w_qkv, self.b_qkv)
-            ops.rope_store(qkv, self.num_heads, self.num_kv_heads, self.head_dim, cos, sin,
-                           slots, kc, vc, cache.page_size)
+        qkv = ops.project_qkv(x, self.w_qkv, self.b_qkv, self.num_heads, self.num_kv_heads,
+                              self.head_dim, self.rotation, self.position.tables(batch, shared),
+                              slots, kc, vc, cache.page_size)
         attn = ops.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
             cache.page_size, group.block_tables, batch, self.scale, self.window)

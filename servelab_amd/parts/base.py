@@ -102,10 +102,34 @@ class Norm(Part):
         raise NotImplementedError
 
 
+@dataclass(frozen=True)
+class RotaryLayout:
+    """Which channels of a head a rotary encoding turns: the first ``rot_dim``
+    (the rest pass), in pairs (j, j + rot_dim / 2) ("half") or (2j, 2j + 1)
+    ("interleaved")."""
+    rot_dim: int
+    pairing: str = "half"
+
+
+@dataclass
+class RotaryTables:
+    """A rotary encoding's work for one step: cos and sin of every token's
+    angles, float32 [T, rot_dim / 2]."""
+    cos: torch.Tensor
+    sin: torch.Tensor
+
+
 class PositionEncoding(Part):
-    """A parameter of a mixer.  ``tables(batch, shared)`` returns what the
-    mixer's kernels need for this step's positions; ``shared`` is a per-step
-    dict so that equal encodings in many layers are prepared once."""
+    """A parameter of a mixer, which never looks inside it.  ``layout()`` says
+    at load time what the encoding does to the channels of a head (None:
+    nothing; a ``RotaryLayout``), from which the kernel table decides the
+    channel order it wants; ``tables(batch, shared)`` returns what the kernels
+    need for this step's positions (None, or ``RotaryTables``), which the mixer
+    hands to the kernel table as it is.  ``shared`` is a per-step dict so that
+    equal encodings in many layers are prepared once."""
+
+    def layout(self):
+        return None
 
     def tables(self, batch, shared):
         raise NotImplementedError

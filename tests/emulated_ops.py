@@ -62,24 +62,27 @@ class EmulatedOps:
         return torch.cos(ang), torch.sin(ang)
 
     def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                   pairs8=False):
-        """Rotate q and k of ``qkv`` in place; write k and v to their pages.
-        ``pairs8``: q and k heads hold blocks of 8 channels and their 8 partners
+                   pairs8=False, rot_dim=None):
+        """Rotate the first ``rot_dim`` channels (default: all) of the q and k
+        heads of ``qkv`` in place; write k and v to their pages.  ``pairs8``:
+        the rotated channels come in blocks of 8 channels and their 8 partners
         (channel order [block][half][8]) instead of first half, second half."""
         T = qkv.shape[0]
-        half = D // 2
+        R = D if rot_dim is None else rot_dim
+        half = R // 2
         qk = qkv[:, :(nh + nkv) * D].view(T, nh + nkv, D)
         if cos is not None:
+            turned = qk[..., :R]
             if pairs8:
-                std = qk.reshape(T, nh + nkv, half // 8, 2, 8).transpose(2, 3).reshape(T, nh + nkv, D)
+                std = turned.reshape(T, nh + nkv, half // 8, 2, 8).transpose(2, 3).reshape(T, nh + nkv, R)
             else:
-                std = qk
+                std = turned
             x1, x2 = _f(std[..., :half]), _f(std[..., half:])
             c, s = cos[:, None, :], sin[:, None, :]
             rot = torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], -1).to(qkv.dtype)
             if pairs8:
-                rot = rot.reshape(T, nh + nkv, 2, half // 8, 8).transpose(2, 3).reshape(T, nh + nkv, D)
-            qk.copy_(rot)
+                rot = rot.reshape(T, nh + nkv, 2, half // 8, 8).transpose(2, 3).reshape(T, nh + nkv, R)
+            turned.copy_(rot)
         if k_cache is None:
             return
         k = qkv[:, nh * D:(nh + nkv) * D].view(T, nkv, D)
@@ -88,9 +91,30 @@ class EmulatedOps:
         k_cache[page, :, off, :] = k.to(k_cache.dtype)
         v_cache[page, :, :, off] = v.to(v_cache.dtype)
 
-    def qkv_rope_store(self, x, w, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size):
+    def qkv_rope_store(self, x, w, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                       rot_dim=None):
         qkv = self.linear(x, w, bias)
-        self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True)
+        self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True, rot_dim)
+        return qkv
+
+    # --------------------------------------------- position encodings of a mixer
+    def plan_rotation(self, head_dim, layout):
+        """Channels stay as the checkpoint has them, except that an interleaved
+        pairing is turned into halves (written independently of the kernel
+        table's own: no blocks of 8 here)."""
+        import types
+        rot = 0 if layout is None else layout.rot_dim
+        order = None
+        if layout is not None and layout.pairing == "interleaved":
+            order = torch.cat([torch.arange(0, rot, 2), torch.arange(1, rot, 2),
+                               torch.arange(rot, head_dim)])
+        return types.SimpleNamespace(order=order, rot_dim=rot, blocked=False)
+
+    def project_qkv(self, x, w, bias, nh, nkv, D, plan, tables, slots, k_cache, v_cache, page_size):
+        qkv = self.linear(x, w, bias)
+        cos, sin = (tables.cos, tables.sin) if tables is not None else (None, None)
+        self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, False,
+                        plan.rot_dim)
         return qkv
 
     # ------------------------------------------------------------ attention

@@ -382,6 +382,61 @@ def test_rope_store(both, nh, nkv, D, page, pairs8, T):
     assert torch.equal(kc[0], k_before)
 
 
+@pytest.mark.parametrize("T", [9, 300])
+@pytest.mark.parametrize("nh,nkv,D,rot,page,pairs8", [(4, 2, 32, 16, 16, True), (4, 2, 32, 16, 16, False),
+                                                      (6, 1, 48, 32, 32, True), (3, 3, 24, 10, 16, False),
+                                                      (2, 1, 128, 64, 64, True), (5, 1, 64, 0, 16, True)])
+def test_rope_store_of_a_part_of_the_head(both, nh, nkv, D, rot, page, pairs8, T):
+    """Only the first ``rot`` channels of every q and k head turn (tables [T, rot / 2]); the rest
+    pass, to the buffer and to the pages; rot = 0 turns nothing and still writes the pages."""
+    ops, emu, dt = both
+    pages = 30
+    qkv = randn(T, (nh + 2 * nkv) * D, dtype=dt, seed=1)
+    cos = sin = None
+    if rot:
+        inv = (1.0 / 10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot)).cuda()
+        cos, sin = emu.rope_tables(torch.arange(100, 100 + T, dtype=torch.int32).cuda(), inv)
+    slots = torch.randperm(pages * page)[:T].to(torch.int32).cuda()
+    kc = [randn(pages, nkv, page, D, dtype=dt, seed=7) for _ in range(2)]
+    vc = [randn(pages, nkv, D, page, dtype=dt, seed=8) for _ in range(2)]
+    q1, q2 = qkv.clone(), qkv.clone()
+    ops.rope_store(q1, nh, nkv, D, cos, sin, slots, kc[0], vc[0], page, pairs8, rot_dim=rot)
+    emu.rope_store(q2, nh, nkv, D, cos, sin, slots, kc[1], vc[1], page, pairs8, rot_dim=rot)
+    assert rel_err(q1, q2) < ELEM_TOL[dt] * 2
+    assert rel_err(kc[0], kc[1]) < ELEM_TOL[dt] * 2
+    assert torch.equal(vc[0], vc[1])
+    heads = q1[:, :(nh + nkv) * D].view(T, nh + nkv, D)
+    assert torch.equal(heads[..., rot:], qkv[:, :(nh + nkv) * D].view(T, nh + nkv, D)[..., rot:])
+    with pytest.raises(Exception, match="rotate"):
+        ops.rope_store(q1, nh, nkv, D, cos, sin, slots, kc[0], vc[0], page, pairs8, rot_dim=D + 2)
+
+
+def test_rotation_plans():
+    """The channel order the kernel table asks a mixer for: identity when nothing turns or the
+    width is no multiple of 16, blocks of 8 and partners otherwise, interleaved pairs first
+    gathered into halves; a permutation in every case, the unrotated channels in place."""
+    import types
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.bfloat16, "cuda:0")
+    lay = lambda rot, pairing="half": types.SimpleNamespace(rot_dim=rot, pairing=pairing)
+    assert ops.plan_rotation(64, None).order is None and ops.plan_rotation(64, None).rot_dim == 0
+    plan = ops.plan_rotation(24, lay(10))
+    assert plan.order is None and not plan.blocked and plan.rot_dim == 10
+    plan = ops.plan_rotation(32, lay(32))
+    assert plan.blocked and plan.order.tolist() == (list(range(0, 8)) + list(range(16, 24)) +
+                                                    list(range(8, 16)) + list(range(24, 32)))
+    plan = ops.plan_rotation(48, lay(16, "interleaved"))
+    assert plan.order.tolist() == [0, 2, 4, 6, 8, 10, 12, 14, 1, 3, 5, 7, 9, 11, 13, 15] + list(range(16, 48))
+    plan = ops.plan_rotation(16, lay(6, "interleaved"))
+    assert plan.order.tolist() == [0, 2, 4, 1, 3, 5] + list(range(6, 16)) and not plan.blocked
+    for bad in (lay(7), lay(40), lay(8, "quads")):
+        with pytest.raises(Exception, match="no kernel"):
+            ops.plan_rotation(32, bad)
+    with pytest.raises(Exception, match="no kernel"):
+        ops.project_qkv(None, None, None, 4, 2, 32, ops.plan_rotation(32, lay(32)), object(),
+                        None, None, None, 16)
+
+
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (28, 4, 128, 16), (5, 1, 48, 32)])
 def test_rope_store_from_partial_sums(both, nh, nkv, D, page):
     """The q/k/v product arrives as float partial sums of a split K plus a bias:
@@ -413,9 +468,11 @@ def test_rope_store_from_partial_sums(both, nh, nkv, D, page):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 40])
-@pytest.mark.parametrize("nh,nkv,D,page,H", [(4, 2, 16, 16, 64), (28, 4, 128, 16, 256), (5, 1, 48, 32, 96)])
+@pytest.mark.parametrize("nh,nkv,D,page,H,rot", [(4, 2, 16, 16, 64, 16), (28, 4, 128, 16, 256, 128),
+                                                 (5, 1, 48, 32, 96, 48), (5, 1, 48, 32, 96, 16),
+                                                 (6, 2, 64, 16, 128, 32)])
 @pytest.mark.parametrize("pairs", [False, True])
-def test_qkv_rope_store(M, nh, nkv, D, page, H, pairs):
+def test_qkv_rope_store(M, nh, nkv, D, page, H, rot, pairs):
     """Product + rotation + cache write: the one fused kernel (at most 16 rows)
     and the product followed by rope_store give the same q, K pages and V
     pages; also with un-normalised input rows and with no rotation or no write;
@@ -430,7 +487,7 @@ def test_qkv_rope_store(M, nh, nkv, D, page, H, pairs):
     x = randn(M, H, dtype=dt, seed=1)
     w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.1, seed=2))
     bias = randn(N, scale=0.1, seed=3)
-    inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
+    inv = (1.0 / 10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot)).cuda()
     cos, sin = emu.rope_tables(torch.arange(7, 7 + M, dtype=torch.int32).cuda(), inv)
     pages = 8
     slots = torch.randperm(pages * page)[:M].to(torch.int32).cuda()
@@ -440,7 +497,7 @@ def test_qkv_rope_store(M, nh, nkv, D, page, H, pairs):
         vc = randn(pages, nkv, D, page, dtype=dt, seed=8)
         qkv = o.qkv_rope_store(xin, w if o is ops else w.w, bias, nh, nkv, D, cos, sin,
                                slots if write else None, kc if write else None,
-                               vc if write else None, page)
+                               vc if write else None, page, rot_dim=rot)
         return qkv[:, :nh * D].float(), kc.float(), vc.float()
     for c, s_, write in ((cos, sin, True), (None, None, True), (cos, sin, False)):
         got, want = run(ops, x, c, s_, write), run(emu, x, c, s_, write)

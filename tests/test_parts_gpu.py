@@ -61,10 +61,11 @@ def test_rotary_part(rt):
     pos_part.load(None, runtime)
     batch = type("B", (), {"positions": torch.tensor([0, 3, 77, 1000], dtype=torch.int32).cuda()})
     shared = {}
-    cos, sin = pos_part.tables(batch, shared)
+    tables = pos_part.tables(batch, shared)
+    cos, sin = tables.cos, tables.sin
     ang = batch.positions.cpu().float()[:, None] * plain.rope_inv_freq(5000.0, 48)[None, :]
     assert (cos.cpu() - torch.cos(ang)).abs().max() < 1e-5 and (sin.cpu() - torch.sin(ang)).abs().max() < 1e-5
-    assert pos_part.tables(batch, shared)[0] is cos          # prepared once per step
+    assert pos_part.tables(batch, shared) is tables          # prepared once per step
     assert NoPosition().tables(batch, shared) is None
     with pytest.raises(ValueError):
         RotaryPosition(15, 1e4)
