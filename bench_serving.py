@@ -38,12 +38,18 @@ class Request:
 
 
 def synthetic_requests(n: int, vocab: int, input_mean: int, output_mean: int, seed: int,
-                       input_std: int = 40, output_std: int = 20, longest: int = 0) -> List[Request]:
-    """``longest`` > 0 bounds prompt + output (the model's positions)."""
+                       input_std: int = 40, output_std: int = 20, longest: int = 0,
+                       input_range=None) -> List[Request]:
+    """``longest`` > 0 bounds prompt + output (the model's positions);
+    ``input_range`` (lo, hi) draws prompt lengths uniformly from it instead of
+    from the Gaussian."""
     rng = random.Random(seed)
     out = []
     for _ in range(n):
-        n_in = max(8, int(rng.gauss(input_mean, input_std)))
+        if input_range:
+            n_in = rng.randint(int(input_range[0]), int(input_range[1]))
+        else:
+            n_in = max(8, int(rng.gauss(input_mean, input_std)))
         n_out = max(1, int(rng.gauss(output_mean, output_std)))
         if longest:
             n_in = min(n_in, max(1, longest - n_out))
@@ -51,45 +57,59 @@ def synthetic_requests(n: int, vocab: int, input_mean: int, output_mean: int, se
     return out
 
 
-def _submit(engine, req: Request, sampling):
+class KeepInFlight:
+    """Closed loop: a new request whenever fewer than ``concurrency`` are in flight."""
+
+    def __init__(self, concurrency: int):
+        self.concurrency = concurrency
+
+    def due(self, now: float, in_flight: int) -> int:
+        return max(0, self.concurrency - in_flight)
+
+    def idle_for(self, now: float) -> float:
+        return 0.0
+
+
+class PoissonArrivals:
+    """Open loop: arrivals with exponential gaps at ``rate`` a second against the
+    wall clock, whatever the engine is doing."""
+
+    def __init__(self, rate: float, seed: int, start: float):
+        self.rng, self.rate, self.next_at = random.Random(seed), rate, start
+
+    def due(self, now: float, in_flight: int) -> int:
+        n = 0
+        while now >= self.next_at:
+            n += 1
+            self.next_at += self.rng.expovariate(self.rate)
+        return n
+
+    def idle_for(self, now: float) -> float:
+        return max(0.0, self.next_at - now)
+
+
+def drive(engine, requests: List[Request], arrivals, sampling) -> list:
+    """One loop for both load patterns: submit what ``arrivals`` says is due,
+    step the engine while it has work, sleep until the next arrival otherwise.
+    Returns the finished requests' outputs."""
     from servelab_amd import SamplingParams
-    return engine.add_request(
-        prompt_token_ids=req.prompt_token_ids,
-        sampling_params=SamplingParams(max_tokens=req.output_tokens, ignore_eos=True, **sampling))
-
-
-def closed_loop(engine, requests: List[Request], concurrency: int, sampling) -> list:
-    """Keeps ``concurrency`` requests in flight until all are done."""
-    waiting = list(reversed(requests))
-    live, done = set(), []
-    while waiting or live:
-        while waiting and len(live) < concurrency:
-            live.add(_submit(engine, waiting.pop(), sampling))
-        for out in engine.step():
-            if out.request_id in live:
-                live.discard(out.request_id)
-                done.append(out)
-    return done
-
-
-def open_loop(engine, requests: List[Request], rate: float, sampling, seed: int = 7) -> list:
-    """Arrivals with exponential gaps against the wall clock; the engine steps
-    whenever it has work and sleeps until the next arrival otherwise."""
-    rng = random.Random(seed)
-    done, at = [], time.monotonic()
-    for req in requests:
-        while True:
-            now = time.monotonic()
-            if now >= at:
-                break
-            if engine.has_unfinished():
-                done.extend(engine.step())
-            else:
-                time.sleep(min(at - now, 0.001))
-        _submit(engine, req, sampling)
-        at += rng.expovariate(rate)
-    while engine.has_unfinished():
-        done.extend(engine.step())
+    queue = list(reversed(requests))
+    ours, done = set(), []
+    while queue or ours:
+        now = time.monotonic()
+        for _ in range(min(len(queue), arrivals.due(now, len(ours)))):
+            req = queue.pop()
+            ours.add(engine.add_request(
+                prompt_token_ids=req.prompt_token_ids,
+                sampling_params=SamplingParams(max_tokens=req.output_tokens, ignore_eos=True,
+                                               **sampling)))
+        if engine.has_unfinished():
+            for out in engine.step():
+                if out.request_id in ours:
+                    ours.discard(out.request_id)
+                    done.append(out)
+        else:
+            time.sleep(min(arrivals.idle_for(now), 0.001))
     return done
 
 
@@ -139,32 +159,34 @@ def build_engine(args):
                             max_num_batched_tokens=args.max_batched_tokens,
                             chunked_prefill=not args.no_chunked_prefill,
                             policy=args.scheduler_policy)
+    warm = dict(tune_products=tune_option(args), capture_graphs_up_to=args.capture_graphs_up_to)
     if args.model:
         cfg = load_config(args.model)
-        return cfg, LLMEngine(cfg, cache, sched, dtype=args.dtype, tune_products=tune_option(args))
+        return cfg, LLMEngine(cfg, cache, sched, dtype=args.dtype, **warm)
     import bench                                     # random weights of a named shape, made on the device
     cfg, model, _ = bench.build(argparse.Namespace(shape=args.shape, layers=args.layers,
                                                    dtype=args.dtype, seed=args.seed))
-    return cfg, LLMEngine(cfg, cache, sched, model=model, tune_products=tune_option(args))
+    return cfg, LLMEngine(cfg, cache, sched, model=model, **warm)
 
 
 def run(args) -> dict:
     cfg, engine = build_engine(args)
     sampling = dict(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k)
+    span = (args.input_min, args.input_max) if args.input_max else None
     requests = synthetic_requests(args.num_prompts, cfg.vocab_size, args.input_mean,
                                   args.output_tokens, args.seed,
-                                  longest=cfg.max_position_embeddings)
+                                  longest=min(cfg.max_position_embeddings, args.max_context or 1 << 30),
+                                  input_range=span)
     if args.warmup_requests:
         # the first steps of a process compile nothing, but capture a graph per decode shape
         warm = synthetic_requests(args.warmup_requests, cfg.vocab_size, args.input_mean, 8,
                                   args.seed + 1, longest=cfg.max_position_embeddings)
-        closed_loop(engine, warm, min(args.concurrency, len(warm)), sampling)
+        drive(engine, warm, KeepInFlight(min(args.concurrency, len(warm))), sampling)
     steps0 = engine.num_steps
     t0 = time.monotonic()
-    if args.load_pattern == "fixed":
-        done = closed_loop(engine, requests, args.concurrency, sampling)
-    else:
-        done = open_loop(engine, requests, args.request_rate, sampling)
+    arrivals = KeepInFlight(args.concurrency) if args.load_pattern == "fixed" else \
+        PoissonArrivals(args.request_rate, args.seed + 2, t0)
+    done = drive(engine, requests, arrivals, sampling)
     elapsed = time.monotonic() - t0
     res = summarise(done, elapsed, args.ttft_slo_ms, args.tpot_slo_ms)
     res["steps"] = engine.num_steps - steps0
@@ -173,7 +195,8 @@ def run(args) -> dict:
         "load_pattern": args.load_pattern,
         "concurrency": args.concurrency if args.load_pattern == "fixed" else None,
         "request_rate": args.request_rate if args.load_pattern == "poisson" else None,
-        "num_prompts": args.num_prompts, "input_mean": args.input_mean,
+        "num_prompts": args.num_prompts,
+        "input": f"uniform {span[0]}..{span[1]}" if span else f"gauss {args.input_mean}",
         "output_tokens": args.output_tokens, "max_num_seqs": args.max_num_seqs,
         "max_batched_tokens": args.max_batched_tokens, "block_size": args.block_size,
         "num_blocks": engine.num_blocks, "temperature": args.temperature, "top_p": args.top_p,
@@ -190,6 +213,9 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--num-prompts", type=int, default=32)
     ap.add_argument("--input-mean", type=int, default=200)
+    ap.add_argument("--input-min", type=int, default=1, help="with --input-max: uniform prompt lengths")
+    ap.add_argument("--input-max", type=int, default=0, help="0 = Gaussian lengths around --input-mean")
+    ap.add_argument("--max-context", type=int, default=0, help="bound on prompt + output (0 = the model's)")
     ap.add_argument("--output-tokens", type=int, default=64)
     ap.add_argument("--load-pattern", choices=["fixed", "poisson"], default="fixed")
     ap.add_argument("--concurrency", type=int, default=8)
@@ -210,6 +236,8 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--warmup-requests", type=int, default=4,
                     help="short requests run before the clock starts (0 = none)")
     ap.add_argument("--tune-products", action="store_true")
+    ap.add_argument("--capture-graphs-up-to", type=int, default=0,
+                    help="capture decode graphs for contexts up to this length before the clock starts")
     ap.add_argument("--tune-rows", default="", help="further step sizes (rows) to tune the library products for")
     return ap
 

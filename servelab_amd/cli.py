@@ -48,6 +48,9 @@ def build_parser():
     ap.add_argument("--tune-products", action="store_true",
                     help="at start-up, time the library's matrix kernels for a full-budget step "
                          "and keep the fastest (bfloat16 only)")
+    ap.add_argument("--capture-graphs-up-to", type=int, default=0, metavar="TOKENS",
+                    help="capture the decode graphs for contexts up to this length at start-up "
+                         "instead of when a request first needs them")
     ap.add_argument("--tune-rows", default="",
                     help="comma-separated further step sizes (rows) to time them for, e.g. typical "
                          "prompt lengths; implies --tune-products")
@@ -97,7 +100,7 @@ def main(argv=None) -> int:
         SchedulerConfig(max_num_seqs=args.max_num_seqs,
                         max_num_batched_tokens=args.max_batched_tokens),
         seed=args.seed, tokenizer=tokenizer, dtype=args.dtype, tune_products=tune_option(args),
-        random_weights=seed)
+        random_weights=seed, capture_graphs_up_to=args.capture_graphs_up_to)
     if args.prompt_ids:
         prompts = [[int(t) for t in args.prompt_ids.split(",")]]
     elif tokenizer is not None:

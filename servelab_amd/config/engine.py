@@ -49,3 +49,5 @@ class EngineConfig:
     dtype: str = "auto"                    # auto (config.json's torch_dtype) | bfloat16 | float32
     device: str = "cuda:0"
     tune_products: object = False          # True, or further row counts: time the library's kernels at start-up
+    capture_graphs_up_to: int = 0          # > 0: capture the decode graphs of 1..max_num_seqs requests for
+                                           # contexts up to this many tokens at start-up (0: at first sight)

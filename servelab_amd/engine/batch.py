@@ -152,11 +152,34 @@ def batch_on_device(arr: BatchArrays, dev: torch.Tensor, max_ctx_len: int = 0) -
         host_state_slots=arr.state_slots)
 
 
+class Staging:
+    """Pinned host memory that a step's arrays pass through on their way to the
+    device, kept from step to step (pinning a fresh buffer costs more than the
+    copy); ``done`` marks when the last copy out of it has finished."""
+
+    def __init__(self):
+        self.buffer = None
+        self.done = None
+
+    def upload(self, flat: np.ndarray, device) -> torch.Tensor:
+        n = flat.size
+        if self.buffer is None or self.buffer.numel() < n:
+            self.buffer = torch.empty(max(4096, 2 * n), dtype=torch.int32).pin_memory()
+            self.done = torch.cuda.Event()
+        else:
+            self.done.synchronize()
+        self.buffer[:n].copy_(torch.from_numpy(flat))
+        dev = self.buffer[:n].to(device, non_blocking=True)
+        self.done.record()
+        return dev
+
+
 def pack_batch(entries: List[StepEntry], starts: List[int], rows: List[int], manager, device,
-               pad_pages_to: int = 8) -> StepBatch:
+               pad_pages_to: int = 8, staging: "Staging" = None) -> StepBatch:
     """Build the arrays of a step and copy them to the device in one transfer."""
     arr = build_arrays(entries, starts, rows, manager, pad_pages_to)
-    host = torch.from_numpy(arr.flat)
-    if torch.device(device).type == "cuda":
-        host = host.pin_memory()
-    return batch_on_device(arr, host.to(device, non_blocking=True))
+    if torch.device(device).type != "cuda":
+        return batch_on_device(arr, torch.from_numpy(arr.flat).to(device))
+    if staging is None:
+        return batch_on_device(arr, torch.from_numpy(arr.flat).pin_memory().to(device, non_blocking=True))
+    return batch_on_device(arr, staging.upload(arr.flat, device))

@@ -24,13 +24,17 @@ class LLMEngine:
                  scheduler_config: Optional[SchedulerConfig] = None, seed: int = 1234,
                  device: str = "cuda:0", tokenizer=None,
                  clock: Optional[Callable[[], float]] = None, dtype: str = "auto",
-                 model=None, ops=None, tune_products=False, random_weights: Optional[int] = None):
+                 model=None, ops=None, tune_products=False, random_weights: Optional[int] = None,
+                 capture_graphs_up_to: int = 0):
         """``model_config.path`` names the model folder (as in the reference,
         servelab/engine/engine.py:86-87); ``model`` may pass an already loaded
         DecoderModel instead, and ``random_weights`` a seed: the model of
         ``model_config`` then gets seeded random weights made on the device and
         no folder is read.  ``tune_products``: True, or a list of further
-        step sizes (rows) to time the library's matrix kernels for."""
+        step sizes (rows) to time the library's matrix kernels for.
+        ``capture_graphs_up_to``: a context length up to which the decode graphs
+        of 1..max_num_seqs requests are captured now rather than when a request
+        first needs them."""
         self.model_config = model_config
         self.cache_config = cache_config or CacheConfig()
         self.scheduler_config = scheduler_config or SchedulerConfig()
@@ -68,6 +72,10 @@ class LLMEngine:
                 rows += sorted({library_rows(n)
                                 for n in range(first, self.scheduler_config.max_num_seqs + 1)})
             self.runner.tune_products(rows)
+        self.graphs_captured = 0
+        if capture_graphs_up_to:
+            self.graphs_captured = self.runner.capture_graphs(
+                range(1, self.scheduler_config.max_num_seqs + 1), capture_graphs_up_to)
         self.scheduler = Scheduler(self.scheduler_config, self.runner.manager, self.clock,
                                    eos_token_id=model.spec.eos_token_id,
                                    max_positions=model.spec.max_position_embeddings)

@@ -15,7 +15,7 @@ import torch
 from ..cache import CacheManager, CachePool
 from ..parts.base import Runtime
 from ..parts.model import DecoderModel
-from .batch import StepBatch, StepEntry, batch_on_device, build_arrays, pack_batch
+from .batch import Staging, StepBatch, StepEntry, batch_on_device, build_arrays, pack_batch
 
 
 class OutOfPages(RuntimeError):
@@ -56,6 +56,7 @@ class ModelRunner:
             self.graph_memory_limit = min(self.GRAPH_MEMORY_MAX, int(free * self.GRAPH_MEMORY_SHARE))
         self.graph_replays = 0
         self.graph_evictions = 0
+        self._staging = Staging()
         self._decoding = None         # the last graph step, for the next one to continue from
 
     # ------------------------------------------------------------ requests
@@ -111,7 +112,8 @@ class ModelRunner:
     def prepare(self, entries: List[StepEntry]):
         """Reserve pages and build the device batch: (batch, packed entries)."""
         packed, starts, rows = self.reserve(entries)
-        return pack_batch(packed, starts, rows, self.manager, self.rt.device), packed
+        return pack_batch(packed, starts, rows, self.manager, self.rt.device,
+                          staging=self._staging), packed
 
     # -------------------------------------------------------------- graphs
     def _graph_key(self, packed, starts, rows):
@@ -173,6 +175,50 @@ class ModelRunner:
         self._graph_bytes += need
         self._decoding = (key, arr)
         return eager
+
+    def capture_graphs(self, batch_sizes, max_context: int) -> int:
+        """Capture, ahead of use, the decode graphs of ``batch_sizes`` requests
+        for every context capacity up to ``max_context`` tokens, so that no
+        request meets the two extra passes (an eager step, then the capture) of
+        a shape seen for the first time.  Runs on throw-away requests of one
+        token; stops when the graphs' memory limit is reached (nothing is
+        dropped to make room).  Returns the number of graphs captured."""
+        if not self.use_graphs:
+            return 0
+        caps, cap = [], self.GRAPH_MIN_CONTEXT
+        limit = min(int(max_context), self.max_positions)
+        while True:
+            caps.append(cap)
+            if cap >= limit:
+                break
+            cap *= 2
+        made = 0
+        for B in sorted({int(b) for b in batch_sizes if 1 <= int(b) <= self.graph_max_seqs}):
+            tags = [("capture_graphs", i) for i in range(B)]
+            opened = []
+            try:
+                for t in tags:
+                    if not self.open(t):
+                        break
+                    opened.append(t)
+                if len(opened) < B or not all(self.manager.grow(t, 1) for t in tags):
+                    continue
+                packed = [StepEntry(t, [0], [0]) for t in tags]
+                for cap in caps:
+                    if (B, cap) in self._graphs or cap // self.manager.page_size < 1:
+                        continue
+                    need = B * self.model.spec.vocab_size * 4
+                    if self._graphs and self._graph_bytes + need > self.graph_memory_limit:
+                        return made
+                    self._step_graph((B, cap), packed, [0] * B, list(range(B)))
+                    made += 1
+            finally:
+                for t in opened:
+                    self.close(t)
+                self._decoding = None
+        if made:
+            torch.cuda.synchronize(self.rt.device)
+        return made
 
     def _entry_bytes(self, dev, B) -> int:
         """What a captured graph keeps alive beside the shared pool of
@@ -294,7 +340,8 @@ class ModelRunner:
         if key is not None:
             logits = self._step_graph(key, packed, starts, rows)
         else:
-            batch = pack_batch(packed, starts, rows, self.manager, self.rt.device)
+            batch = pack_batch(packed, starts, rows, self.manager, self.rt.device,
+                               staging=self._staging)
             logits = self.model.forward(batch, self.bindings)
         for e, start in zip(packed, starts):
             self.manager.commit(e.request, start + len(e.tokens))

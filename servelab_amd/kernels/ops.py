@@ -129,6 +129,10 @@ class HipOps:
             raise KernelError("servelab_amd needs a GPU: the HIP kernels have no CPU fallback")
         self.act_dtype = act_dtype
         self.device = torch.device(device)
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        # the current stream's handle without the wrapper objects torch.cuda.current_stream() builds
+        # (a launch is a few microseconds of host time, and this was one of them)
+        self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self.dtype_name = "float32" if act_dtype == torch.float32 else "bfloat16"
         units = [build.unit(stem, self.dtype_name) for stem in build.DEFAULT_STEMS]
         build.ensure(units)
@@ -153,11 +157,15 @@ class HipOps:
             fn = getattr(self._lib[stem], name)
             fn.restype = ctypes.c_char_p
             self._fn[name] = fn
-        err = fn(*args, _c_void_p(torch.cuda.current_stream().cuda_stream))
+        stream = self._raw_stream(self._device_index) if self._raw_stream is not None else \
+            torch.cuda.current_stream(self.device).cuda_stream
+        err = fn(*args, _c_void_p(stream))
         if err is not None:
             raise KernelError(f"{name}: {err.decode()}")
 
     def _check(self, t, dtype, shape=None, name="tensor"):
+        if t.is_cuda and t.dtype is dtype and t.is_contiguous() and (shape is None or t.shape == shape):
+            return                                        # (a torch.Size equals a tuple of the same numbers)
         if t.device.type != "cuda":
             raise KernelError(f"{name} is on {t.device}, not on the GPU")
         if t.dtype != dtype:

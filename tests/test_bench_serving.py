@@ -62,14 +62,15 @@ class ScriptedEngine:
 def test_closed_loop_keeps_the_concurrency():
     reqs = bs.synthetic_requests(20, 100, 30, 6, seed=0)
     eng = ScriptedEngine()
-    done = bs.closed_loop(eng, reqs, 3, dict(temperature=0.0))
+    done = bs.drive(eng, reqs, bs.KeepInFlight(3), dict(temperature=0.0))
     assert len(done) == 20 and eng.most_live == 3 and not eng.has_unfinished()
 
 
 def test_open_loop_submits_everything():
     reqs = bs.synthetic_requests(10, 100, 30, 4, seed=0)
     eng = ScriptedEngine()
-    done = bs.open_loop(eng, reqs, rate=5000.0, sampling=dict(temperature=0.0))
+    import time
+    done = bs.drive(eng, reqs, bs.PoissonArrivals(5000.0, 1, time.monotonic()), dict(temperature=0.0))
     assert sorted(o.request_id for o in done) == sorted(f"r{i}" for i in range(10))
 
 
@@ -84,3 +85,9 @@ def test_summary_formulas():
     assert res["ttft_ms_p50"] == 100.0
     assert res["tpot_ms_p50"] == pytest.approx(75.0)       # (500 ms / 10 + 400 ms / 4) / 2
     assert res["goodput"] == 0.5                           # one of the two with a TPOT is inside both bounds
+
+
+def test_uniform_prompt_lengths():
+    reqs = bs.synthetic_requests(200, 1000, 0, 16, seed=3, input_range=(512, 4096), longest=8192)
+    lengths = [len(r.prompt_token_ids) for r in reqs]
+    assert min(lengths) >= 512 and max(lengths) <= 4096 and 2000 < sum(lengths) / 200 < 2600

@@ -362,3 +362,19 @@ def test_command_line_generates_the_plain_tokens(dtype, capsys):
         for i, t in enumerate(got):
             row = logits[len(prompt) - 1 + i]
             assert row[t] >= row.max() - 0.02 * row.abs().max(), f"token {i}"
+
+
+def test_graphs_captured_at_start_up_are_the_ones_requests_then_replay(tmp_path, monkeypatch):
+    monkeypatch.setattr(ModelRunner, "GRAPH_MIN_CONTEXT", 32)
+    folder = make_folder(tmp_path, "B", seed=29)
+    cfg, w = plain.load_folder(folder)
+    eng = LLMEngine(load_config(folder), CacheConfig(num_blocks=64),
+                    SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=64), dtype="float32",
+                    capture_graphs_up_to=128)
+    assert eng.graphs_captured == 4 * 3 and len(eng.runner._graphs) == 12     # 1..4 requests x {32, 64, 128}
+    assert eng.runner.manager.num_free_pages() == 64
+    eng.runner.manager.check()
+    outs = eng.generate(PROMPTS, SamplingParams.greedy(12))
+    for p, o in zip(PROMPTS, outs):
+        assert o.outputs[0].token_ids == plain.greedy_generate(cfg, w, p, 12)
+    assert len(eng.runner._graphs) == 12 and eng.runner.graph_replays >= 10   # nothing new was captured
