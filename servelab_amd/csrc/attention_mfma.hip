@@ -129,6 +129,13 @@ struct Columns {
 #pragma unroll
       for (int dd = 0; dd < DD; ++dd) o[b][dd] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    // The queries have to be in their registers before the loop over the key blocks starts: the
+    // counter of outstanding loads is one for all of them, so a wait for a query inside the loop
+    // would, on every pass, also wait for the keys and values just requested for the next block.
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) asm volatile("" : "+v"(qf[b][kk]));
     const int tok_first = c0 / g;
     const int c_last = c0 + 16 * NB - 1 < ncols - 1 ? c0 + 16 * NB - 1 : ncols - 1;
     const int kmax = pos0 + c_last / g;
