@@ -3,8 +3,8 @@
 
 Default run: the layer sizes of the Qwen2.5-7B shape with random weights,
 bfloat16, a batch of 8 requests whose context ends at 4,096 tokens, 16-token
-pages.  A "step" is one decode step of the whole batch through the engine's
-step function and greedy sampling; ``value`` is decoded tokens per second.
+pages.  A "step" is one decode step of the whole batch through the engine
+(scheduler, step function, greedy sampling); ``value`` is decoded tokens per second.
 The same line carries a 2,048-token prefill, the decode step's HBM roofline
 (every weight the step uses once plus the cache of the live requests, over its
 time) and decode at batch 1 and 64.
@@ -85,51 +85,47 @@ def prefill_flops(cfg, T):
     return 2 * T * linear + attn + 2 * cfg.vocab_size * h
 
 
-def fill_cache(runner, requests, ctx, seed):
-    """Open ``requests`` with ``ctx`` tokens of random K/V already cached."""
+def time_decode(cfg, model, batch, ctx_end, steps, warmup, page, seed=0):
+    """Contract timing of decode steps through the engine itself (scheduler,
+    step function, sampler): ``batch`` requests with prompts of random ids are
+    prefilled (untimed), then ``warmup`` untimed decode steps, then exactly
+    ``steps`` steps between two synchronisations.  The longest context reaches
+    ``ctx_end`` at the last step (requests whose prompts were prefilled a step
+    later are a token shorter each).  The engine keeps one decode step
+    queued ahead of the host; the region starts with that step finished and not
+    yet consumed, so exactly ``steps`` steps are queued and finished inside it."""
     import torch
-    gen = torch.Generator(device=runner.rt.device)
-    gen.manual_seed(seed)
-    for t in runner.pool.k + runner.pool.v:
-        for s in range(t.shape[0]):                   # stream by stream: bounded temporaries
-            t[s].copy_(torch.randn(t[s].shape, generator=gen, device=t.device,
-                                   dtype=torch.float32).mul_(0.5))
-    for r in requests:
-        assert runner.open(r) and runner.manager.grow(r, ctx)
-        runner.manager.commit(r, ctx)
-
-
-def time_decode(model, batch, ctx_end, steps, warmup, page, seed=0):
-    """Median-free, contract timing: ``warmup`` untimed steps, then exactly
-    ``steps`` steps between two synchronisations.  The context of every request
-    reaches ``ctx_end`` at the last step."""
-    import torch
-    from servelab_amd.engine import ModelRunner, StepEntry
+    from servelab_amd import CacheConfig, LLMEngine, SamplingParams, SchedulerConfig
     total = warmup + steps
-    start = ctx_end - total
-    pages = batch * (-(-ctx_end // page)) + 8
-    runner = ModelRunner(model, pages, page, max_num_seqs=batch)
-    requests = [f"b{i}" for i in range(batch)]
-    fill_cache(runner, requests, start, seed)
-    vocab = model.spec.vocab_size
-    tokens = torch.randint(0, vocab, (batch,), generator=torch.Generator().manual_seed(seed)).tolist()
-    ops = model.rt.ops
-
-    def one_step(toks):
-        logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(requests, toks)])
-        return ops.argmax(logits).tolist()             # the engine needs the token on the host
-
+    budget = 8192
+    prompt_len = ctx_end - total - 1
+    prompt_len -= -(-batch * prompt_len // budget) - 1   # the first request decodes while the others prefill
+    pages = batch * (-(-(ctx_end + 2) // page)) + 16
+    engine = LLMEngine(cfg, CacheConfig(block_size=page, num_blocks=pages),
+                       SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget),
+                       model=model)
+    gen = torch.Generator().manual_seed(seed)
+    params = SamplingParams(temperature=0.0, max_tokens=total + 64, ignore_eos=True)
+    for _ in range(batch):
+        engine.add_request(prompt_token_ids=torch.randint(0, cfg.vocab_size, (prompt_len,),
+                                                          generator=gen).tolist(),
+                           sampling_params=params)
+    while any(not r.decoding for r in engine.scheduler.active) or engine.scheduler.queue:
+        engine.step()                                  # prompts, in portions
+    before = engine.num_steps
     for _ in range(warmup):
-        tokens = one_step(tokens)
+        engine.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        tokens = one_step(tokens)
+        engine.step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    assert runner.manager.length(requests[0]) == ctx_end
-    mean_ctx = ctx_end - (steps + 1) / 2.0
-    del runner
+    assert engine.num_steps - before == total and len(engine.scheduler.active) == batch
+    lengths = [engine.runner.manager.length(r.request_id) for r in engine.scheduler.active]
+    assert ctx_end - 2 <= max(lengths) <= ctx_end and min(lengths) >= ctx_end - 2 - batch, lengths
+    mean_ctx = sum(lengths) / batch - (steps + 1) / 2.0
+    del engine
     torch.cuda.empty_cache()
     return dt / steps, mean_ctx
 
@@ -199,7 +195,7 @@ def main():
     itemsize = 2 if short == "bf16" else 4
     page = args.block_size
 
-    step_s, mean_ctx = time_decode(model, args.batch, args.context, args.steps, args.warmup, page)
+    step_s, mean_ctx = time_decode(cfg, model, args.batch, args.context, args.steps, args.warmup, page)
     value = args.batch / step_s
     step_bytes = weight_bytes_per_step(cfg, itemsize) + \
         args.batch * mean_ctx * cache_bytes_per_token(cfg, itemsize)
@@ -209,8 +205,8 @@ def main():
         "metric": "decode_tokens_per_s", "value": round(value, 2), "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short,
-        "data": "synthetic: seeded random weights, uniform random token ids, cache filled with "
-                "random keys and values up to the context",
+        "data": "synthetic: seeded random weights, prompts of uniform random token ids prefilled "
+                "by the engine up to the context",
         "config": {
             "model": SHAPES[args.shape][0], "global_batch": args.batch, "seq_len": args.context,
             "parallelism": "none", "layers": cfg.num_layers, "layers_of_shape": full_layers,
@@ -234,7 +230,7 @@ def main():
     if not args.no_points:
         points = {}
         for b in (1, 64):
-            s, _ = time_decode(model, b, args.context, max(5, args.steps // 2), 2, page)
+            s, _ = time_decode(cfg, model, b, args.context, max(5, args.steps // 2), 2, page)
             points[f"decode_b{b}"] = round(b / s, 2)
         line["points"] = points
     print(json.dumps(line))

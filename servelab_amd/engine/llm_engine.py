@@ -19,13 +19,55 @@ from .request import Request
 from .session import load_model_on_device, make_runner, random_model_on_device
 
 
+class _TokenBuffers:
+    """Two pinned host buffers for sampled tokens, used in turn: the step ahead
+    copies into one while the host still reads the other."""
+
+    def __init__(self, rows: int, device):
+        self.cuda = torch.device(device).type == "cuda"
+        self.buffers = [torch.empty(max(1, rows), dtype=torch.int32) for _ in range(2)]
+        if self.cuda:
+            self.buffers = [b.pin_memory() for b in self.buffers]
+        self.turn = 0
+
+    def take(self, n: int) -> torch.Tensor:
+        self.turn ^= 1
+        if self.buffers[self.turn].numel() < n:
+            grown = torch.empty(2 * n, dtype=torch.int32)
+            self.buffers[self.turn] = grown.pin_memory() if self.cuda else grown
+        return self.buffers[self.turn][:n]
+
+
+class _Flight:
+    """A step that is queued on the device: its plan, the requests it samples
+    for (in row order), the sampled tokens on the device and their copy on the
+    way to the host."""
+
+    def __init__(self, plan, drawing, device_tokens, buffers: _TokenBuffers):
+        self.plan, self.drawing, self.device_tokens = plan, drawing, device_tokens
+        self.host = self.arrived = None
+        if device_tokens is not None:
+            self.host = buffers.take(len(drawing))
+            self.host.copy_(device_tokens, non_blocking=True)
+            if device_tokens.is_cuda:
+                self.arrived = torch.cuda.Event()
+                self.arrived.record()
+
+    def tokens(self) -> List[int]:
+        if self.host is None:
+            return []
+        if self.arrived is not None:
+            self.arrived.synchronize()
+        return self.host.tolist()
+
+
 class LLMEngine:
     def __init__(self, model_config, cache_config: Optional[CacheConfig] = None,
                  scheduler_config: Optional[SchedulerConfig] = None, seed: int = 1234,
                  device: str = "cuda:0", tokenizer=None,
                  clock: Optional[Callable[[], float]] = None, dtype: str = "auto",
                  model=None, ops=None, tune_products=False, random_weights: Optional[int] = None,
-                 capture_graphs_up_to: int = 0):
+                 capture_graphs_up_to: int = 0, run_ahead: bool = True):
         """``model_config.path`` names the model folder (as in the reference,
         servelab/engine/engine.py:86-87); ``model`` may pass an already loaded
         DecoderModel instead, and ``random_weights`` a seed: the model of
@@ -80,6 +122,9 @@ class LLMEngine:
                                    eos_token_id=model.spec.eos_token_id,
                                    max_positions=model.spec.max_position_embeddings)
         self.sampler = Sampler(model.rt.ops, self.device, seed)
+        self.run_ahead = bool(run_ahead)
+        self._flight: Optional[_Flight] = None
+        self._token_buffers = _TokenBuffers(self.scheduler_config.max_num_seqs, self.device)
         self._submitted = 0
         self.num_steps = 0
 
@@ -104,9 +149,6 @@ class LLMEngine:
             arrived=self.clock(), number=self._submitted))
         return request_id
 
-    def abort_request(self, request_id: str) -> bool:
-        return self.scheduler.abort_request(request_id)
-
     def has_unfinished(self) -> bool:
         return self.scheduler.has_unfinished()
 
@@ -114,24 +156,63 @@ class LLMEngine:
     def step(self) -> List[RequestOutput]:
         """One scheduler pass, one model step, one sampling call.  Returns the
         requests that finished (or were aborted) in this step
-        (servelab/engine/engine.py:169-241)."""
-        plan = self.scheduler.schedule()
-        outputs = [result_of(r, self._to_text) for r in plan.aborted]
-        if plan.is_empty():
-            if not outputs and self.scheduler.has_unfinished():
-                raise RuntimeError("nothing can be scheduled although requests are unfinished")
-            return outputs
-        items = plan.items()                     # portions first, then single tokens
-        entries = [StepEntry(it.request.request_id, it.token_ids,
-                             [it.count - 1] if it.samples else []) for it in items]
-        drawing = [it.request for it in items if it.samples]
-        logits = self.runner.step(entries)
-        tokens = self.sampler.sample(logits, [r.params for r in drawing],
-                                     [r.number for r in drawing], [r.num_output for r in drawing])
+        (servelab/engine/engine.py:169-241).
+
+        Decoding runs one step ahead of the host: while a step's tokens are
+        still on their way, the next decode step of the same requests is
+        already queued behind it on the device, taking its token ids from the
+        sampler's output there (``run_ahead``; the reference waits for every
+        step's tokens before it plans the next).  What the host does between
+        two steps then costs no device time.  A request that a stop token ends
+        has one wasted row in the step ahead; a newcomer waits for that step."""
+        flight, self._flight = self._flight, None
+        outputs: List[RequestOutput] = []
+        if flight is None:
+            plan = self.scheduler.schedule()
+            outputs = [result_of(r, self._to_text) for r in plan.aborted]
+            if plan.is_empty():
+                if not outputs and self.scheduler.has_unfinished():
+                    raise RuntimeError("nothing can be scheduled although requests are unfinished")
+                return outputs
+            flight = self._launch(plan, None)
+        if self.run_ahead:
+            ahead = self.scheduler.plan_ahead(flight.plan)
+            if ahead is not None:
+                self._flight = self._launch(ahead, flight)
+        tokens = flight.tokens()                 # waits for this step's tokens, not for the step ahead
         finished = self.scheduler.complete(
-            plan, {r.request_id: t for r, t in zip(drawing, tokens)}, now=self.clock())
+            flight.plan, {r.request_id: t for r, t in zip(flight.drawing, tokens)}, now=self.clock())
         self.num_steps += 1
+        if self._flight is not None and all(it.request.done for it in self._flight.plan.items()):
+            self._flight = None                  # every request of the step ahead has ended: its result is void
         return outputs + [result_of(r, self._to_text) for r in finished]
+
+    def _launch(self, plan, after: Optional["_Flight"]) -> "_Flight":
+        """Queue ``plan`` on the device: the model step, the sampling call and
+        the copy of the sampled tokens to the host.  ``after``: the step whose
+        tokens this one continues from, not yet known to the host."""
+        items = plan.items()                     # portions first, then single tokens
+        drawing = [it.request for it in items if it.samples or after is not None]
+        if after is None:
+            entries = [StepEntry(it.request.request_id, it.token_ids,
+                                 [it.count - 1] if it.samples else []) for it in items]
+            logits = self.runner.step(entries)
+        else:
+            entries = [StepEntry(it.request.request_id, [0], [0]) for it in items]
+            row_of = {r.request_id: i for i, r in enumerate(after.drawing)}
+            rows = [row_of[it.request.request_id] for it in items]
+            ids = after.device_tokens
+            if rows != list(range(len(after.drawing))):
+                ids = ids[torch.tensor(rows, dtype=torch.long, device=ids.device)]
+            logits = self.runner.step(entries, device_ids=ids)
+        drawn_before = 1 if after is not None else 0     # the token of the step this one follows
+        device_tokens = self.sampler.sample_on_device(
+            logits, [r.params for r in drawing], [r.number for r in drawing],
+            [r.num_output + drawn_before for r in drawing]) if drawing else None
+        return _Flight(plan, drawing, device_tokens, self._token_buffers)
+
+    def abort_request(self, request_id: str) -> bool:
+        return self.scheduler.abort_request(request_id)
 
     @property
     def _to_text(self):

@@ -130,7 +130,7 @@ class ModelRunner:
             cap *= 2
         return (B, cap)
 
-    def _step_graph(self, key, packed, starts, rows):
+    def _step_graph(self, key, packed, starts, rows, device_ids=None):
         """Decode step through a HIP graph.  The first step of a shape runs
         eagerly on a side stream (its result is returned) and is then captured;
         later steps overwrite the graph's metadata buffer and replay it.
@@ -149,6 +149,8 @@ class ModelRunner:
             staging.copy_(host)
             dev.copy_(staging, non_blocking=True)
             copied.record()
+            if device_ids is not None:
+                dev[arr.offsets[0]:arr.offsets[0] + B].copy_(device_ids)
             graph.replay()
             self.graph_replays += 1
             self._decoding = (key, arr)
@@ -156,6 +158,8 @@ class ModelRunner:
         staging = torch.empty_like(host).pin_memory()
         staging.copy_(host)
         dev = staging.to(self.rt.device, non_blocking=True)
+        if device_ids is not None:
+            dev[arr.offsets[0]:arr.offsets[0] + B].copy_(device_ids)
         batch = batch_on_device(arr, dev, max_ctx_len=cap)
         side = torch.cuda.Stream(device=self.rt.device)
         side.wait_stream(torch.cuda.current_stream())
@@ -241,7 +245,7 @@ class ModelRunner:
                 self._decoding = None
             del graph, dev, staging, logits, copied
 
-    def _continue_decoding(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+    def _continue_decoding(self, entries: List[StepEntry], device_ids=None) -> Optional[torch.Tensor]:
         """The common decode step — the same requests as the last graph step,
         one more token each — without rebuilding the step's arrays: ids are
         replaced, positions and contexts advance by one, slots follow the block
@@ -288,6 +292,8 @@ class ModelRunner:
         staging.copy_(torch.from_numpy(flat))
         dev.copy_(staging, non_blocking=True)
         copied.record()
+        if device_ids is not None:
+            dev[off[0]:off[0] + B].copy_(device_ids)
         graph.replay()
         self.graph_replays += 1
         for request, p in zip(arr.requests, starts):
@@ -324,24 +330,36 @@ class ModelRunner:
             torch.cuda.synchronize(self.rt.device)
         return done
 
-    def step(self, entries: List[StepEntry]) -> torch.Tensor:
+    def step(self, entries: List[StepEntry], device_ids: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run one batch; returns float32 logits [wanted, vocab] in the order of
         the entries and of their ``want``.  The tensor may be a captured graph's
-        output buffer: it is valid until the next call of ``step``."""
+        output buffer: it is valid until the next call of ``step``.
+
+        ``device_ids`` (int32 on the device, one per entry, in the order of the
+        entries) gives the token ids of a step whose entries bring one token
+        each when the host does not know them yet (the last step's sampled
+        tokens, still on the device); the entries' own ids are then ignored."""
         if not entries:
             return torch.empty((0, self.model.spec.vocab_size), dtype=torch.float32,
                                device=self.rt.device)
-        logits = self._continue_decoding(entries)
+        if device_ids is not None:
+            if any(len(e.tokens) != 1 for e in entries):
+                raise ValueError("token ids from the device go with entries of one token each")
+            if device_ids.dtype != torch.int32 or tuple(device_ids.shape) != (len(entries),):
+                raise ValueError("device_ids must be int32, one per entry")
+        logits = self._continue_decoding(entries, device_ids)
         if logits is not None:
             return logits
         self._decoding = None
         packed, starts, rows = self.reserve(entries)
         key = self._graph_key(packed, starts, rows)
         if key is not None:
-            logits = self._step_graph(key, packed, starts, rows)
+            logits = self._step_graph(key, packed, starts, rows, device_ids)
         else:
             batch = pack_batch(packed, starts, rows, self.manager, self.rt.device,
                                staging=self._staging)
+            if device_ids is not None:           # (one token each: packed order is the callers' order)
+                batch.ids.copy_(device_ids)
             logits = self.model.forward(batch, self.bindings)
         for e, start in zip(packed, starts):
             self.manager.commit(e.request, start + len(e.tokens))

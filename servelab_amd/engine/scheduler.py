@@ -183,6 +183,35 @@ class Scheduler:
             budget -= count
         return budget
 
+    def plan_ahead(self, plan: Plan) -> Optional[Plan]:
+        """The step after ``plan``, planned while ``plan`` still runs and its
+        sampled tokens are not known: one more token for every request of
+        ``plan`` that cannot end with this step by its length.  Possible only
+        when ``plan`` samples for every active request and nothing waits for
+        admission (so the step after it would be exactly this one, unless a
+        stop token ends a request: its row of the step ahead is then wasted and
+        ignored).  Pages are reserved; None when the step cannot be planned
+        ahead.  ``complete`` must see ``plan`` before the plan ahead."""
+        if self.queue or not plan.items() or len(plan.items()) != len(self.active):
+            return None
+        if not all(item.samples and item.request.phase == ACTIVE for item in plan.items()):
+            return None
+        ahead = Plan()
+        for item in plan.items():
+            req = item.request
+            length = len(req.tokens) + 1                      # once this step's token is appended
+            if req.num_output + 1 >= req.params.max_tokens:
+                continue                                      # ends with this step
+            if self.max_positions is not None and length >= self.max_positions:
+                continue
+            ahead.decodes.append(Planned(req, item.start + item.count, 1))
+        if not ahead.decodes or len(ahead.decodes) > self.cfg.max_num_batched_tokens:
+            return None
+        for item in ahead.decodes:
+            if not self.manager.grow(item.request.request_id, item.start + 1):
+                return None                                   # (pages taken so far stay with their requests)
+        return ahead
+
     # ------------------------------------------------------------- helpers
     def _portion(self, req: Request, budget: int) -> int:
         """Next portion of what a request is owed: what the budget leaves, at

@@ -33,11 +33,17 @@ class Sampler:
                draws: Sequence[int]) -> List[int]:
         """``logits`` [B, V] float32; ``params[i]`` the SamplingParams of row i,
         ``numbers[i]`` its request's submission number, ``draws[i]`` how many
-        tokens that request has sampled before."""
+        tokens that request has sampled before.  Returns the tokens on the host."""
         if logits.shape[0] == 0:
             return []
+        return self.sample_on_device(logits, params, numbers, draws).tolist()
+
+    def sample_on_device(self, logits: torch.Tensor, params: Sequence, numbers: Sequence[int],
+                         draws: Sequence[int]) -> torch.Tensor:
+        """The same, but the tokens stay on the device (int32 [B]) and nothing
+        waits for them: the next step can take them from there."""
         if all(p.temperature == 0.0 for p in params):
-            return self.ops.argmax(logits).tolist()
+            return self.ops.argmax(logits)
         # one host buffer and one copy for the five per-row arrays:
         # seeds and draw counters (int64), temperature and top_p (float32), top_k (int32)
         B = len(params)
@@ -52,4 +58,4 @@ class Sampler:
         return self.ops.sample(
             logits, dev[4 * B:5 * B].view(torch.float32), dev[6 * B:] if cut else None,
             dev[5 * B:6 * B].view(torch.float32) if cut else None,
-            dev[:2 * B].view(torch.int64), dev[2 * B:4 * B].view(torch.int64)).tolist()
+            dev[:2 * B].view(torch.int64), dev[2 * B:4 * B].view(torch.int64))

@@ -14,11 +14,11 @@ from tiny_configs import make_folder
 
 
 def make_engine(folder, num_blocks=64, max_batched=256, max_seqs=8, block_size=16, chunked=True,
-                policy="fcfs"):
+                policy="fcfs", run_ahead=True):
     return LLMEngine(load_config(folder), CacheConfig(block_size=block_size, num_blocks=num_blocks),
                      SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched,
                                      chunked_prefill=chunked, policy=policy),
-                     device="cpu", dtype="float32", ops=EmulatedOps())
+                     device="cpu", dtype="float32", ops=EmulatedOps(), run_ahead=run_ahead)
 
 
 PROMPTS = [list(range(10, 40)), [5, 9, 200, 31], list(range(300, 377)), [7]]
@@ -66,8 +66,11 @@ def test_running_requests_keep_the_invariant(folder_and_plain):
         eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(5))
     while eng.has_unfinished():
         eng.step()
+        ahead = {it.request.request_id for it in eng._flight.plan.items()} if eng._flight else set()
         for r in eng.scheduler.active:                # tests/test_engine_smoke.py:113-127
-            assert r.owed >= 1 and eng.runner.manager.length(r.request_id) == r.cached
+            # (a request in the step that runs ahead has that step's token in the cache already)
+            assert r.owed >= 1
+            assert eng.runner.manager.length(r.request_id) == r.cached + (r.request_id in ahead)
 
 
 @pytest.mark.parametrize("max_seqs,num_blocks", [(2, 64), (8, 9)])
@@ -163,3 +166,43 @@ def test_float16_checkpoints_are_served_in_bfloat16_and_say_so(tmp_path, capsys)
     with pytest.raises(ValueError, match="no kernels"):
         resolve_dtype("float16", cfg)
     assert resolve_dtype("float32", cfg) == torch.float32 and capsys.readouterr().err == ""
+
+
+def test_decoding_a_step_ahead_changes_nothing_but_the_number_of_model_steps(folder_and_plain):
+    """With and without the step ahead: the same tokens; a stop token costs one wasted row, never
+    a wrong token; requests that arrive while a step is ahead join after it; an abort while a
+    step is ahead leaves nothing held."""
+    folder, want = folder_and_plain
+    stop = want[0][5]
+    cut = [w[:w.index(stop) + 1] if stop in w else w for w in want]
+    params = SamplingParams(temperature=0.0, max_tokens=12, stop_token_ids=(stop,))
+    runs = {}
+    for ahead in (False, True):
+        eng = make_engine(folder, run_ahead=ahead)
+        outs = eng.generate(PROMPTS, params)
+        assert [o.outputs[0].token_ids for o in outs] == cut
+        assert eng.runner.manager.num_free_pages() == 64 and eng._flight is None
+        runs[ahead] = eng.runner.steps
+    assert runs[True] >= runs[False]                      # steps whose every row was void are the difference
+    # arrivals during decoding
+    eng = make_engine(folder, max_batched=32)
+    first = eng.add_request(prompt_token_ids=PROMPTS[0], sampling_params=SamplingParams.greedy(12))
+    done = {}
+    for i in range(40):
+        if i == 3:
+            assert eng._flight is not None                # a step is ahead at this point
+            second = eng.add_request(prompt_token_ids=PROMPTS[2], sampling_params=SamplingParams.greedy(12))
+        if not eng.has_unfinished():
+            break
+        for out in eng.step():
+            done[out.request_id] = out.outputs[0].token_ids
+    assert done[first] == want[0] and done[second] == want[2]
+    # abort while a step is ahead
+    eng = make_engine(folder)
+    rid = eng.add_request(prompt_token_ids=PROMPTS[0], sampling_params=SamplingParams.greedy(12))
+    eng.step(), eng.step()
+    assert eng._flight is not None and eng.abort_request(rid)
+    assert not eng.has_unfinished() and eng.runner.manager.num_free_pages() == 64
+    other = eng.generate([PROMPTS[1]], SamplingParams.greedy(12))[0]
+    assert other.outputs[0].token_ids == want[1]
+    eng.runner.manager.check()
