@@ -99,12 +99,28 @@ struct AttnParams {
   int pair;                      // prompt workgroups take a late tile and its early mirror
 };
 
-// The columns of one wavefront: queries, running maxima and sums, outputs.
-template <int NB>
+// The columns of one wavefront: queries, reference points and sums, outputs.
+//
+// Vector work per score is what limits these kernels beside the matrix
+// products (a block of 32 keys is 32 matrix instructions a wavefront, and was
+// about 150 vector instructions), so the softmax is arranged to need few:
+//   - FOLD: the queries arrive multiplied by scale * log2(e) (the producer of q
+//     does that before its one rounding), and the score product starts from an
+//     accumulator that holds -reference point: the matrix cores deliver
+//     s * scale * log2(e) - m, ready for exp2, with no multiply-add per score;
+//   - the sums of the probabilities come from the matrix cores as well (one
+//     more product of P with a tile of ones), not from an add per score;
+//   - a lane compares only its own largest score with the threshold; the
+//     maximum over the lanes of a column is taken only when some lane's has
+//     crossed it and the reference point has to move, which is rare.
+template <int NB, bool FOLD>
 struct Columns {
   int tok[NB], head[NB], pos_c[NB], lo_c[NB];
   bf16x8 qf[NB][KK];
-  float m_run[NB], l_run[NB];
+  float thr[NB];                 // a score (less the reference) above this moves the reference; -inf
+                                 // before the column's first visible key, when there is no reference yet
+  f32x4 negm[NB];                // -reference point (units of log 2) in all four entries; 0 before there is one
+  f32x4 l_acc[NB];               // sum of the probabilities, every entry the same
   f32x4 o[NB][DD];
   int kb_begin, kb_end;          // key blocks (of 32) some column sees
   int full_begin, full_end;      // blocks in [full_begin, full_end) are seen whole by every column
@@ -124,8 +140,9 @@ struct Columns {
       const __bf16* q = P.qkv + (size_t)(q0 + tok[b]) * P.row_stride + (size_t)head[b] * D + 8 * gq;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) qf[b][kk] = *(const bf16x8*)(q + 32 * kk);
-      m_run[b] = -INFINITY;
-      l_run[b] = 0.f;
+      thr[b] = -INFINITY;
+      negm[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+      l_acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int dd = 0; dd < DD; ++dd) o[b][dd] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -152,60 +169,93 @@ struct Columns {
     scale_log2 = P.scale * 1.4426950408889634f;
   }
 
-  // One block of 32 keys.  kf: row i of tile m is key kbase + 8 (i / 4) + 4 m + i % 4;
-  // vf: row d of V^T, keys kbase + 8 gq .. + 7.
+  // Scores of tile b for one block of 32 keys, less the reference point and in
+  // units of log 2: this lane gets column n, keys kbase + 8 gq + j, j = 0..7.
+  // kf: row i of tile m is key kbase + 8 (i / 4) + 4 m + i % 4.
+  __device__ __forceinline__ void scores(int b, const bf16x8 (&kf)[2][KK], f32x4& s0, f32x4& s1) const {
+    s0 = FOLD ? negm[b] : f32x4{0.f, 0.f, 0.f, 0.f};
+    s1 = s0;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kk], qf[b][kk], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kk], qf[b][kk], s1, 0, 0, 0);
+    }
+  }
+
+  // From the products to what exp2 takes, with the keys a column does not see
+  // masked out on edge blocks; returns this lane's largest.
+  __device__ __forceinline__ float settle(int b, const f32x4& s0, const f32x4& s1, bool edge, int kbase,
+                                          int gq, float (&s)[8]) const {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float raw = j < 4 ? s0[j] : s1[j - 4];
+      s[j] = FOLD ? raw : fmaf(raw, scale_log2, negm[b][0]);
+    }
+    if (edge) {                                    // a block some column does not see whole
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = kbase + 8 * gq + j;
+        if (key > pos_c[b] || key < lo_c[b]) s[j] = -INFINITY;
+      }
+    }
+    return fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+  }
+
+  // The reference point of a column moves up to its largest score so far (and
+  // is set by the first visible key): outputs and sums are rescaled, the
+  // scores of this block shifted.  It is a reference, not the exact running
+  // maximum: until a score exceeds it by LAZY (in units of log 2) it stays, so
+  // probabilities reach 2^LAZY at most, far from any overflow, with the same
+  // relative rounding, and this path is rare.
+  __device__ __forceinline__ void move(int b, float lane_max, float (&s)[8]) {
+    const float top = column_max(lane_max) - negm[b][0];          // back in absolute units
+    const float m_old = reference(b);
+    if (!(top > m_old)) return;
+    const float alpha = m_old == -INFINITY ? 0.f : fast_exp2(m_old - top);
+    const float shift = -top - negm[b][0];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s[j] += shift;
+    thr[b] = LAZY;
+    negm[b] = f32x4{-top, -top, -top, -top};
+    l_acc[b] *= alpha;
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd) o[b][dd] *= alpha;
+  }
+
+  __device__ __forceinline__ float reference(int b) const {
+    return thr[b] == -INFINITY ? -INFINITY : -negm[b][0];
+  }
+
+  __device__ __forceinline__ bf16x8 probabilities(const float (&s)[8]) const {
+    bf16x8 pb;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pb[j] = (__bf16)fast_exp2(s[j]);
+    return pb;
+  }
+
+  // O^T += V^T P^T and the column sums of P (a tile of ones in the place of V^T).
+  __device__ __forceinline__ void weigh(int b, const bf16x8 (&vf)[DD], const bf16x8& pb) {
+    const __bf16 one = (__bf16)1.0f;
+    const bf16x8 ones = {one, one, one, one, one, one, one, one};
+    l_acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb, l_acc[b], 0, 0, 0);
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd)
+      o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb, o[b][dd], 0, 0, 0);
+  }
+
+  // One block of 32 keys.  vf: row d of V^T, keys kbase + 8 gq .. + 7.
   __device__ __forceinline__ void block(int kb, const bf16x8 (&kf)[2][KK], const bf16x8 (&vf)[DD],
                                         int gq) {
     const int kbase = kb * 32;
     const bool edge = kb >= full_end || kb < full_begin;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kk], qf[b][kk], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kk], qf[b][kk], s1, 0, 0, 0);
-      }
-      // this lane: column n, keys kbase + 8 gq + j, j = 0..7
+      f32x4 s0, s1;
       float s[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) s[j] = j < 4 ? s0[j] : s1[j - 4];
-      if (edge) {                                  // a block some column does not see whole
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int key = kbase + 8 * gq + j;
-          if (key > pos_c[b] || key < lo_c[b]) s[j] = -INFINITY;
-        }
-      }
-      float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
-                       fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-      mx = column_max(mx);
-      // m_run is a reference point, not the exact maximum: it moves only when
-      // the maximum has grown by more than LAZY (in units of log 2), so that
-      // the outputs are rescaled rarely; until then probabilities reach 2^LAZY
-      // at most, far from any overflow, with the same relative rounding.
-      const float mxs = mx * scale_log2;
-      if (__builtin_expect(__any(mxs > m_run[b] + LAZY), 0)) {
-        const float m_new = fmaxf(m_run[b], mxs);
-        const float alpha = fast_exp2(m_run[b] - (m_new == -INFINITY ? 0.f : m_new));
-        m_run[b] = m_new;
-        l_run[b] *= alpha;
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) o[b][dd] *= alpha;
-      }
-      const float neg_m = m_run[b] == -INFINITY ? 0.f : -m_run[b];
-      float psum = 0.f;
-      bf16x8 pb;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float p = fast_exp2(fmaf(s[j], scale_log2, neg_m));
-        psum += p;
-        pb[j] = (__bf16)p;
-      }
-      l_run[b] += psum;
-#pragma unroll
-      for (int dd = 0; dd < DD; ++dd)
-        o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb, o[b][dd], 0, 0, 0);
+      scores(b, kf, s0, s1);
+      const float lane_max = settle(b, s0, s1, edge, kbase, gq, s);
+      if (__builtin_expect(__any(lane_max > thr[b]), 0)) move(b, lane_max, s);
+      weigh(b, vf, probabilities(s));
     }
   }
 
@@ -218,87 +268,25 @@ struct Columns {
     const int kbase = kb * 32;
     const bool edge = kb >= full_end || kb < full_begin;
     f32x4 s0[NB], s1[NB];
-    float s[NB][8], mxs[NB];
-    bool move = false;
-    auto scores = [&](int b) {
-      s0[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-      s1[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float s[NB][8], lane_max[NB];
+    bool crossed = false;
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        s0[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][kk], qf[b][kk], s0[b], 0, 0, 0);
-        s1[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][kk], qf[b][kk], s1[b], 0, 0, 0);
-      }
-    };
-    auto maximum = [&](int b) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) s[b][j] = j < 4 ? s0[b][j] : s1[b][j - 4];
-      if (edge) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int key = kbase + 8 * gq + j;
-          if (key > pos_c[b] || key < lo_c[b]) s[b][j] = -INFINITY;
-        }
-      }
-      float mx = fmaxf(fmaxf(fmaxf(s[b][0], s[b][1]), fmaxf(s[b][2], s[b][3])),
-                       fmaxf(fmaxf(s[b][4], s[b][5]), fmaxf(s[b][6], s[b][7])));
-      mxs[b] = column_max(mx) * scale_log2;
-      move = move || mxs[b] > m_run[b] + LAZY;
-    };
-    // in source order the products of tile b + 1 stand before the vector work
-    // of tile b, which can then run while the matrix cores are busy
-    scores(0);
+    for (int b = 0; b < NB; ++b) scores(b, kf, s0[b], s1[b]);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      if (b + 1 < NB) scores(b + 1);
-      maximum(b);
+      lane_max[b] = settle(b, s0[b], s1[b], edge, kbase, gq, s[b]);
+      crossed = crossed || lane_max[b] > thr[b];
     }
-    if (__builtin_expect(__any(move), 0)) {
+    if (__builtin_expect(__any(crossed), 0)) {
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        const float m_new = fmaxf(m_run[b], mxs[b]);
-        const float alpha = fast_exp2(m_run[b] - (m_new == -INFINITY ? 0.f : m_new));
-        m_run[b] = m_new;
-        l_run[b] *= alpha;
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) o[b][dd] *= alpha;
-      }
+      for (int b = 0; b < NB; ++b) move(b, lane_max[b], s[b]);
     }
     bf16x8 pb[NB];
-    float psum[NB];
-    auto probability = [&](int b, int j) {
-      const float neg_m = m_run[b] == -INFINITY ? 0.f : -m_run[b];
-      const float p = fast_exp2(fmaf(s[b][j], scale_log2, neg_m));
-      psum[b] += p;
-      pb[b][j] = (__bf16)p;
-    };
-    psum[0] = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) probability(0, j);
+    pb[0] = probabilities(s[0]);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      if (b + 1 < NB) psum[b + 1] = 0.f;
-#pragma unroll
-      for (int dd = 0; dd < DD; ++dd) {
-        o[b][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dd], pb[b], o[b][dd], 0, 0, 0);
-        if (b + 1 < NB) {                        // the next tile's probabilities, spread over these products
-#pragma unroll
-          for (int j = 8 * dd / DD; j < 8 * (dd + 1) / DD; ++j) probability(b + 1, j);
-        }
-      }
-      l_run[b] += psum[b];
-    }
-    if (NB == 2) {
-      // order asked of the scheduler for the straight-line stretch above: the
-      // first tile's probabilities, then one output product of the first tile
-      // per few vector instructions of the second tile's probabilities, then
-      // the second tile's products (0x402: vector and transcendental, 0x8: matrix)
-      __builtin_amdgcn_sched_group_barrier(0x402, 30, 0);
-#pragma unroll
-      for (int dd = 0; dd < DD; ++dd) {
-        __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x402, 32 / DD, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x8, DD, 0);
+      if (b + 1 < NB) pb[b + 1] = probabilities(s[b + 1]);       // beside the products of tile b
+      weigh(b, vf, pb[b]);
     }
   }
 
@@ -307,7 +295,7 @@ struct Columns {
   __device__ __forceinline__ void store(const AttnParams& P, int q0, int split, int gq) {
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      const float l = column_sum(l_run[b]);
+      const float l = l_acc[b][0];
       if (pos_c[b] < 0) continue;
       const size_t row = (size_t)(q0 + tok[b]);
       if (SPLIT) {
@@ -316,7 +304,7 @@ struct Columns {
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd) *(f32x4*)(po + 16 * dd) = o[b][dd];
         if (gq == 0) {
-          P.part_ml[pr * 2] = m_run[b];
+          P.part_ml[pr * 2] = reference(b);
           P.part_ml[pr * 2 + 1] = l;
         }
       } else {
@@ -337,7 +325,7 @@ struct Columns {
 // One wavefront per workgroup; operands straight from the pages.  Used for
 // decode tokens (SPLIT: the wavefront takes one share of the key blocks) and
 // for prompt portions whose launch does not saturate L2.
-template <int NB, bool SPLIT>
+template <int NB, bool SPLIT, bool FOLD>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 256 ? 2 : 1))) void attention_mfma_kernel(const AttnParams P) {
   const int lane = threadIdx.x, n = lane & 15, gq = lane >> 4;
   const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
@@ -353,7 +341,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 25
   const int* table = P.block_tables + (size_t)seq * P.max_pages;
   const int page = P.page, page_shift = 31 - __builtin_clz(page);
 
-  Columns<NB> C;
+  Columns<NB, FOLD> C;
   C.init(P, q0, ncols, tile * 16 * NB, pos0, kvh, g, n, gq);
   int kb_begin = C.kb_begin, kb_end = C.kb_end;
   if (SPLIT) {
@@ -411,25 +399,60 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 25
 // cache hierarchy once per 128 columns instead of once per 32 (measured on
 // MI355X: with one wavefront per workgroup the kernel ran at the rate at which
 // L2 delivers the operands, 32 flop a byte, not at the rate of the matrix
-// cores).  Two buffers: the next block travels pages -> registers while this
-// one is computed, registers -> LDS afterwards, one barrier a block.
+// cores).
 //
-// LDS rows are padded by 16 bytes, which makes the row stride an odd number
-// of 16-byte units: the 16 lanes that read one operand column of a tile
-// (rows r..r+15, same offset) then fall into 16 different bank groups.  K rows
-// are stored in the order the product wants them (tile m, row i), not in key
-// order.
+// The blocks travel from the pages straight into LDS (global_load_lds_dwordx4
+// of gfx950: a wavefront's 64 loads of 16 bytes land side by side in 1 KB of
+// LDS, each lane choosing its own source), into a ring of STAGES buffers:
+// while block kb is computed, the loads of the next STAGES - 1 blocks are on
+// their way, no register carries them, no wavefront writes them to LDS, and
+// the one wait before the barrier at the end of a block is for loads asked for
+// a whole block earlier.  (Measured with the loads going through registers
+// and ds_write, one block ahead: the staging alone cost 28 % of the kernel's
+// time at 8,192 tokens, the loads and the writes about equally.)
+//
+// A stage holds K as 32 rows of D / 8 units of 16 bytes, in the order the
+// score product wants its rows (tile m, row i), and then V^T as D rows of 4
+// units.  No padding: a lane can put any unit anywhere at no cost, so the units
+// of K row r are rotated by r % 16 places, which spreads the 16 lanes that read one
+// operand column of a tile (rows r..r+15, same channel) over the banks; V^T's
+// reads cover 1 KB side by side as they are.
+typedef const __attribute__((address_space(4))) int* ConstInts;
 constexpr int SHARED_WAVES = 4;
-constexpr int KS = D + 8;                          // K row stride in LDS, elements
-constexpr int VS = 32 + 8;                         // V^T row stride
-constexpr int STAGE = (4 * D + 64 * SHARED_WAVES - 1) / (64 * SHARED_WAVES);   // 16-byte units a thread carries, K and V each
-constexpr bool SHARED_FITS = 2 * (32 * KS + D * VS) * 2 <= 65536;
+constexpr int KU = D / 8;                          // 16-byte units in a row of K
+constexpr int STAGE_UNITS = 8 * D;                 // K: 32 rows x KU, then V^T: D rows x 4
+constexpr int STAGE_BYTES = 16 * STAGE_UNITS;
+constexpr int STAGES = 3 * STAGE_BYTES <= 65536 ? 3 : 2;
+constexpr int CHUNKS = STAGE_UNITS / 64;           // wavefront-wide loads a block: D / 8, half of them K
+constexpr int LOADS = CHUNKS / SHARED_WAVES;       // ... per wavefront: D / 32
+constexpr bool SHARED_FITS = STAGES * STAGE_BYTES <= 65536;
+struct Stage0 { static constexpr int value = 0; };
+struct Stage1 { static constexpr int value = 1; };
+struct Stage2 { static constexpr int value = 2; };
 
+// One wavefront-wide load of 16 bytes a lane from `from` (any address per lane) to the 1 KB of
+// LDS at byte `lds_at` (the same for all lanes): lane i's bytes land at lds_at + 16 i.  Written
+// out as the instruction, with the compiler told nothing of what it writes: told, it waits for
+// every such load before the next read of LDS that it cannot tell apart, which is all of them,
+// and the loads would never be more than one block ahead.  The waits are explicit instead
+// (wait_loads below; the loads complete in order).
+__device__ __forceinline__ void load_to_lds(const void* from, unsigned lds_at) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(from), "s"(lds_at) : "m0");
+}
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters left at their maxima)
+template <int N> __device__ __forceinline__ void wait_loads() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+template <bool FOLD>
 __global__ __launch_bounds__(64 * SHARED_WAVES) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1)))
 void attention_mfma_shared_kernel(const AttnParams P) {
-  constexpr int NB = 2, THREADS = 64 * SHARED_WAVES, COLS = 16 * NB * SHARED_WAVES;
-  __shared__ __attribute__((aligned(16))) __bf16 k_lds[2][SHARED_FITS ? 32 * KS : 8];
-  __shared__ __attribute__((aligned(16))) __bf16 v_lds[2][SHARED_FITS ? D * VS : 8];
+  constexpr int NB = 2, COLS = 16 * NB * SHARED_WAVES;
+  // one array per stage, so that the compiler can tell the loads into one from the reads of another
+  __shared__ __attribute__((aligned(1024))) char ring0[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char ring1[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char ring2[STAGES == 3 ? STAGE_BYTES : 16];
   // (wave as a scalar: the products below sit under conditions that depend on it, and matrix
   // instructions ignore the execution mask)
   const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63, n = lane & 15, gq = lane >> 4;
@@ -440,8 +463,65 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   const int ncols = qlen * g;
   const int ntiles = (ncols + COLS - 1) / COLS;
   const int pos0 = P.positions[q0];
-  const int* table = P.block_tables + (size_t)seq * P.max_pages;
+  // (read through the constant address space: the same entries for all lanes, so they come by
+  // scalar loads into scalar registers, and the addresses made from them cost no vector work)
+  const ConstInts table = (ConstInts)(P.block_tables + (size_t)seq * P.max_pages);
   const int page = P.page, page_shift = 31 - __builtin_clz(page);
+
+  // What a lane fetches is fixed for the whole kernel: unit u = 64 chunk + lane of a stage.
+  // K unit (row r = 16 m + i, place s) holds channels 8 ((s - i) mod KU) of key
+  // 8 (i / 4) + 4 m + i % 4; V^T unit (row d, place q) holds keys 8 q .. 8 q + 7 of channel d.
+  int src[LOADS];                                    // offset inside the page's slice of this kv head, elements
+  bool second[LOADS];                                // the unit lies in the second page of the block (16-key pages)
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int u = 64 * (wave + SHARED_WAVES * i) + lane;
+    if (u < 32 * KU) {
+      const int r = u / KU, c = (u % KU + KU - (r & 15) % KU) % KU;
+      const int ko = 8 * ((r & 15) >> 2) + 4 * (r >> 4) + (r & 3);
+      src[i] = (ko & (page - 1)) * D + 8 * c;
+      second[i] = ko >= 16;
+    } else {
+      const int d = (u - 32 * KU) >> 2, q = u & 3;
+      src[i] = d * page + ((8 * q) & (page - 1));
+      second[i] = q >= 2;
+    }
+  }
+  const size_t per_page = (size_t)P.nkv * page * D, head_at = (size_t)kvh * page * D;   // elements
+  // where this lane reads its operands in a stage: K row 16 m + n, channels 32 kk + 8 gq (the place
+  // of unit 4 kk + gq rotated by the row); V^T row 16 dd + n, keys 8 gq
+  int k_at[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) k_at[kk] = 16 * (n * KU + (4 * kk + gq + n) % KU);
+  const int v_at = 16 * 32 * KU + 64 * n + 16 * gq;
+
+  auto ring = [&](auto stage) -> char* {
+    constexpr int S = decltype(stage)::value;
+    return S == 0 ? ring0 : S == 1 ? ring1 : ring2;
+  };
+  int pg[2];
+  auto load_pages = [&](int kb) {
+    const int kbase = kb * 32;
+    pg[0] = table[kbase >> page_shift];
+    pg[1] = table[(kbase + 16) >> page_shift];
+  };
+  // ask for block kb into a stage (its page ids are in pg)
+  auto fetch = [&](int kb, auto stage) {
+    const int within = (kb * 32) & (page - 1);       // where the block starts inside its page (64-key pages: 0 or 32)
+    const __bf16* k0 = P.kc + ((size_t)pg[0] * per_page + head_at + (size_t)within * D);
+    const __bf16* k1 = P.kc + ((size_t)pg[1] * per_page + head_at + (size_t)within * D);
+    const __bf16* v0 = P.vc + ((size_t)pg[0] * per_page + head_at + within);
+    const __bf16* v1 = P.vc + ((size_t)pg[1] * per_page + head_at + within);
+    const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)ring(stage);
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int chunk = wave + SHARED_WAVES * i;
+      const bool keys = chunk < CHUNKS / 2;            // the same for the whole wavefront
+      const __bf16* from = (second[i] ? (keys ? k1 : v1) : (keys ? k0 : v0)) + src[i];
+      load_to_lds(from, base + 1024 * chunk);
+    }
+  };
+
   // A workgroup takes a late tile (many key blocks) and then the early tile
   // that mirrors it (few): every workgroup of a sequence then has about the
   // same number of blocks and none is left running alone at the end (MI355X,
@@ -461,7 +541,7 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   const int wg_c0 = tile * COLS;
   const int c0 = wg_c0 + 16 * NB * wave;
   const bool active = c0 < ncols;                  // a wavefront past the last column only helps loading
-  Columns<NB> C;
+  Columns<NB, FOLD> C;
   C.init(P, q0, ncols, active ? c0 : wg_c0, pos0, kvh, g, n, gq);
 
   // key blocks of the workgroup: from the first block its first wavefront
@@ -476,72 +556,63 @@ void attention_mfma_shared_kernel(const AttnParams P) {
     wg_begin = first + (int)((long long)nblk * split / P.nsplit);
     wg_end = first + (int)((long long)nblk * (split + 1) / P.nsplit);
   }
-
-  bf16x8 k_stage[STAGE], v_stage[STAGE];
-  int pg[2];
-  auto load_pages = [&](int kb) {
-    const int kbase = kb * 32;
-    pg[0] = table[kbase >> page_shift];
-    pg[1] = table[(kbase + 16) >> page_shift];
-  };
-  // 16-byte unit id of K: key id / (D/8), channels 8 (id % (D/8));  of V^T: row id / 4, keys 8 (id % 4)
-  auto stage_load = [&](int kb) {
-    const int kbase = kb * 32;
-#pragma unroll
-    for (int i = 0; i < STAGE; ++i) {
-      const int id = t + THREADS * i;
-      if (id < 4 * D) {
-        const int ko = id / (D / 8), c = id % (D / 8);
-        const int p = ko < 16 ? pg[0] : pg[1];
-        k_stage[i] = *(const bf16x8*)(P.kc + (((size_t)p * P.nkv + kvh) * page + ((kbase + ko) & (page - 1))) * D + 8 * c);
-        const int d = id >> 2, q = id & 3;
-        const int pv = q < 2 ? pg[0] : pg[1];
-        v_stage[i] = *(const bf16x8*)(P.vc + (((size_t)pv * P.nkv + kvh) * D + d) * page + ((kbase + 8 * q) & (page - 1)));
-      }
-    }
-  };
-  auto stage_store = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < STAGE; ++i) {
-      const int id = t + THREADS * i;
-      if (id < 4 * D) {
-        const int ko = id / (D / 8), c = id % (D / 8);
-        const int row = 16 * ((ko >> 2) & 1) + 4 * (ko >> 3) + (ko & 3);   // key ko is row i = 4 (ko / 8) + ko % 4 of tile (ko / 4) % 2
-        *(bf16x8*)&k_lds[buf][row * KS + 8 * c] = k_stage[i];
-        const int d = id >> 2, q = id & 3;
-        *(bf16x8*)&v_lds[buf][d * VS + 8 * q] = v_stage[i];
-      }
-    }
-  };
-
   const int last = wg_end - 1;
-  if (wg_begin < wg_end) {                           // (a share may be empty; the same for the whole workgroup)
-  load_pages(wg_begin);
-  stage_load(wg_begin);
-  load_pages(wg_begin + 1 < last ? wg_begin + 1 : last);
-  stage_store(0);
-  __syncthreads();
-  }
-  for (int kb = wg_begin; kb < wg_end; ++kb) {
-    const int buf = (kb - wg_begin) & 1;
-    const bool more = kb + 1 < wg_end;
+
+  // one block: ask for block kb + STAGES - 1 (into the stage that block kb - 1 was read from; the
+  // barrier that ended that block has passed), compute block kb out of `here`, then make sure
+  // that this wavefront's loads of block kb + 1 have landed and meet the others
+  auto step = [&](int kb, auto here, auto ahead) {
+    const bool more = kb + STAGES - 1 < wg_end;
     if (more) {
-      stage_load(kb + 1);
-      load_pages(kb + 2 < last ? kb + 2 : last);
+      fetch(kb + STAGES - 1, ahead);
+      load_pages(kb + STAGES < last ? kb + STAGES : last);
     }
     if (active && kb >= C.kb_begin && kb < C.kb_end) {
+      const char* at = ring(here);
       bf16x8 kf[2][KK], vf[DD];
 #pragma unroll
       for (int m = 0; m < 2; ++m)
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk)
-          kf[m][kk] = *(const bf16x8*)&k_lds[buf][(16 * m + n) * KS + 32 * kk + 8 * gq];
+        for (int kk = 0; kk < KK; ++kk) kf[m][kk] = *(const bf16x8*)(at + 256 * KU * m + k_at[kk]);
 #pragma unroll
-      for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)&v_lds[buf][(16 * dd + n) * VS + 8 * gq];
+      for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)(at + v_at + 1024 * dd);
       C.block_abreast(kb, kf, vf, gq);
     }
-    if (more) stage_store(buf ^ 1);
-    __syncthreads();                               // the other buffer is complete; this one is free
+    if (more && STAGES == 3) wait_loads<LOADS>();    // all but the block just asked for
+    else wait_loads<0>();
+    // (the bare barrier: __syncthreads() would first wait for every load on its way, the block
+    // just asked for included; what must be complete here is this wavefront's share of block
+    // kb + 1, waited for above, and its reads of block kb, whose values the products have used)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" : : : "memory");               // (the compiler reads LDS again from here on, whatever it held)
+  };
+
+  if (wg_begin < wg_end) {                           // (a share may be empty; the same for the whole workgroup)
+    load_pages(wg_begin);
+    fetch(wg_begin, Stage0{});
+    load_pages(wg_begin + 1 < last ? wg_begin + 1 : last);
+    if (STAGES == 3) {
+      if (wg_begin + 1 < wg_end) fetch(wg_begin + 1, Stage1{});
+      load_pages(wg_begin + 2 < last ? wg_begin + 2 : last);
+      if (wg_begin + 1 < wg_end) wait_loads<LOADS>();
+      else wait_loads<0>();
+    } else {
+      wait_loads<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" : : : "memory");
+  }
+  if (STAGES == 3) {
+    for (int kb = wg_begin; kb < wg_end; kb += 3) {
+      step(kb, Stage0{}, Stage2{});
+      if (kb + 1 < wg_end) step(kb + 1, Stage1{}, Stage0{});
+      if (kb + 2 < wg_end) step(kb + 2, Stage2{}, Stage1{});
+    }
+  } else {
+    for (int kb = wg_begin; kb < wg_end; kb += 2) {
+      step(kb, Stage0{}, Stage1{});
+      if (kb + 1 < wg_end) step(kb + 1, Stage1{}, Stage0{});
+    }
   }
   if (active) {
     if (P.nsplit > 1) C.template store<true>(P, q0, split, gq);
@@ -618,15 +689,23 @@ extern "C" const char* sl_attention_mfma(
                max_pages, cu_q, positions, seq_begin, nh, nkv, page, scale, window, nsplit,
                (__bf16*)out, part_o, part_ml, part_row0, pair_tiles};
   const long long cols = (long long)max_q_len * g;
+  // scale * log2(e) == 1: the caller's q is already in units of log 2 (see Columns)
+  const bool fold = fabsf(scale * 1.4426950408889634f - 1.f) < 1e-6f;
   if (nsplit > 1 && max_q_len == 1) {
     SL_CHECK(part_o != nullptr && part_ml != nullptr && part_rows == num_seqs,
              "attention_mfma: a split launch needs partial buffers for its rows");
     SL_CHECK(g <= 64, "attention_mfma: more than 64 query heads per kv head");
     SL_CHECK(nsplit <= 64, "attention_mfma: at most 64 splits of the context");
     const dim3 grid(nsplit, nkv, num_seqs);
-    if (g <= 16) attention_mfma_kernel<1, true><<<grid, 64, 0, stream>>>(P);
-    else if (g <= 32) attention_mfma_kernel<2, true><<<grid, 64, 0, stream>>>(P);
-    else attention_mfma_kernel<4, true><<<grid, 64, 0, stream>>>(P);
+    if (fold) {
+      if (g <= 16) attention_mfma_kernel<1, true, true><<<grid, 64, 0, stream>>>(P);
+      else if (g <= 32) attention_mfma_kernel<2, true, true><<<grid, 64, 0, stream>>>(P);
+      else attention_mfma_kernel<4, true, true><<<grid, 64, 0, stream>>>(P);
+    } else {
+      if (g <= 16) attention_mfma_kernel<1, true, false><<<grid, 64, 0, stream>>>(P);
+      else if (g <= 32) attention_mfma_kernel<2, true, false><<<grid, 64, 0, stream>>>(P);
+      else attention_mfma_kernel<4, true, false><<<grid, 64, 0, stream>>>(P);
+    }
     const char* e = sl_launch_status();
     if (e) return e;
     attention_combine_kernel<<<dim3(num_seqs, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh,
@@ -649,13 +728,17 @@ extern "C" const char* sl_attention_mfma(
              "attention_mfma: a split launch needs partial buffers for its rows and at most 64 splits");
   }
   if (cols <= 16) {
-    attention_mfma_kernel<1, false><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);
+    if (fold) attention_mfma_kernel<1, false, true><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);
+    else attention_mfma_kernel<1, false, false><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);
   } else if (!shared) {
-    attention_mfma_kernel<2, false><<<dim3((unsigned)tiles, nkv, num_seqs), 64, 0, stream>>>(P);
+    const dim3 grid((unsigned)tiles, nkv, num_seqs);
+    if (fold) attention_mfma_kernel<2, false, true><<<grid, 64, 0, stream>>>(P);
+    else attention_mfma_kernel<2, false, false><<<grid, 64, 0, stream>>>(P);
   } else {
     const long long wg = (tiles + SHARED_WAVES - 1) / SHARED_WAVES;
-    attention_mfma_shared_kernel<<<dim3((unsigned)(pair_tiles ? (wg + 1) / 2 : wg * nsplit), nkv, num_seqs),
-                                   64 * SHARED_WAVES, 0, stream>>>(P);
+    const dim3 grid((unsigned)(pair_tiles ? (wg + 1) / 2 : wg * nsplit), nkv, num_seqs);
+    if (fold) attention_mfma_shared_kernel<true><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
+    else attention_mfma_shared_kernel<false><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
     if (nsplit > 1) {
       const char* e = sl_launch_status();
       if (e) return e;

@@ -145,8 +145,9 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const SplitProduct sp
                                   const float* __restrict__ cosv,
                                   const float* __restrict__ sinv, const int* __restrict__ slots,
                                   act_t* __restrict__ kc, act_t* __restrict__ vc, int nh, int nkv,
-                                  int D, int rot, int page, int pairs8) {
+                                  int D, int rot, int page, int pairs8, float qscale) {
   const int t = blockIdx.x, hd = blockIdx.y;
+  const float qs = hd < nh ? qscale : 1.f;         // q heads leave multiplied by qscale
   const int half = rot / 2;
   const size_t row = ((size_t)t * (nh + 2 * nkv) + hd) * D;
   act_t* x = qkv + row;
@@ -172,8 +173,10 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const SplitProduct sp
         x1 = r1;
         x2 = r2;
       }
-      // in place: whatever was rotated; from partial sums: q (k lives on in the pages only)
-      if (sp.parts != nullptr ? hd < nh : cosv != nullptr) {
+      x1 *= qs;
+      x2 *= qs;
+      // in place: whatever changed; from partial sums: q (k lives on in the pages only)
+      if (sp.parts != nullptr ? hd < nh : (cosv != nullptr || qs != 1.f)) {
         x[p1] = from_f<act_t>(x1);
         x[p2] = from_f<act_t>(x2);
       }
@@ -183,8 +186,8 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const SplitProduct sp
       }
     }
     for (int c = rot + threadIdx.x; c < D; c += blockDim.x) {       // channels beyond the rotated ones pass
-      const float v = input(c);
-      if (sp.parts != nullptr && hd < nh) x[c] = from_f<act_t>(v);
+      const float v = input(c) * qs;
+      if (hd < nh && (sp.parts != nullptr || qs != 1.f)) x[c] = from_f<act_t>(v);
       if (dst != nullptr) dst[c] = from_f<act_t>(v);
     }
   } else if (vc != nullptr) {
@@ -208,7 +211,7 @@ struct __attribute__((aligned(16))) F4 { float v[4]; };
 __global__ __launch_bounds__(256) void rope_store_qk_kernel(
     act_t* __restrict__ qkv, const float* __restrict__ cosv, const float* __restrict__ sinv,
     const int* __restrict__ slots, act_t* __restrict__ kc, int nh, int nkv, int D, int rot,
-    int page, int pairs8) {
+    int page, int pairs8, float qscale) {
   const int t = blockIdx.x, half = rot / 2, chunks = D / 16, rotated = rot / 16;
   const int items = (nh + nkv) * chunks;
   for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < items; w += gridDim.y * blockDim.x) {
@@ -218,17 +221,21 @@ __global__ __launch_bounds__(256) void rope_store_qk_kernel(
     const int p1 = !turn || pairs8 ? 16 * c : 8 * c, p2 = !turn || pairs8 ? p1 + 8 : p1 + half;
     act_t* x = qkv + ((size_t)t * (nh + 2 * nkv) + hd) * D;
     Act8 a = *(const Act8*)(x + p1), b = *(const Act8*)(x + p2);
-    if (cosv != nullptr && turn) {
-      const float* cp = cosv + (size_t)t * half + 8 * c;
-      const float* sp = sinv + (size_t)t * half + 8 * c;
-      const F4 c0 = *(const F4*)cp, c1 = *(const F4*)(cp + 4);
-      const F4 s0 = *(const F4*)sp, s1 = *(const F4*)(sp + 4);
+    const float qs = hd < nh ? qscale : 1.f;
+    if ((cosv != nullptr && turn) || qs != 1.f) {
+      F4 c0{{1.f, 1.f, 1.f, 1.f}}, c1 = c0, s0{{0.f, 0.f, 0.f, 0.f}}, s1 = s0;
+      if (cosv != nullptr && turn) {
+        const float* cp = cosv + (size_t)t * half + 8 * c;
+        const float* sp = sinv + (size_t)t * half + 8 * c;
+        c0 = *(const F4*)cp, c1 = *(const F4*)(cp + 4);
+        s0 = *(const F4*)sp, s1 = *(const F4*)(sp + 4);
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float cs = j < 4 ? c0.v[j] : c1.v[j - 4], sn = j < 4 ? s0.v[j] : s1.v[j - 4];
         const float x1 = to_f(a.v[j]), x2 = to_f(b.v[j]);
-        a.v[j] = from_f<act_t>(x1 * cs - x2 * sn);
-        b.v[j] = from_f<act_t>(x2 * cs + x1 * sn);
+        a.v[j] = from_f<act_t>((x1 * cs - x2 * sn) * qs);
+        b.v[j] = from_f<act_t>((x2 * cs + x1 * sn) * qs);
       }
       *(Act8*)(x + p1) = a;
       *(Act8*)(x + p2) = b;
@@ -269,10 +276,13 @@ __global__ __launch_bounds__(256) void store_v_kernel(
 
 // parts != nullptr: the input is the sum of nparts float partial products
 // [nparts][T][N] plus bias; q is then written to qkv, k and v only to the pages.
+// qscale: q heads are multiplied by it after the rotation and before their one
+// rounding (an attention kernel that wants its scores in units of log 2 asks
+// for scale * log2(e) here and then needs no multiply per score).
 extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* sinv,
                                      const int* slots, void* kc, void* vc, int T, int nh, int nkv,
                                      int D, int rot, int page, int pairs8, const float* parts,
-                                     int nparts, const float* bias, hipStream_t stream) {
+                                     int nparts, const float* bias, float qscale, hipStream_t stream) {
   SL_CHECK(T >= 0 && nh > 0 && nkv > 0, "rope_store: sizes must be positive");
   SL_CHECK(D > 0 && rot >= 0 && rot <= D && rot % 2 == 0,
            "rope_store: the rotated width must be even and at most head_dim");
@@ -286,14 +296,14 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
   const SplitProduct sp{parts, nparts, (size_t)T * (nh + 2 * nkv) * D, bias};
   if (T == 0) return nullptr;
   const int heads = kc != nullptr ? nh + 2 * nkv : nh + nkv;
-  if (cosv == nullptr && kc == nullptr && parts == nullptr) return nullptr;
+  if (cosv == nullptr && kc == nullptr && parts == nullptr && qscale == 1.f) return nullptr;
   const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kc % 16) == 0 &&
                        ((uintptr_t)cosv % 16) == 0 && ((uintptr_t)sinv % 16) == 0;
   if (parts == nullptr && T >= VECTOR_MIN_TOKENS && D % 16 == 0 && rot % 16 == 0 && D <= 256 && aligned &&
       nkv <= 65535) {
     const int items = (nh + nkv) * (D / 16);
     rope_store_qk_kernel<<<dim3(T, (items + 255) / 256 < 64 ? (items + 255) / 256 : 64), 256, 0, stream>>>(
-        (act_t*)qkv, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, rot, page, pairs8);
+        (act_t*)qkv, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, rot, page, pairs8, qscale);
     const char* e = sl_launch_status();
     if (e || vc == nullptr) return e;
     store_v_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>((const act_t*)qkv, slots, (act_t*)vc, T,
@@ -301,6 +311,6 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
     return sl_launch_status();
   }
   rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, sp, cosv, sinv, slots, (act_t*)kc,
-                                                       (act_t*)vc, nh, nkv, D, rot, page, pairs8);
+                                                       (act_t*)vc, nh, nkv, D, rot, page, pairs8, qscale);
   return sl_launch_status();
 }

@@ -370,6 +370,7 @@ struct RopeStore {
   __bf16* vc;                // [pages, nkv, D, page]
   int nh, nkv, D, page;
   int rot;                   // the first rot channels of a head are rotated (rot % 16 == 0), the rest pass
+  float qscale;              // q heads are multiplied by this before their rounding (1: as they are)
 };
 
 // NT tiles (16 columns of y each) per workgroup share every load of x: with 8
@@ -527,7 +528,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
             val = p % 16 < 8 ? s * c - partner * sn : s * c + partner * sn;
           }
           if (hd < R.nh) {
-            ((__bf16*)y)[(size_t)m * N + n] = (__bf16)val;
+            ((__bf16*)y)[(size_t)m * N + n] = (__bf16)(val * R.qscale);
           } else if (R.slots != nullptr) {
             const int slot = R.slots[m];
             R.kc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh)) * R.page + slot % R.page) * R.D + p] = (__bf16)val;

@@ -41,7 +41,7 @@ class _RopeStore(ctypes.Structure):
     """``RopeStore`` of gemm.hip."""
     _fields_ = [("cosv", _c_void_p), ("sinv", _c_void_p), ("slots", _c_void_p), ("kc", _c_void_p),
                 ("vc", _c_void_p), ("nh", _c_int), ("nkv", _c_int), ("D", _c_int), ("page", _c_int),
-                ("rot", _c_int)]
+                ("rot", _c_int), ("qscale", _c_float)]
 
 
 class RotationPlan:
@@ -621,14 +621,15 @@ class HipOps:
         return pages
 
     def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                   pairs8=False, split=None, rot_dim=None):
+                   pairs8=False, split=None, rot_dim=None, q_scale=1.0):
         """Rotate q and k of ``qkv`` in place (``cos`` None: no rotation) and write
         k and v to their cache rows (``k_cache`` None: no write).  The first
         ``rot_dim`` channels of a head are rotated (default: all), pair j being
         (j, j + rot_dim / 2); ``pairs8``: they come in blocks of 8 channels and
         their 8 partners (the order ``qkv_rope_store`` uses) instead.
         ``split``: the product arrives as ``PartialSums``; ``qkv`` is then only
-        written (its q columns)."""
+        written (its q columns).  ``q_scale`` multiplies the q heads after the
+        rotation, before their rounding."""
         T = qkv.shape[0]
         rot = D if rot_dim is None else int(rot_dim)
         if rot % 2 or not 0 <= rot <= D or (pairs8 and rot % 16) or (cos is not None and rot == 0):
@@ -649,10 +650,10 @@ class HipOps:
             self._check(slots, torch.int32, (T,), "slots")
         self._call("elementwise", "sl_rope_store", _p(qkv), _p(cos), _p(sin), _p(slots),
                    _p(k_cache), _p(v_cache), T, nh, nkv, D, rot, page_size, int(pairs8),
-                   _p(parts), parts.shape[0] if parts is not None else 0, _p(bias))
+                   _p(parts), parts.shape[0] if parts is not None else 0, _p(bias), _c_float(q_scale))
 
     def qkv_rope_store(self, x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
-                       page_size, rot_dim=None):
+                       page_size, rot_dim=None, q_scale=1.0):
         """q/k/v product, rotation and cache write.  The rows of ``weight`` (and
         ``bias``) hold every q and k head in the blocked pair order (``pairs8``
         above).  Returns the [T, (nh + 2 nkv) D] buffer whose q columns the
@@ -676,7 +677,7 @@ class HipOps:
                 if isinstance(product, PartialSums):
                     qkv = self._new((M, N))
                     self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                                    True, split=product, rot_dim=rot)
+                                    True, split=product, rot_dim=rot, q_scale=q_scale)
                     return qkv
                 qkv = product
             elif (self.act_dtype == torch.bfloat16 and not isinstance(x, ScaledRows)
@@ -687,12 +688,13 @@ class HipOps:
                 sums = self.library_sums(x, self.rows_of(weight), torch.float32)
                 qkv = self._new((M, N))
                 self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                                True, split=PartialSums(sums.unsqueeze(0), bias), rot_dim=rot)
+                                True, split=PartialSums(sums.unsqueeze(0), bias), rot_dim=rot,
+                                q_scale=q_scale)
                 return qkv
             else:
                 qkv = self.linear(x, weight, bias)
             self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True,
-                            rot_dim=rot)
+                            rot_dim=rot, q_scale=q_scale)
             return qkv
         scaled = x if isinstance(x, ScaledRows) else None
         if scaled is None:
@@ -706,7 +708,7 @@ class HipOps:
             self._check_pages(k_cache, v_cache, nkv, D, page_size)
             self._check(slots, torch.int32, (M,), "slots")
         rope = _RopeStore(_ptr(cos), _ptr(sin), _ptr(slots if k_cache is not None else None),
-                          _ptr(k_cache), _ptr(v_cache), nh, nkv, D, page_size, rot)
+                          _ptr(k_cache), _ptr(v_cache), nh, nkv, D, page_size, rot, q_scale)
         qkv = self._new((M, N))
         self._skinny(scaled.x if scaled is not None else x, weight, bias, qkv, M, N, K,
                      scaled=scaled, rope=rope)
@@ -740,14 +742,27 @@ class HipOps:
         plain = order == list(range(D))
         return RotationPlan(None if plain else torch.tensor(order, dtype=torch.long), rot, blocked)
 
+    LOG2E = 1.4426950408889634
+
+    def split_attention_scale(self, scale: float):
+        """(factor for q at its producer, scale left for ``paged_attention``).
+        The matrix-core attention kernels want their scores in units of log 2:
+        q then leaves ``project_qkv`` multiplied by scale * log2(e) (before its
+        one rounding) and the attention call gets ln 2, whose product with
+        log2(e) is 1, so no multiply-add per score is left.  The float32 table
+        keeps the scale where the reference has it."""
+        if self.act_dtype != torch.bfloat16 or not self.use_mfma_attention:
+            return 1.0, float(scale)
+        return float(scale) * self.LOG2E, 1.0 / self.LOG2E
+
     def project_qkv(self, x, weight, bias, nh, nkv, D, plan, tables, slots, k_cache, v_cache,
-                    page_size):
+                    page_size, q_scale=1.0):
         """What a mixer calls: the q/k/v product of ``x`` (rows of ``weight`` in
         the order of ``plan``), the position encoding's work on q and k for this
         step's ``tables`` (whatever the encoding's ``tables()`` returned: None,
         or an object with ``cos`` and ``sin`` [T, rot_dim / 2]) and the write of
         k and v into the cache.  Returns [T, (nh + 2 nkv) D] whose q columns the
-        attention reads."""
+        attention reads, multiplied by ``q_scale`` (see ``split_attention_scale``)."""
         cos = sin = None
         if tables is not None:
             cos, sin = getattr(tables, "cos", None), getattr(tables, "sin", None)
@@ -758,10 +773,10 @@ class HipOps:
                 raise KernelError("the position encoding gives tables but its layout rotates nothing")
         if plan.blocked:
             return self.qkv_rope_store(x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
-                                       page_size, rot_dim=plan.rot_dim)
+                                       page_size, rot_dim=plan.rot_dim, q_scale=q_scale)
         qkv = self.linear(x, weight, bias)
         self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
-                        rot_dim=plan.rot_dim)
+                        rot_dim=plan.rot_dim, q_scale=q_scale)
         return qkv
 
     # ------------------------------------------------------------ attention

@@ -76,6 +76,9 @@ class PagedAttention(Mixer):
                  reorder(tensors("k_proj.bias").float(), self.num_kv_heads),
                  tensors("v_proj.bias").float()], 0))
         self.w_o = rt.linear_weight(tensors("o_proj.weight"))
+        # a kernel table may want part of the score scale applied to q where q is made
+        split = getattr(rt.ops, "split_attention_scale", None)
+        self.q_scale, self.score_scale = split(self.scale) if split is not None else (1.0, self.scale)
 
     # ---- compute
     def forward(self, x, batch, cache, shared):
@@ -84,8 +87,8 @@ class PagedAttention(Mixer):
         slots, kc, vc = (group.slots, cache.k, cache.v) if cache.write else (None, None, None)
         qkv = ops.project_qkv(x, self.w_qkv, self.b_qkv, self.num_heads, self.num_kv_heads,
                               self.head_dim, self.rotation, self.position.tables(batch, shared),
-                              slots, kc, vc, cache.page_size)
+                              slots, kc, vc, cache.page_size, q_scale=self.q_scale)
         attn = ops.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
-            cache.page_size, group.block_tables, batch, self.scale, self.window)
+            cache.page_size, group.block_tables, batch, self.score_scale, self.window)
         return ops.linear(attn, self.w_o, None, defer=True)

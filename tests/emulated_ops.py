@@ -110,7 +110,9 @@ class EmulatedOps:
                                torch.arange(rot, head_dim)])
         return types.SimpleNamespace(order=order, rot_dim=rot, blocked=False)
 
-    def project_qkv(self, x, w, bias, nh, nkv, D, plan, tables, slots, k_cache, v_cache, page_size):
+    def project_qkv(self, x, w, bias, nh, nkv, D, plan, tables, slots, k_cache, v_cache, page_size,
+                    q_scale=1.0):
+        assert q_scale == 1.0                # (this table leaves the whole scale to paged_attention)
         qkv = self.linear(x, w, bias)
         cos, sin = (tables.cos, tables.sin) if tables is not None else (None, None)
         self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, False,

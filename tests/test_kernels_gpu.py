@@ -409,6 +409,17 @@ def test_rope_store_of_a_part_of_the_head(both, nh, nkv, D, rot, page, pairs8, T
     assert torch.equal(heads[..., rot:], qkv[:, :(nh + nkv) * D].view(T, nh + nkv, D)[..., rot:])
     with pytest.raises(Exception, match="rotate"):
         ops.rope_store(q1, nh, nkv, D, cos, sin, slots, kc[0], vc[0], page, pairs8, rot_dim=D + 2)
+    # q_scale: the q heads (and nothing else) leave multiplied by it, rounded once
+    q3 = qkv.clone()
+    k3, v3 = kc[1].clone(), vc[1].clone()
+    ops.rope_store(q3, nh, nkv, D, cos, sin, slots, k3, v3, page, pairs8, rot_dim=rot, q_scale=0.1275)
+    want = q2.float()
+    q_exact = qkv.float().clone()
+    emu32 = EmulatedOps(torch.float32)
+    emu32.rope_store(q_exact, nh, nkv, D, cos, sin, None, None, None, page, pairs8, rot_dim=rot)
+    want[:, :nh * D] = (q_exact[:, :nh * D] * 0.1275).to(dt).float()
+    assert rel_err(q3[:, :nh * D], want[:, :nh * D]) < ELEM_TOL[dt] * 2
+    assert torch.equal(q3[:, nh * D:], q1[:, nh * D:]) and torch.equal(k3, kc[0]) and torch.equal(v3, vc[0])
 
 
 def test_rotation_plans():
@@ -591,17 +602,32 @@ def make_attention_case(dt, nh, nkv, D, page, seqs, seed=0):
 
 
 ATTN_TOL = {torch.float32: 2e-5, torch.bfloat16: 2 ** -7}
+UNITS = ["scale at the scores", "scores in units of log 2"]
+
+
+def in_units(units, qkv, nh, D, scale):
+    """(qkv, scale) as the attention call takes them.  "scores in units of log 2": the queries are
+    multiplied by scale * log2(e) where they are made (here: before their rounding) and the call
+    gets ln 2, so that scale * log2(e) is 1 for the kernel: the form the engine uses, in which
+    the matrix-core kernels need no multiply-add per score."""
+    if units == UNITS[0]:
+        return qkv, scale
+    out = qkv.clone()
+    out[:, :nh * D] = (qkv[:, :nh * D].float() * (scale * math.log2(math.e))).to(qkv.dtype)
+    return out, math.log(2.0)
+
 
 
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (8, 1, 32, 16), (7, 7, 48, 32),
                                            (28, 4, 128, 16), (6, 2, 256, 64), (5, 5, 80, 16),
                                            (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16)])
 @pytest.mark.parametrize("window", [None, 16, 50])
-def test_paged_attention(both, nh, nkv, D, page, window):
+@pytest.mark.parametrize("units", UNITS)
+def test_paged_attention(both, nh, nkv, D, page, window, units):
     ops, emu, dt = both
     seqs = [(130, 130), (77, 5), (64, 64), (200, 2), (16, 1), (145, 1), (1, 1), (333, 1)]
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs)
-    scale = 1.0 / math.sqrt(D)
+    qkv, scale = in_units(units, qkv, nh, D, 1.0 / math.sqrt(D))
     got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
     ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
                               types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
@@ -615,7 +641,8 @@ def test_paged_attention(both, nh, nkv, D, page, window):
                                            (4, 2, 256, 16)])     # 256: no LDS form; the same calls take the other kernel
 @pytest.mark.parametrize("window", [None, 16, 50])
 @pytest.mark.parametrize("form", ["paired", "unpaired", "shares"])
-def test_prompt_attention_through_lds(nh, nkv, D, page, window, form):
+@pytest.mark.parametrize("units", UNITS)
+def test_prompt_attention_through_lds(nh, nkv, D, page, window, form, units):
     """The prompt kernel whose wavefronts share each block of keys through LDS,
     forced at sizes far below its crossover: portions that end inside a
     workgroup's 128 columns, that start deep in a context, and one-token rows;
@@ -632,7 +659,7 @@ def test_prompt_attention_through_lds(nh, nkv, D, page, window, form):
     if form == "shares":
         ops.PROMPT_SPLIT_MIN_BLOCKS, ops.PROMPT_SPLIT_WORKGROUPS = 1, 1 << 20
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=5)
-    scale = 1.0 / math.sqrt(D)
+    qkv, scale = in_units(units, qkv, nh, D, 1.0 / math.sqrt(D))
     got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
     ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
                               types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
@@ -641,7 +668,8 @@ def test_prompt_attention_through_lds(nh, nkv, D, page, window, form):
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
-def test_attention_reference_point_moves_late():
+@pytest.mark.parametrize("units", UNITS)
+def test_attention_reference_point_moves_late(units):
     """Scores that keep growing along the context, by more than the kernels'
     lazy-rescale margin from block to block: the running reference of every
     column has to move many times, in prompt portions and in split decode."""
@@ -660,17 +688,19 @@ def test_attention_reference_point_moves_late():
         for s, (ctx, _) in enumerate(seqs):
             for r in range(ctx):
                 kc[int(tables[s, r // page]), :, r % page, 0] = r / 2
-        got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, None)
+        qkv, scale = in_units(units, qkv, nh, D, 1.0)
+        got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, None)
         ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
                                   types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
                                                            for k, v in vars(batch).items()}),
-                                  1.0, None)
+                                  scale, None)
         assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (7, 7, 48, 32), (5, 5, 80, 16), (28, 4, 128, 16)])
 @pytest.mark.parametrize("window", [None, 50])
-def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window):
+@pytest.mark.parametrize("units", UNITS)
+def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window, units):
     """Single-token rows only: the general kernel (float32, and bfloat16 head
     sizes the matrix-core kernels refuse) and the matrix-core kernel both split
     every row's keys over several wavefronts and merge the shares; contexts of
@@ -678,7 +708,7 @@ def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window):
     ops, emu, dt = both
     seqs = [(1, 1), (5, 1), (64, 1), (65, 1), (333, 1), (700, 1), (129, 1)]
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=9)
-    scale = 1.0 / math.sqrt(D)
+    qkv, scale = in_units(units, qkv, nh, D, 1.0 / math.sqrt(D))
     got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
     ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
                               types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
@@ -689,7 +719,8 @@ def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window):
 
 @pytest.mark.parametrize("D,page", [(16, 16), (32, 16), (128, 32)])
 @pytest.mark.parametrize("q_len", [1, 5])
-def test_attention_finds_one_key_at_edges(both, D, page, q_len):
+@pytest.mark.parametrize("units", UNITS)
+def test_attention_finds_one_key_at_edges(both, D, page, q_len, units):
     """One key among hundreds carries all the weight (its score stands out by
     construction), placed at a page's last and first slot, at the first and the
     last visible position, and just inside and just outside a window: the
@@ -706,7 +737,8 @@ def test_attention_finds_one_key_at_edges(both, D, page, q_len):
             kc[:, :, :, 0] = 0
             pg, off = int(tables[0, target // page]), target % page
             kc[pg, :, off, 0] = 30.0                   # score 900 for the target, 0 elsewhere
-            got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0, window)
+            qkv, scale = in_units(units, qkv, nh, D, 1.0)
+            got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
             last = got[-1].float().view(nh, D)         # the query at position ctx - 1
             visible = window is None or target > p_last - window
             for h in range(nh):
