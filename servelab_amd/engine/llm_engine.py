@@ -110,9 +110,13 @@ class LLMEngine:
                 rows += [int(n) for n in tune_products]
             library_rows = getattr(model.rt.ops, "library_rows", None)
             if library_rows is not None:
-                first = model.rt.ops.SKINNY_MAX_M + 1
-                rows += sorted({library_rows(n)
-                                for n in range(first, self.scheduler_config.max_num_seqs + 1)})
+                # decode steps of more requests than the few-rows kernels take, and the steps that
+                # carry a newcomer's short prompt beside decoded tokens: below LIBRARY_PADDED_MAX_M
+                # rows they run on a multiple of LIBRARY_ROW_STEP rows, so these few shapes cover them
+                first = int(getattr(model.rt.ops, "graph_rows_limit", model.rt.ops.SKINNY_MAX_M)) + 1
+                top = max(self.scheduler_config.max_num_seqs,
+                          min(model.rt.ops.LIBRARY_PADDED_MAX_M, self.scheduler_config.max_num_batched_tokens))
+                rows += sorted({library_rows(n) for n in range(first, top + 1)})
             self.runner.tune_products(rows)
         self.graphs_captured = 0
         if capture_graphs_up_to:
