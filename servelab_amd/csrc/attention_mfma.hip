@@ -445,10 +445,15 @@ template <int N> __device__ __forceinline__ void wait_loads() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-template <bool FOLD>
-__global__ __launch_bounds__(64 * SHARED_WAVES) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1)))
+// NB: column tiles of 16 a wavefront takes.  Two is the form for launches that fill the chip (a
+// block read from LDS serves 32 columns); one makes twice the workgroups of half the registers,
+// for launches too small to give every SIMD two wavefronts otherwise (a prompt of 2,048 tokens
+// of the 7B shape: 224 workgroups of 128 columns for 256 CUs; MI355X: 88 us with two tiles a
+// wavefront, 77 us with one).
+template <bool FOLD, int NB>
+__global__ __launch_bounds__(64 * SHARED_WAVES) __attribute__((amdgpu_waves_per_eu(D <= 128 ? (NB == 1 ? 3 : 2) : 1)))
 void attention_mfma_shared_kernel(const AttnParams P) {
-  constexpr int NB = 2, COLS = 16 * NB * SHARED_WAVES;
+  constexpr int COLS = 16 * NB * SHARED_WAVES;
   // one array per stage, so that the compiler can tell the loads into one from the reads of another
   __shared__ __attribute__((aligned(1024))) char ring0[STAGE_BYTES];
   __shared__ __attribute__((aligned(1024))) char ring1[STAGE_BYTES];
@@ -668,13 +673,15 @@ extern "C" int sl_attention_mfma_shares_keys() { return SHARED_FITS ? 1 : 0; }
 // [part_row0, part_row0 + part_rows) these sequences own (one token each).
 // Prompt portions go to the workgroups that share keys through LDS once the
 // launch would have shared_min_waves wavefronts of 32 columns or more;
-// pair_tiles: see the kernel.
+// pair_tiles: see the kernel; narrow_below: with fewer workgroups of 128
+// columns than this (but a third of it at least: smaller launches are all
+// latency either way), workgroups of 64 columns are launched instead.
 extern "C" const char* sl_attention_mfma(
     const void* qkv, int row_stride, const void* kc, const void* vc, const int* block_tables,
     int max_pages, const int* cu_q, const int* positions, int seq_begin, int num_seqs,
     int max_q_len, int nh, int nkv, int head_dim, int page, float scale, int window, int nsplit,
     int shared_min_waves, int pair_tiles, void* out, float* part_o, float* part_ml, int part_row0, int part_rows,
-    hipStream_t stream) {
+    int narrow_below, hipStream_t stream) {
   SL_CHECK(head_dim == D, "attention_mfma: built for another head size");
   SL_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: heads must be a multiple of kv heads");
   SL_CHECK(page == 16 || page == 32 || page == 64, "attention_mfma: page size must be 16, 32 or 64");
@@ -735,10 +742,19 @@ extern "C" const char* sl_attention_mfma(
     if (fold) attention_mfma_kernel<2, false, true><<<grid, 64, 0, stream>>>(P);
     else attention_mfma_kernel<2, false, false><<<grid, 64, 0, stream>>>(P);
   } else {
-    const long long wg = (tiles + SHARED_WAVES - 1) / SHARED_WAVES;
+    // workgroups of 128 columns, or of 64 when those would leave SIMDs with one wavefront
+    long long wg = (cols + 32 * SHARED_WAVES - 1) / (32 * SHARED_WAVES);
+    const long long wide = (pair_tiles ? (wg + 1) / 2 : wg) * nkv * num_seqs;
+    const bool narrow = nsplit == 1 && wide < narrow_below && wide >= narrow_below / 3;
+    if (narrow) wg = (cols + 16 * SHARED_WAVES - 1) / (16 * SHARED_WAVES);
     const dim3 grid((unsigned)(pair_tiles ? (wg + 1) / 2 : wg * nsplit), nkv, num_seqs);
-    if (fold) attention_mfma_shared_kernel<true><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
-    else attention_mfma_shared_kernel<false><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
+    if (narrow) {
+      if (fold) attention_mfma_shared_kernel<true, 1><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
+      else attention_mfma_shared_kernel<false, 1><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
+    } else {
+      if (fold) attention_mfma_shared_kernel<true, 2><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
+      else attention_mfma_shared_kernel<false, 2><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
+    }
     if (nsplit > 1) {
       const char* e = sl_launch_status();
       if (e) return e;

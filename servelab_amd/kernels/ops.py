@@ -844,6 +844,9 @@ class HipOps:
     PROMPT_SPLIT_MIN_BLOCKS = 64
     PROMPT_SPLIT_MAX = 8
     PROMPT_SPLIT_BYTES = 512 << 20   # ... and no more shares than keep the partial outputs below this
+    # ... and a launch of fewer workgroups of 128 columns than this takes workgroups of 64 columns (a
+    # wavefront then holds 16 columns and half the registers: three wavefronts fit a SIMD)
+    NARROW_ATTENTION_WORKGROUPS = 400
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples
@@ -899,7 +902,7 @@ class HipOps:
                 part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
                        0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
-                       n_pre_tok if nsplit > 1 else 0)
+                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
@@ -910,7 +913,7 @@ class HipOps:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, 0, _p(out),
-                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0)
+                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0, 0)
 
     # ------------------------------------------------------------- sampling
     SAMPLE_SLICE = 2048           # logits per workgroup of the two-stage argmax and draw (at most 64 slices)
