@@ -422,10 +422,9 @@ constexpr int SHARED_WAVES = 4;
 constexpr int KU = D / 8;                          // 16-byte units in a row of K
 constexpr int STAGE_UNITS = 8 * D;                 // K: 32 rows x KU, then V^T: D rows x 4
 constexpr int STAGE_BYTES = 16 * STAGE_UNITS;
-constexpr int STAGES = 3 * STAGE_BYTES <= 65536 ? 3 : 2;
 constexpr int CHUNKS = STAGE_UNITS / 64;           // wavefront-wide loads a block: D / 8, half of them K
 constexpr int LOADS = CHUNKS / SHARED_WAVES;       // ... per wavefront: D / 32
-constexpr bool SHARED_FITS = STAGES * STAGE_BYTES <= 65536;
+constexpr bool SHARED_FITS = 2 * STAGE_BYTES <= 65536;
 struct Stage0 { static constexpr int value = 0; };
 struct Stage1 { static constexpr int value = 1; };
 struct Stage2 { static constexpr int value = 2; };
@@ -454,10 +453,16 @@ template <bool FOLD, int NB>
 __global__ __launch_bounds__(64 * SHARED_WAVES) __attribute__((amdgpu_waves_per_eu(D <= 128 ? (NB == 1 ? 3 : 2) : 1)))
 void attention_mfma_shared_kernel(const AttnParams P) {
   constexpr int COLS = 16 * NB * SHARED_WAVES;
+  // A stage of the ring holds SUB blocks of 32 keys, which a pass of the loop computes between
+  // two barriers.  The wide form (two column tiles a wavefront) takes two blocks a pass where
+  // two such stages fit the 64 KB (one barrier per 64 keys: 3-4 % at 4,096 tokens and beyond);
+  // the narrow form one block a pass and three stages, which leaves LDS for three workgroups.
+  constexpr int SUB = NB == 2 && 4 * STAGE_BYTES <= 65536 ? 2 : 1;
+  constexpr int STAGES = SUB == 2 ? 2 : 3 * STAGE_BYTES <= 65536 ? 3 : 2;
   // one array per stage, so that the compiler can tell the loads into one from the reads of another
-  __shared__ __attribute__((aligned(1024))) char ring0[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) char ring1[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) char ring2[STAGES == 3 ? STAGE_BYTES : 16];
+  __shared__ __attribute__((aligned(1024))) char ring0[SUB * STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char ring1[SUB * STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) char ring2[STAGES == 3 ? SUB * STAGE_BYTES : 16];
   // (wave as a scalar: the products below sit under conditions that depend on it, and matrix
   // instructions ignore the execution mask)
   const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63, n = lane & 15, gq = lane >> 4;
@@ -504,26 +509,35 @@ void attention_mfma_shared_kernel(const AttnParams P) {
     constexpr int S = decltype(stage)::value;
     return S == 0 ? ring0 : S == 1 ? ring1 : ring2;
   };
-  int pg[2];
-  auto load_pages = [&](int kb) {
-    const int kbase = kb * 32;
-    pg[0] = table[kbase >> page_shift];
-    pg[1] = table[(kbase + 16) >> page_shift];
-  };
-  // ask for block kb into a stage (its page ids are in pg)
-  auto fetch = [&](int kb, auto stage) {
-    const int within = (kb * 32) & (page - 1);       // where the block starts inside its page (64-key pages: 0 or 32)
-    const __bf16* k0 = P.kc + ((size_t)pg[0] * per_page + head_at + (size_t)within * D);
-    const __bf16* k1 = P.kc + ((size_t)pg[1] * per_page + head_at + (size_t)within * D);
-    const __bf16* v0 = P.vc + ((size_t)pg[0] * per_page + head_at + within);
-    const __bf16* v1 = P.vc + ((size_t)pg[1] * per_page + head_at + within);
-    const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)ring(stage);
+  // A pass of the loop computes SUB blocks of 32 keys out of one stage, with one barrier.  The
+  // page ids of a pass are read (scalar loads) a pass before its blocks are asked for.
+  int pg[SUB][2];
+  auto load_pages = [&](int kb, int last) {
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const int chunk = wave + SHARED_WAVES * i;
-      const bool keys = chunk < CHUNKS / 2;            // the same for the whole wavefront
-      const __bf16* from = (second[i] ? (keys ? k1 : v1) : (keys ? k0 : v0)) + src[i];
-      load_to_lds(from, base + 1024 * chunk);
+    for (int sub = 0; sub < SUB; ++sub) {
+      const int kbase = (kb + sub < last ? kb + sub : last) * 32;
+      pg[sub][0] = table[kbase >> page_shift];
+      pg[sub][1] = table[(kbase + 16) >> page_shift];
+    }
+  };
+  // ask for the blocks kb .. kb + SUB - 1 below `end` into a stage (their page ids are in pg)
+  auto fetch = [&](int kb, int end, auto stage) {
+#pragma unroll
+    for (int sub = 0; sub < SUB; ++sub) {
+      if (kb + sub >= end) break;                    // (the same for the whole workgroup)
+      const int within = ((kb + sub) * 32) & (page - 1);   // where the block starts inside its page (64-key pages: 0 or 32)
+      const __bf16* k0 = P.kc + ((size_t)pg[sub][0] * per_page + head_at + (size_t)within * D);
+      const __bf16* k1 = P.kc + ((size_t)pg[sub][1] * per_page + head_at + (size_t)within * D);
+      const __bf16* v0 = P.vc + ((size_t)pg[sub][0] * per_page + head_at + within);
+      const __bf16* v1 = P.vc + ((size_t)pg[sub][1] * per_page + head_at + within);
+      const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) char*)ring(stage) + STAGE_BYTES * sub;
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i) {
+        const int chunk = wave + SHARED_WAVES * i;
+        const bool keys = chunk < CHUNKS / 2;          // the same for the whole wavefront
+        const __bf16* from = (second[i] ? (keys ? k1 : v1) : (keys ? k0 : v0)) + src[i];
+        load_to_lds(from, base + 1024 * chunk);
+      }
     }
   };
 
@@ -563,43 +577,49 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   }
   const int last = wg_end - 1;
 
-  // one block: ask for block kb + STAGES - 1 (into the stage that block kb - 1 was read from; the
-  // barrier that ended that block has passed), compute block kb out of `here`, then make sure
-  // that this wavefront's loads of block kb + 1 have landed and meet the others
+  // one pass: ask for the pass STAGES - 1 ahead (into the stage that the last pass was read from;
+  // the barrier that ended that pass has been passed), compute this pass's blocks out of `here`,
+  // then make sure that this wavefront's loads of the next pass have landed and meet the others
   auto step = [&](int kb, auto here, auto ahead) {
-    const bool more = kb + STAGES - 1 < wg_end;
+    const int next = kb + (STAGES - 1) * SUB;
+    const bool more = next < wg_end;
     if (more) {
-      fetch(kb + STAGES - 1, ahead);
-      load_pages(kb + STAGES < last ? kb + STAGES : last);
+      fetch(next, wg_end, ahead);
+      load_pages(next + SUB, last);
     }
-    if (active && kb >= C.kb_begin && kb < C.kb_end) {
-      const char* at = ring(here);
-      bf16x8 kf[2][KK], vf[DD];
+    const char* at = ring(here);
 #pragma unroll
-      for (int m = 0; m < 2; ++m)
+    for (int sub = 0; sub < SUB; ++sub) {
+      const int k = kb + sub;
+      if (active && k < wg_end && k >= C.kb_begin && k < C.kb_end) {
+        const char* from = at + STAGE_BYTES * sub;
+        bf16x8 kf[2][KK], vf[DD];
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) kf[m][kk] = *(const bf16x8*)(at + 256 * KU * m + k_at[kk]);
+        for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)(at + v_at + 1024 * dd);
-      C.block_abreast(kb, kf, vf, gq);
+          for (int kk = 0; kk < KK; ++kk) kf[m][kk] = *(const bf16x8*)(from + 256 * KU * m + k_at[kk]);
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)(from + v_at + 1024 * dd);
+        C.block_abreast(k, kf, vf, gq);
+      }
     }
-    if (more && STAGES == 3) wait_loads<LOADS>();    // all but the block just asked for
+    if (more && STAGES == 3) wait_loads<LOADS * SUB>();    // all but the pass just asked for
     else wait_loads<0>();
-    // (the bare barrier: __syncthreads() would first wait for every load on its way, the block
-    // just asked for included; what must be complete here is this wavefront's share of block
-    // kb + 1, waited for above, and its reads of block kb, whose values the products have used)
+    // (the bare barrier: __syncthreads() would first wait for every load on its way, the pass
+    // just asked for included; what must be complete here is this wavefront's share of the next
+    // pass, waited for above, and its reads of this pass, whose values the products have used)
     __builtin_amdgcn_s_barrier();
     asm volatile("" : : : "memory");               // (the compiler reads LDS again from here on, whatever it held)
   };
 
   if (wg_begin < wg_end) {                           // (a share may be empty; the same for the whole workgroup)
-    load_pages(wg_begin);
-    fetch(wg_begin, Stage0{});
-    load_pages(wg_begin + 1 < last ? wg_begin + 1 : last);
+    load_pages(wg_begin, last);
+    fetch(wg_begin, wg_end, Stage0{});
+    load_pages(wg_begin + SUB, last);
     if (STAGES == 3) {
-      if (wg_begin + 1 < wg_end) fetch(wg_begin + 1, Stage1{});
-      load_pages(wg_begin + 2 < last ? wg_begin + 2 : last);
-      if (wg_begin + 1 < wg_end) wait_loads<LOADS>();
+      if (wg_begin + SUB < wg_end) fetch(wg_begin + SUB, wg_end, Stage1{});
+      load_pages(wg_begin + 2 * SUB, last);
+      if (wg_begin + SUB < wg_end) wait_loads<LOADS * SUB>();
       else wait_loads<0>();
     } else {
       wait_loads<0>();
@@ -608,15 +628,15 @@ void attention_mfma_shared_kernel(const AttnParams P) {
     asm volatile("" : : : "memory");
   }
   if (STAGES == 3) {
-    for (int kb = wg_begin; kb < wg_end; kb += 3) {
+    for (int kb = wg_begin; kb < wg_end; kb += 3 * SUB) {
       step(kb, Stage0{}, Stage2{});
-      if (kb + 1 < wg_end) step(kb + 1, Stage1{}, Stage0{});
-      if (kb + 2 < wg_end) step(kb + 2, Stage2{}, Stage1{});
+      if (kb + SUB < wg_end) step(kb + SUB, Stage1{}, Stage0{});
+      if (kb + 2 * SUB < wg_end) step(kb + 2 * SUB, Stage2{}, Stage1{});
     }
   } else {
-    for (int kb = wg_begin; kb < wg_end; kb += 2) {
+    for (int kb = wg_begin; kb < wg_end; kb += 2 * SUB) {
       step(kb, Stage0{}, Stage1{});
-      if (kb + 1 < wg_end) step(kb + 1, Stage1{}, Stage0{});
+      if (kb + SUB < wg_end) step(kb + SUB, Stage1{}, Stage0{});
     }
   }
   if (active) {
