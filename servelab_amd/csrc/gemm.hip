@@ -324,6 +324,13 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
+// Eight weights that this kernel reads once and nobody reads again before the caches have
+// turned over: loaded with the streaming hint, so that they do not push x and the partial
+// results out of the caches (MI355X, 1 GiB read once: 7.0 TB/s with the hint, 6.3 without).
+__device__ __forceinline__ bf16x8 stream_load(const __bf16* p) {
+  return __builtin_nontemporal_load((const bf16x8*)p);
+}
+
 //
 // GATED: the 16 rows of a tile are 8 gate rows followed by the 8 up rows of the
 // same channels; the workgroup then writes silu(gate) * up, 8 columns of an
@@ -435,7 +442,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)(ks + u));
+      for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const bf16x8 bv = *(const bf16x8*)(xp + 32 * (size_t)(ks + u));
@@ -452,7 +459,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(
     for (int u = 0; u < U - 1; ++u)
       if (ks + u < ks1) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)(ks + u));
+        for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
         bv[u] = *(const bf16x8*)(xp + 32 * (size_t)(ks + u));
       }
 #pragma unroll
@@ -686,7 +693,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(
     for (int u = 0; u < U; ++u) {
       const size_t ks = (size_t)(ks0 + g * U + u);
 #pragma unroll
-      for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * ks);
+      for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * ks);
 #pragma unroll
       for (int b = 0; b < MB; ++b) bv[b][u] = *(const bf16x8*)(xp[b] + 32 * ks);
     }
@@ -706,7 +713,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(
 #pragma unroll
       for (int u = 0; u < U; ++u) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)(ks + u));
+        for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
 #pragma unroll
         for (int b = 0; b < MB; ++b) bv[b][u] = *(const bf16x8*)(xp[b] + 32 * (size_t)(ks + u));
       }
@@ -737,7 +744,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(
     for (int b = 0; b < MB; ++b) bv[b] = *(const bf16x8*)(xp[b] + 32 * (size_t)ks);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const bf16x8 a = *(const bf16x8*)(wp[t] + 512 * (size_t)ks);
+      const bf16x8 a = stream_load(wp[t] + 512 * (size_t)ks);
 #pragma unroll
       for (int b = 0; b < MB; ++b)
         acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bv[b], acc[t][b], 0, 0, 0);
@@ -883,7 +890,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
       int ks = kbeg + c * KC + u;
       if (ks >= kend) ks = kend - 1;               // its x is zero
 #pragma unroll
-      for (int t = 0; t < NT; ++t) a[t][u] = *(const bf16x8*)(wp[t] + 512 * (size_t)ks);
+      for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)ks);
     }
   };
   f32x4 acc[NT][MB];
