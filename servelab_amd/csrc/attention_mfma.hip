@@ -366,12 +366,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 25
       const int p = ko < 16 ? pg[0] : pg[1];
       const __bf16* kr = P.kc + (((size_t)p * P.nkv + kvh) * page + ((kbase + ko) & (page - 1))) * D + 8 * gq;
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) kf[m][kk] = *(const bf16x8*)(kr + 32 * kk);
+      for (int kk = 0; kk < KK; ++kk) kf[m][kk] = __builtin_nontemporal_load((const bf16x8*)(kr + 32 * kk));
     }
     const int p = gq < 2 ? pg[0] : pg[1];
     const __bf16* vr = P.vc + ((size_t)p * P.nkv + kvh) * D * page + ((kbase + 8 * gq) & (page - 1));
 #pragma unroll
-    for (int dd = 0; dd < DD; ++dd) vf[dd] = *(const bf16x8*)(vr + (size_t)(16 * dd + n) * page);
+    for (int dd = 0; dd < DD; ++dd) vf[dd] = __builtin_nontemporal_load((const bf16x8*)(vr + (size_t)(16 * dd + n) * page));
   };
 
   // Two wavefronts share a SIMD where the registers allow it: one computes
