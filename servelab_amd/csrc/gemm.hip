@@ -7,6 +7,7 @@
 //                 rows of x at a time.
 //   sl_gemm_tiled any M: 64x64 LDS tiles, 4x4 outputs per thread.
 #include "common.h"
+#include <type_traits>
 
 #if defined(SL_F32)
 #define SL_VEC 4
@@ -637,6 +638,184 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
   else if (consumer) gemm_skinny_kernel<false, true, false, 16><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F);
   else if (gated) gemm_skinny_kernel<true, false, false, 1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F);
   else gemm_skinny_kernel<false, false, false, 1><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32, F);
+  return sl_launch_status();
+}
+
+// ------------------------------- few rows, x resident, tile after tile
+// The consumer products with many tiles (gate/up, the head).  The kernel above
+// starts a workgroup per tile, and each one begins by asking for its share of
+// the sums of squares and for x (with 8 rows a third of the bytes it pulls
+// through L1) before its weights stream.  Here a workgroup stays: grid =
+// what the chip holds at once, tiles blockIdx.x, blockIdx.x + grid, ...  A
+// wavefront keeps its share of K throughout (NS k-steps, the same for all
+// eight: K = 256 NS), so its part of x sits in registers, the row scales are
+// computed once, and the loads of the next tile's weights are issued as this
+// tile's are used up (a ring of R k-steps per wavefront), so they are in flight
+// during the reduction and the epilogue.  NS is a template argument: the loop is
+// straight-line code whose every wait the compiler can count (with a run-time
+// number of steps it waited for all loads at every step).  Result as
+// gemm_skinny_kernel's CONSUMER forms, bit for bit: the same products in the same
+// order.
+template <bool GATED, int PARTS, int NS, int R>
+__global__ __launch_bounds__(512) void gemm_resident_kernel(
+    const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
+    void* __restrict__ y, int M, int N, int out_f32, const NormFusion F) {
+  constexpr int WAVES = 8, KT = WAVES * NS, K = 32 * KT;
+  static_assert(NS % R == 0, "the ring divides the steps");
+  __shared__ f32x4 red[2][WAVES][64];
+  __shared__ float wsum[WAVES][16];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);     // (a scalar: see gemm_skinny_kernel)
+  const int lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
+  const int ntiles = (N + 15) / 16;
+  const int ks0 = NS * wave;
+  int xrow = i < M ? i : M - 1;
+  if (F.rows != nullptr) xrow = F.rows[xrow];
+  const __bf16* xp = x + (size_t)xrow * K + 32 * (size_t)ks0 + 8 * gq;
+  const __bf16* wbase = wt + ((size_t)ks0 * 64 + lane) * 8;
+  constexpr size_t tile_stride = (size_t)KT * 512;
+  bf16x8 a[R];
+  int tile = blockIdx.x;                           // < ntiles: the grid is no larger
+#pragma unroll
+  for (int u = 0; u < R; ++u) a[u] = stream_load(wbase + tile * tile_stride + 512 * u);
+  float pv[PARTS];
+#pragma unroll
+  for (int j = 0; j < PARTS; ++j) {
+    const int p = threadIdx.x / 16 + 32 * j;
+    pv[j] = p < F.in_nparts ? F.in_parts[p * 16 + i] : 0.f;
+  }
+  bf16x8 xr[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) xr[s] = *(const bf16x8*)(xp + 32 * s);
+  {
+    float sacc = 0.f;
+#pragma unroll
+    for (int j = 0; j < PARTS; ++j) sacc += pv[j];
+    sacc += __shfl_xor(sacc, 16, 64);
+    sacc += __shfl_xor(sacc, 32, 64);
+    if (lane < 16) wsum[wave][lane] = sacc;
+  }
+  __syncthreads();
+  // the epilogue row of this thread and its scale
+  const int em = GATED ? threadIdx.x / 8 : threadIdx.x / 16;
+  float inv = 0.f;
+  if (em < M) {
+    const int tok = F.rows != nullptr ? F.rows[em] : em;
+    float ss = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) ss += wsum[wv][tok];
+    inv = rsqrtf(ss / (float)K + F.eps);
+  }
+  // one tile: its products, the refills of the ring, the reduction and the epilogue
+  auto one_tile = [&](auto has_next, int buf) {
+    const __bf16* wcur = wbase + tile * tile_stride;
+    const __bf16* wnext = wcur + gridDim.x * tile_stride;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s % R], xr[s], acc, 0, 0, 0);
+      if (s + R < NS) a[s % R] = stream_load(wcur + 512 * (s + R));
+      else if (decltype(has_next)::value) a[s % R] = stream_load(wnext + 512 * (s + R - NS));
+    }
+    red[buf][wave][lane] = acc;
+    __syncthreads();
+    // lane (m + 16 (n_local / 4)) holds y[m, n_local] in element n_local % 4
+    if (GATED) {
+      if (threadIdx.x < 128) {
+        const int m = em, j = threadIdx.x % 8;
+        const int col = tile * 8 + j;
+        if (m < M && col < N / 2) {
+          float gsum = 0.f, usum = 0.f;
+#pragma unroll
+          for (int wv = 0; wv < WAVES; ++wv) {
+            gsum += red[buf][wv][m + 16 * (j / 4)][j % 4];
+            usum += red[buf][wv][m + 16 * (2 + j / 4)][j % 4];
+          }
+          gsum *= inv;
+          usum *= inv;
+          ((__bf16*)y)[(size_t)m * (N / 2) + col] = (__bf16)(gsum / (1.f + expf(-gsum)) * usum);
+        }
+      }
+    } else if (threadIdx.x < 256) {
+      const int m = em, n_local = threadIdx.x % 16, col = tile * 16 + n_local;
+      if (m < M && col < N) {
+        float sum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; ++wv) sum += red[buf][wv][m + 16 * (n_local / 4)][n_local % 4];
+        sum *= inv;
+        if (bias != nullptr) sum += bias[col];
+        if (out_f32) ((float*)y)[(size_t)m * N + col] = sum;
+        else ((__bf16*)y)[(size_t)m * N + col] = (__bf16)sum;
+      }
+    }
+  };
+  int buf = 0;
+  for (; tile + (int)gridDim.x < ntiles; tile += gridDim.x, buf ^= 1) one_tile(std::true_type{}, buf);
+  one_tile(std::false_type{}, buf);
+}
+
+// How many workgroups of 512 threads of a kernel the current device holds at once.
+template <typename Kernel>
+static int resident_workgroups(Kernel kernel) {
+  int dev = 0, cus = 0, per_cu = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 512, 0) != hipSuccess) return 0;
+  return cus * per_cu;
+}
+
+// Whether sl_gemm_resident has a kernel for rows of K values (K = 256 * steps for one of
+// the step counts it is built for).
+extern "C" int sl_gemm_resident_takes(int K) {
+  switch (K) {
+    case 256 * 6: case 256 * 8: case 256 * 14: case 256 * 16: case 256 * 20: return 1;
+    default: return 0;
+  }
+}
+
+// The consumer forms of sl_gemm_skinny (x: un-normalised rows) for matrices of
+// many tiles; same arguments, same result.
+extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const float* bias, void* y,
+                                        int M, int N, int K, int out_f32, int gated,
+                                        const float* in_parts, int in_nparts, float eps,
+                                        const int* rows, hipStream_t stream) {
+  SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_resident: sizes must be positive");
+  SL_CHECK(M <= 16, "gemm_resident: at most 16 rows");
+  SL_CHECK(sl_gemm_resident_takes(K), "gemm_resident: no kernel for rows of this length");
+  SL_CHECK(!gated || (N % 16 == 0 && bias == nullptr && !out_f32),
+           "gemm_resident: the gated form needs N % 16 == 0, no bias, activation output");
+  SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
+           "gemm_resident: x and W must be 16-byte aligned");
+  SL_CHECK(in_parts != nullptr && in_nparts > 0 && eps > 0.f, "gemm_resident: needs parts and eps");
+  SL_CHECK(in_nparts <= 32 * SL_MAX_PARTS_PER_THREAD, "gemm_resident: un-normalised rows of more than 8192 values");
+  if (M == 0) return nullptr;
+  const int ntiles = (N + 15) / 16;
+  const NormFusion F{in_parts, in_nparts, eps, rows, nullptr, nullptr, nullptr};
+  const __bf16* xx = (const __bf16*)x;
+  const __bf16* ww = (const __bf16*)wt;
+#define SL_RESIDENT(G, NS, R)                                                                   \
+  do {                                                                                          \
+    constexpr int PARTS = NS <= 16 ? 8 : 16;          /* K / 16 parts, 32 per pass */           \
+    static int slots = 0;                                                                       \
+    if (slots == 0) slots = resident_workgroups(gemm_resident_kernel<G, PARTS, NS, R>);         \
+    SL_CHECK(slots > 0, "gemm_resident: the device holds no workgroup of this kernel");         \
+    const int rounds = (ntiles + slots - 1) / slots;                                            \
+    const int grid = (ntiles + rounds - 1) / rounds;                                            \
+    gemm_resident_kernel<G, PARTS, NS, R><<<grid, 512, 0, stream>>>(xx, ww, bias, y, M, N,      \
+                                                                   out_f32, F);                 \
+  } while (0)
+#define SL_RESIDENT_CASE(NS, R)                                     \
+  case 256 * NS:                                                    \
+    if (gated) SL_RESIDENT(true, NS, R); else SL_RESIDENT(false, NS, R); \
+    break
+  switch (K) {
+    SL_RESIDENT_CASE(6, 6);
+    SL_RESIDENT_CASE(8, 8);
+    SL_RESIDENT_CASE(14, 14);
+    SL_RESIDENT_CASE(16, 16);
+    SL_RESIDENT_CASE(20, 10);
+  }
+#undef SL_RESIDENT_CASE
+#undef SL_RESIDENT
   return sl_launch_status();
 }
 

@@ -141,6 +141,7 @@ class HipOps:
         self._fn = {}
         self.use_mfma_attention = True
         self._num_cus = max(1, torch.cuda.get_device_properties(self.device).multi_processor_count)
+        self._resident_k = {}
         self.fuse_norms = act_dtype == torch.bfloat16
         self.fuse_rope = act_dtype == torch.bfloat16
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
@@ -473,8 +474,26 @@ class HipOps:
         if bias is not None:
             self._check(bias, torch.float32, (N,), "bias")
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
-        self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs)
+        if self._takes_resident(N, K):
+            self._call("gemm", "sl_gemm_resident", _p(xs.x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
+                       int(out_f32), int(gated), _p(xs.parts), xs.parts.shape[0], _c_float(xs.eps),
+                       _p(xs.rows))
+        else:
+            self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs)
         return y
+
+    RESIDENT_MIN_ROUNDS = 3       # tiles per CU from which workgroups that stay beat one per tile
+
+    def _takes_resident(self, N, K) -> bool:
+        """Whether a consumer product runs on the workgroups that stay and walk the tiles
+        (x in registers, row scales computed once): matrices with several tiles per CU whose
+        row length the kernel is built for."""
+        if -(-N // 16) < self.RESIDENT_MIN_ROUNDS * self._num_cus:
+            return False
+        takes = self._resident_k.get(K)
+        if takes is None:
+            takes = self._resident_k[K] = bool(self._lib["gemm"].sl_gemm_resident_takes(K))
+        return takes
 
     GATE_BLOCK = 8                # gate and up rows alternate in blocks of 8 (half an MFMA tile)
 

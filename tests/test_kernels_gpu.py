@@ -340,6 +340,42 @@ def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs):
     assert torch.is_tensor(ops.linear(big, w1, None, defer=True))
 
 
+@pytest.mark.parametrize("M,H,N2", [(1, 1536, 96), (8, 3584, 4608), (16, 5120, 1008), (5, 2048, 1000),
+                                    (7, 2048, 17600), (16, 4096, 18000), (3, 5120, 16), (8, 3584, 20000)])
+def test_consumer_products_on_workgroups_that_stay(M, H, N2):
+    """The products that read un-normalised rows, on workgroups that keep x in registers and walk
+    the tiles (several rounds where the matrix has more tiles than the chip holds workgroups):
+    the very numbers of the kernel with a workgroup per tile, which the test above holds to the
+    unfused sequence.  Row lengths the kernel is not built for are refused."""
+    from servelab_amd.kernels import HipOps, KernelError
+    from servelab_amd.kernels.ops import ScaledRows
+    ops = HipOps(torch.bfloat16, "cuda:0")
+    assert ops._takes_resident(1 << 20, H) and not ops._takes_resident(1 << 20, H + 32)
+    assert not ops._takes_resident(16 * ops._num_cus, H)
+    x = randn(M, H, dtype=torch.bfloat16, seed=1)
+    parts = randn(-(-H // 16), 16, seed=2).abs().contiguous()
+    w2 = ops.prepare_weight(randn(N2, H, dtype=torch.bfloat16, scale=0.05, seed=5))
+    b2 = randn(N2, seed=6)
+    rows = torch.tensor([M - 1, 0, M // 2][:min(3, M)], dtype=torch.int32).cuda()
+    cases = [(ScaledRows(x, parts, 1e-5), b2, False), (ScaledRows(x, parts, 1e-5), None, True),
+             (ScaledRows(x, parts, 1e-5, rows), None, True)]
+    got = {}
+    for stay in (False, True):
+        ops._takes_resident = lambda N, K, stay=stay: stay
+        got[stay] = [ops.linear(xs, w2, b, out_f32=f32) for xs, b, f32 in cases]
+        if N2 % 16 == 0:
+            got[stay].append(ops.gated_linear(ScaledRows(x, parts, 1e-5), w2, 8))
+    for a, b in zip(got[False], got[True]):
+        assert a.shape == b.shape and torch.equal(a, b)
+    # and against the formula
+    inv = torch.rsqrt(parts.sum(0)[:M] / H + 1e-5)
+    ref = (x.float() @ w2.w.float().T) * inv[:, None] + b2
+    assert rel_err(got[True][0], ref) < 2 ** -6
+    odd = ScaledRows(randn(M, H + 32, dtype=torch.bfloat16, seed=1), randn(-(-(H + 32) // 16), 16, seed=2).abs(), 1e-5)
+    with pytest.raises(KernelError, match="no kernel for rows of this length"):
+        ops.linear(odd, ops.prepare_weight(randn(32, H + 32, dtype=torch.bfloat16, seed=3)), None)
+
+
 def test_rope_tables(both):
     ops, emu, dt = both
     D, theta = 48, 1e6
