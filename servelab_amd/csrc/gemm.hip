@@ -435,6 +435,28 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
       g_next[t] = F.next_w[en];
     }
   }
+  // (ROPE: the bias, the angle's cosine and sine and the cache row of this thread's element)
+  float b_pre[NT], c_pre[NT], s_pre[NT];
+  int slot_pre = 0;
+  if (ROPE) {
+    if (threadIdx.x < 256 && em < M && R.slots != nullptr) slot_pre = R.slots[em];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int en = (blockIdx.x * NT + t) * 16 + threadIdx.x % 16;
+      b_pre[t] = 0.f;
+      c_pre[t] = 1.f;
+      s_pre[t] = 0.f;
+      if (threadIdx.x < 256 && em < M && en < N) {
+        if (bias != nullptr) b_pre[t] = bias[en];
+        const int hd = en / R.D, p = en % R.D;
+        if (R.cosv != nullptr && hd < R.nh + R.nkv && p < R.rot) {
+          const int j = 8 * (p / 16) + p % 8, half = R.rot / 2;
+          c_pre[t] = R.cosv[(size_t)em * half + j];
+          s_pre[t] = R.sinv[(size_t)em * half + j];
+        }
+      }
+    }
+  }
   f32x4 acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -524,30 +546,27 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
 #pragma unroll
       for (int wv = 0; wv < WAVES; ++wv) s += red[t][wv][m + 16 * (n_local / 4)][n_local % 4];
       if (CONSUMER && live) s *= inv_of(m);
-      if (live && bias != nullptr) s += bias[n];
       if (ROPE) {
+        s += b_pre[t];
         const float partner = __shfl_xor(s, 8, 64);      // the other half of the pair, same row
         if (!live) continue;
         const int hd = n / R.D, p = n % R.D;
+        const int slot = slot_pre;
         if (hd < R.nh + R.nkv) {
           float val = s;
-          if (R.cosv != nullptr && p < R.rot) {
-            const int j = 8 * (p / 16) + p % 8, half = R.rot / 2;
-            const float c = R.cosv[(size_t)m * half + j], sn = R.sinv[(size_t)m * half + j];
-            val = p % 16 < 8 ? s * c - partner * sn : s * c + partner * sn;
-          }
+          if (R.cosv != nullptr && p < R.rot)
+            val = p % 16 < 8 ? s * c_pre[t] - partner * s_pre[t] : s * c_pre[t] + partner * s_pre[t];
           if (hd < R.nh) {
             ((__bf16*)y)[(size_t)m * N + n] = (__bf16)(val * R.qscale);
           } else if (R.slots != nullptr) {
-            const int slot = R.slots[m];
             R.kc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh)) * R.page + slot % R.page) * R.D + p] = (__bf16)val;
           }
         } else if (R.slots != nullptr) {
-          const int slot = R.slots[m];
           R.vc[(((size_t)(slot / R.page) * R.nkv + (hd - R.nh - R.nkv)) * R.D + p) * R.page + slot % R.page] = (__bf16)s;
         }
         continue;
       }
+      if (live && bias != nullptr) s += bias[n];
       if (PRODUCER) {
         float sq = 0.f;
         if (live) {
