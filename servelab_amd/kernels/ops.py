@@ -183,7 +183,7 @@ class HipOps:
         """Whether a few-rows product gives its workgroups two tiles of W (16
         rows each) instead of one.  Two tiles share one pass over x; these
         kernels are bound by what the busiest CU has to pull through its L1
-        (about 37 GB/s a CU on MI355X, W and the re-read x alike) unless HBM
+        (45-50 GB/s a CU at most on MI355X, W and the re-read x alike) unless HBM
         is slower still, so the choice goes by the workgroups the busiest CU
         gets times the bytes of one.  Up to 8 rows x is small enough that the
         two forms measured within a few per cent of each other on the 7B, 32B
