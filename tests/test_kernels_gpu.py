@@ -517,7 +517,9 @@ def test_rope_store_from_partial_sums(both, nh, nkv, D, page):
 @pytest.mark.parametrize("M", [1, 8, 16, 40])
 @pytest.mark.parametrize("nh,nkv,D,page,H,rot", [(4, 2, 16, 16, 64, 16), (28, 4, 128, 16, 256, 128),
                                                  (5, 1, 48, 32, 96, 48), (5, 1, 48, 32, 96, 16),
-                                                 (6, 2, 64, 16, 128, 32)])
+                                                 (6, 2, 64, 16, 128, 32),
+                                                 # the 7B shape's own (more tiles than CUs) and an uneven split of K
+                                                 (28, 4, 128, 16, 3584, 128), (40, 8, 128, 64, 2144, 64)])
 @pytest.mark.parametrize("pairs", [False, True])
 def test_qkv_rope_store(M, nh, nkv, D, page, H, rot, pairs):
     """Product + rotation + cache write: the one fused kernel (at most 16 rows)
@@ -532,7 +534,7 @@ def test_qkv_rope_store(M, nh, nkv, D, page, H, rot, pairs):
         ops._pair_tiles = lambda M, N, K: True
     N = (nh + 2 * nkv) * D
     x = randn(M, H, dtype=dt, seed=1)
-    w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.1, seed=2))
+    w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.1 * min(1.0, (256 / H) ** 0.5), seed=2))
     bias = randn(N, scale=0.1, seed=3)
     inv = (1.0 / 10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot)).cuda()
     cos, sin = emu.rope_tables(torch.arange(7, 7 + M, dtype=torch.int32).cuda(), inv)
