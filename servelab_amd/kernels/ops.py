@@ -21,6 +21,7 @@ from typing import Optional
 import torch
 
 from . import build
+from .tuning import Tuning
 
 _c_int, _c_float, _c_void_p = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 
@@ -120,15 +121,19 @@ class HipOps:
     #   "rows"   row-major only: decode uses the slower row-major kernels.
     # ``plan_weights(total_bytes)`` picks "dual" while two copies stay below
     # DUAL_MEMORY_SHARE of the device's memory, else "tiled".
-    DUAL_MEMORY_SHARE = 0.45
+    #
+    # The numbers that choose between kernels (DUAL_MEMORY_SHARE, WIDE_MIN_M, MID_*, TARGET_WAVES,
+    # SHARED_ATTENTION_*, ...) are the fields of ``tuning.Tuning``, set on the table at construction.
 
-    def __init__(self, act_dtype: torch.dtype, device="cuda:0"):
+    def __init__(self, act_dtype: torch.dtype, device="cuda:0", tuning: Optional[Tuning] = None):
         if act_dtype not in (torch.bfloat16, torch.float32):
             raise KernelError(f"kernels exist for bfloat16 and float32, not {act_dtype}")
         if not torch.cuda.is_available():
             raise KernelError("servelab_amd needs a GPU: the HIP kernels have no CPU fallback")
         self.act_dtype = act_dtype
         self.device = torch.device(device)
+        self.tuning = tuning if tuning is not None else Tuning()
+        self.tuning.apply(self)
         self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         # the current stream's handle without the wrapper objects torch.cuda.current_stream() builds
         # (a launch is a few microseconds of host time, and this was one of them)
@@ -391,8 +396,6 @@ class HipOps:
             return self.linear_tiled(x, w, bias, out_f32)
         return self.linear_library(x, w, bias)
 
-    WIDE_MIN_M = 17               # from this many rows on, two tiles of W share one read of x
-
     def linear_wide(self, x, weight, bias, out_f32=False, gated=False):
         M, K = x.shape
         N = weight.shape[0]
@@ -402,13 +405,6 @@ class HipOps:
         self._call("gemm", "sl_gemm_wide", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                    int(out_f32), int(gated))
         return y
-
-    MID_TARGET_WORKGROUPS = 224    # K is split until about this many workgroups stream W (fewer splits, fewer partial sums)
-    MID_DEFERRED_WORKGROUPS = 224  # the same when the next norm adds the partial sums of a residual delta
-    MID_PARTIAL_WORKGROUPS = 128   # fewer splits when the reader adds the partial sums (their bytes count twice)
-    MID_WIDE_WORKGROUPS = 128      # workgroups of 8 wavefronts (16 tiles of W per pass over x) if this many remain
-    MID_MIN_ELEMENTS = 48 << 20   # matrices from this size on take the LDS-staged kernel at 17..32 rows ...
-    MID_MIN_ELEMENTS_MANY = 8 << 20   # ... and from this size on at 33..64 rows (x costs more there)
 
     def _takes_mid(self, M, N, K) -> bool:
         return N * K >= (self.MID_MIN_ELEMENTS if M <= 32 else self.MID_MIN_ELEMENTS_MANY)
@@ -482,8 +478,6 @@ class HipOps:
             self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs)
         return y
 
-    RESIDENT_MIN_ROUNDS = 3       # tiles per CU from which workgroups that stay beat one per tile
-
     def _takes_resident(self, N, K) -> bool:
         """Whether a consumer product runs on the workgroups that stay and walk the tiles
         (x in registers, row scales computed once): matrices with several tiles per CU whose
@@ -534,8 +528,8 @@ class HipOps:
         self._call("gemm", "sl_gemm_tiled", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32))
         return y
 
-    LIBRARY_ROW_STEP = 32         # library products of fewer than LIBRARY_PADDED_MAX_M rows run on a
-    LIBRARY_PADDED_MAX_M = 512    # multiple of this many: few distinct shapes, each of which can be tuned
+    # (library products of fewer than LIBRARY_PADDED_MAX_M rows run on a multiple of LIBRARY_ROW_STEP
+    # rows: few distinct shapes, each of which can be tuned)
 
     def library_rows(self, M: int) -> int:
         """The number of rows a library product of M rows of x runs with."""
@@ -848,24 +842,6 @@ class HipOps:
                    _p(batch.positions[first:]), rest, nh, nkv, D, page_size, _c_float(scale),
                    int(window or 0), _p(out[first:]), nsplit, _p(part_o), _p(part_ml))
         return out
-
-    GENERAL_ATTENTION_WAVES = 4096  # the general kernel's decode launches aim for this many wavefronts
-    TARGET_WAVES = 512            # wavefronts a decode launch aims for when it splits the context
-    # Prompt launches share keys through LDS when they have at least MIN_WAVES 32-column wavefronts (enough
-    # workgroups of four, two tiles each) and contexts of MIN_CONTEXT tokens (measured on MI355X, 7B shape:
-    # one prompt of 1,024 tokens 46 us either way, 1,536: 65 against 70 us, 2,048: 80 against 95 us,
-    # 8,192: 737 against 1,125 us; eight prompts of 256: 23.5 against 21.6 us).
-    SHARED_ATTENTION_MIN_WAVES = 1024
-    SHARED_ATTENTION_MIN_CONTEXT = 1024
-    # ... and when such a launch has fewer workgroups than this and its tiles are unpaired (a portion deep
-    # in a long context), every tile is cut into shares of at least MIN_BLOCKS key blocks, at most MAX
-    PROMPT_SPLIT_WORKGROUPS = 4096
-    PROMPT_SPLIT_MIN_BLOCKS = 64
-    PROMPT_SPLIT_MAX = 8
-    PROMPT_SPLIT_BYTES = 512 << 20   # ... and no more shares than keep the partial outputs below this
-    # ... and a launch of fewer workgroups of 128 columns than this takes workgroups of 64 columns (a
-    # wavefront then holds 16 columns and half the registers: three wavefronts fit a SIMD)
-    NARROW_ATTENTION_WORKGROUPS = 400
 
     def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
         """The matrix-core kernels take bfloat16, head sizes that are multiples

@@ -1,0 +1,74 @@
+"""The numbers that choose between kernels, in one place.
+
+Kernel *limits* (how many rows a kernel can take, which head sizes) stay with
+the kernels' wrappers in ``ops.py``: they are facts of the code.  What is here
+are *choices* that were measured on one MI355X with the projection sizes of the
+Qwen2.5 7B, 32B and 72B shapes; another GPU or another architecture's sizes may
+want others.  ``HipOps(dtype, device, tuning=Tuning(target_waves=...))`` takes a
+changed set; every field becomes an attribute of the kernel table under its
+upper-case name (``ops.TARGET_WAVES``), which is what the routing code reads.
+"""
+from dataclasses import dataclass, fields
+
+
+@dataclass
+class Tuning:
+    # ---- weight layouts
+    # both copies of a matrix (row-major for the library, tiled for the few-rows kernels) are kept
+    # while they stay below this share of the device's memory; beyond it only the tiled copy
+    dual_memory_share: float = 0.45
+
+    # ---- products of 17 and more rows over the tiled copy
+    # from this many rows on two tiles of W share one read of x (gemm_wide / gemm_mid)
+    wide_min_m: int = 17
+    # the LDS-staged kernel splits K until about this many workgroups stream W
+    # (fewer splits, fewer partial sums); 224 of 256 CUs busy measured best for o and down
+    mid_target_workgroups: int = 224
+    # the same when the next norm adds the partial sums of a residual delta
+    mid_deferred_workgroups: int = 224
+    # fewer splits when the reader adds the partial sums itself (their bytes count twice)
+    mid_partial_workgroups: int = 128
+    # workgroups of 8 wavefronts (16 tiles of W per pass over x) if this many remain, else 4
+    mid_wide_workgroups: int = 128
+    # matrices of this many elements take the LDS-staged kernel at 17..32 rows ...
+    mid_min_elements: int = 48 << 20
+    # ... and of this many at 33..128 rows, where re-reading x costs more
+    mid_min_elements_many: int = 8 << 20
+
+    # ---- few-rows consumer products on workgroups that stay
+    # tiles per CU from which walking the tiles beats a workgroup per tile (gate/up: 9, head: 37;
+    # q/k/v with one or two tiles a CU has nothing to walk)
+    resident_min_rounds: int = 3
+
+    # ---- library products
+    # products of fewer than library_padded_max_m rows run on a multiple of library_row_step rows:
+    # few distinct shapes, each of which the start-up tuning can time
+    library_row_step: int = 32
+    library_padded_max_m: int = 512
+
+    # ---- attention
+    # wavefronts a decode launch of the general (float32) kernel aims for when it splits the context
+    general_attention_waves: int = 4096
+    # the same for the matrix-core kernel (384, 768 and 1,024 measured within noise or slower)
+    target_waves: int = 512
+    # prompt launches share keys through LDS from this many 32-column wavefronts and this context
+    # on (7B shape, one prompt: 1,024 tokens 46 us either way, 2,048: 80 against 95 us, 8,192: 737
+    # against 1,125 us; eight prompts of 256: 23.5 against 21.6 us)
+    shared_attention_min_waves: int = 1024
+    shared_attention_min_context: int = 1024
+    # such a launch with fewer workgroups than this and unpaired tiles (a portion deep in a long
+    # context) has every tile cut into shares of at least min_blocks key blocks, at most max, and
+    # no more than keep the partial outputs below split_bytes
+    prompt_split_workgroups: int = 4096
+    prompt_split_min_blocks: int = 64
+    prompt_split_max: int = 8
+    prompt_split_bytes: int = 512 << 20
+    # a launch of fewer workgroups of 128 columns than this (and a third of it at least) takes
+    # workgroups of 64 columns: a wavefront then holds 16 columns and three fit a SIMD
+    # (2,048 tokens of the 7B shape: 77 against 88 us)
+    narrow_attention_workgroups: int = 400
+
+    def apply(self, table) -> None:
+        """Sets every field on ``table`` under its upper-case name."""
+        for f in fields(self):
+            setattr(table, f.name.upper(), getattr(self, f.name))
