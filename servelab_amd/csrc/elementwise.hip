@@ -207,11 +207,13 @@ struct __attribute__((aligned(16))) Act8 { act_t v[8]; };
 struct __attribute__((aligned(16))) F4 { float v[4]; };
 
 // q and k heads: a thread rotates 8 pairs (two 8-channel runs) of one head of
-// one token and writes them back, k also to its cache row.
+// one token and writes them back, k also to its cache row.  From partial sums
+// (sp.parts): the 16 inputs are bias + the sums, q is written to qkv and k only
+// to its cache row, as in the kernel above.
 __global__ __launch_bounds__(256) void rope_store_qk_kernel(
-    act_t* __restrict__ qkv, const float* __restrict__ cosv, const float* __restrict__ sinv,
-    const int* __restrict__ slots, act_t* __restrict__ kc, int nh, int nkv, int D, int rot,
-    int page, int pairs8, float qscale) {
+    act_t* __restrict__ qkv, const SplitProduct sp, const float* __restrict__ cosv,
+    const float* __restrict__ sinv, const int* __restrict__ slots, act_t* __restrict__ kc, int nh,
+    int nkv, int D, int rot, int page, int pairs8, float qscale) {
   const int t = blockIdx.x, half = rot / 2, chunks = D / 16, rotated = rot / 16;
   const int items = (nh + nkv) * chunks;
   for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < items; w += gridDim.y * blockDim.x) {
@@ -219,24 +221,53 @@ __global__ __launch_bounds__(256) void rope_store_qk_kernel(
     // chunks below `rotated` hold 8 pairs; the others 16 channels that pass unrotated
     const bool turn = c < rotated;
     const int p1 = !turn || pairs8 ? 16 * c : 8 * c, p2 = !turn || pairs8 ? p1 + 8 : p1 + half;
-    act_t* x = qkv + ((size_t)t * (nh + 2 * nkv) + hd) * D;
-    Act8 a = *(const Act8*)(x + p1), b = *(const Act8*)(x + p2);
+    const size_t row = ((size_t)t * (nh + 2 * nkv) + hd) * D;
+    act_t* x = qkv + row;
+    float xa[8], xb[8];
+    if (sp.parts == nullptr) {
+      const Act8 a = *(const Act8*)(x + p1), b = *(const Act8*)(x + p2);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) xa[j] = to_f(a.v[j]), xb[j] = to_f(b.v[j]);
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        F4 va{{0.f, 0.f, 0.f, 0.f}}, vb = va;
+        if (sp.bias != nullptr) {
+          va = *(const F4*)(sp.bias + hd * D + p1 + 4 * h);
+          vb = *(const F4*)(sp.bias + hd * D + p2 + 4 * h);
+        }
+        for (int j = 0; j < sp.nparts; ++j) {
+          const F4 pa = *(const F4*)(sp.parts + j * sp.stride + row + p1 + 4 * h);
+          const F4 pb = *(const F4*)(sp.parts + j * sp.stride + row + p2 + 4 * h);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) va.v[i] += pa.v[i], vb.v[i] += pb.v[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xa[4 * h + i] = va.v[i], xb[4 * h + i] = vb.v[i];
+      }
+    }
     const float qs = hd < nh ? qscale : 1.f;
-    if ((cosv != nullptr && turn) || qs != 1.f) {
+    const bool changed = (cosv != nullptr && turn) || qs != 1.f;
+    if (changed) {
       F4 c0{{1.f, 1.f, 1.f, 1.f}}, c1 = c0, s0{{0.f, 0.f, 0.f, 0.f}}, s1 = s0;
       if (cosv != nullptr && turn) {
         const float* cp = cosv + (size_t)t * half + 8 * c;
-        const float* sp = sinv + (size_t)t * half + 8 * c;
+        const float* sn = sinv + (size_t)t * half + 8 * c;
         c0 = *(const F4*)cp, c1 = *(const F4*)(cp + 4);
-        s0 = *(const F4*)sp, s1 = *(const F4*)(sp + 4);
+        s0 = *(const F4*)sn, s1 = *(const F4*)(sn + 4);
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float cs = j < 4 ? c0.v[j] : c1.v[j - 4], sn = j < 4 ? s0.v[j] : s1.v[j - 4];
-        const float x1 = to_f(a.v[j]), x2 = to_f(b.v[j]);
-        a.v[j] = from_f<act_t>((x1 * cs - x2 * sn) * qs);
-        b.v[j] = from_f<act_t>((x2 * cs + x1 * sn) * qs);
+        const float x1 = xa[j], x2 = xb[j];
+        xa[j] = (x1 * cs - x2 * sn) * qs;
+        xb[j] = (x2 * cs + x1 * sn) * qs;
       }
+    }
+    Act8 a, b;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) a.v[j] = from_f<act_t>(xa[j]), b.v[j] = from_f<act_t>(xb[j]);
+    if (sp.parts != nullptr ? hd < nh : changed) {
       *(Act8*)(x + p1) = a;
       *(Act8*)(x + p2) = b;
     }
@@ -253,8 +284,8 @@ __global__ __launch_bounds__(256) void rope_store_qk_kernel(
 // that neighbouring lanes write neighbouring slots of a channel's row (tokens
 // of one request usually sit in consecutive slots of a page).
 __global__ __launch_bounds__(256) void store_v_kernel(
-    const act_t* __restrict__ qkv, const int* __restrict__ slots, act_t* __restrict__ vc, int T,
-    int nh, int nkv, int D, int page) {
+    const act_t* __restrict__ qkv, const SplitProduct sp, const int* __restrict__ slots,
+    act_t* __restrict__ vc, int T, int nh, int nkv, int D, int page) {
   __shared__ act_t tile[16][256 + 2];
   __shared__ int slot_of[16];
   const int t0 = blockIdx.x * 16, kvh = blockIdx.y;
@@ -262,7 +293,14 @@ __global__ __launch_bounds__(256) void store_v_kernel(
   if (threadIdx.x < 16) slot_of[threadIdx.x] = threadIdx.x < nt ? slots[t0 + threadIdx.x] : 0;
   for (int idx = threadIdx.x; idx < nt * D; idx += blockDim.x) {
     const int i = idx / D, d = idx % D;
-    tile[i][d] = qkv[((size_t)(t0 + i) * (nh + 2 * nkv) + nh + nkv + kvh) * D + d];
+    const size_t at = ((size_t)(t0 + i) * (nh + 2 * nkv) + nh + nkv + kvh) * D + d;
+    if (sp.parts == nullptr) {
+      tile[i][d] = qkv[at];
+    } else {
+      float v = sp.bias != nullptr ? sp.bias[(nh + nkv + kvh) * D + d] : 0.f;
+      for (int j = 0; j < sp.nparts; ++j) v += sp.parts[j * sp.stride + at];
+      tile[i][d] = from_f<act_t>(v);
+    }
   }
   __syncthreads();
   for (int idx = threadIdx.x; idx < 16 * D; idx += blockDim.x) {
@@ -299,14 +337,16 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
   if (cosv == nullptr && kc == nullptr && parts == nullptr && qscale == 1.f) return nullptr;
   const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)kc % 16) == 0 &&
                        ((uintptr_t)cosv % 16) == 0 && ((uintptr_t)sinv % 16) == 0;
-  if (parts == nullptr && T >= VECTOR_MIN_TOKENS && D % 16 == 0 && rot % 16 == 0 && D <= 256 && aligned &&
+  const bool sums_aligned = parts == nullptr || (((uintptr_t)parts % 16) == 0 && ((uintptr_t)bias % 16) == 0 &&
+                                                  ((size_t)T * (nh + 2 * nkv) * D) % 4 == 0);
+  if (T >= VECTOR_MIN_TOKENS && D % 16 == 0 && rot % 16 == 0 && D <= 256 && aligned && sums_aligned &&
       nkv <= 65535) {
     const int items = (nh + nkv) * (D / 16);
     rope_store_qk_kernel<<<dim3(T, (items + 255) / 256 < 64 ? (items + 255) / 256 : 64), 256, 0, stream>>>(
-        (act_t*)qkv, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, rot, page, pairs8, qscale);
+        (act_t*)qkv, sp, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, rot, page, pairs8, qscale);
     const char* e = sl_launch_status();
     if (e || vc == nullptr) return e;
-    store_v_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>((const act_t*)qkv, slots, (act_t*)vc, T,
+    store_v_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>((const act_t*)qkv, sp, slots, (act_t*)vc, T,
                                                                  nh, nkv, D, page);
     return sl_launch_status();
   }

@@ -484,13 +484,15 @@ def test_rotation_plans():
                         None, None, None, 16)
 
 
-@pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (28, 4, 128, 16), (5, 1, 48, 32)])
-def test_rope_store_from_partial_sums(both, nh, nkv, D, page):
+@pytest.mark.parametrize("T", [40, 300])
+@pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (28, 4, 128, 16), (5, 1, 48, 32), (3, 1, 96, 64)])
+def test_rope_store_from_partial_sums(both, nh, nkv, D, page, T):
     """The q/k/v product arrives as float partial sums of a split K plus a bias:
-    rotation and cache write see their sum; q lands in the buffer."""
+    rotation and cache write see their sum; q lands in the buffer.  With few tokens one
+    block per token and head, with many the vectorised pair of kernels."""
     from servelab_amd.kernels.ops import PartialSums
     ops, emu, dt = both
-    T, pages, N = 40, 9, (nh + 2 * nkv) * D
+    pages, N = -(-T // page) + 3, (nh + 2 * nkv) * D
     parts = randn(3, T, N, seed=1)
     bias = randn(N, seed=2)
     inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
