@@ -1036,7 +1036,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ wt, const float* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int out_f32, int gated, int KS) {
   constexpr int THREADS = 64 * WAVES;
-  __shared__ bf16x8 xs[2][KC][MB][64];
+  // chunks of W in flight or in use (LDS holds as many of x): three for the workgroups of eight
+  // wavefronts where the registers and LDS allow it (gate/up of the 7B shape at 64 rows: 52 -> 49 us);
+  // with four wavefronts (K split over workgroups) the third set measured slower (17.1 -> 17.8 us)
+  constexpr int DEPTH = MB <= 4 && WAVES == 8 ? 3 : 2;
+  __shared__ bf16x8 xs[DEPTH][KC][MB][64];
   // the wavefront's index as a scalar: what depends on it (its share of K, its tiles) then steers
   // real branches; matrix instructions ignore the execution mask, so they must not sit under a
   // condition the compiler takes for divergent and may turn into masking
@@ -1094,77 +1098,135 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
       xs[buf][idx / (MB * 64)][idx / 64 % MB][idx % 64] = kbeg + c * KC + xks[j] < kend ? xr[j] : zero;
     }
   };
-  auto load_w = [&](int c, bf16x8 (&a)[NT][KC]) {
-#pragma unroll
-    for (int u = 0; u < KC; ++u) {
-      int ks = kbeg + c * KC + u;
-      if (ks >= kend) ks = kend - 1;               // its x is zero
-#pragma unroll
-      for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)ks);
-    }
-  };
   f32x4 acc[NT][MB];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int b = 0; b < MB; ++b) acc[t][b] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // Two sets of W registers, the chunk loop unrolled over them: the loads of
-  // the next chunk stay in flight until its own products need them (a copy
-  // from one set into the other would wait for them at once).
-  bf16x8 a0[NT][KC], a1[NT][KC], xr[XF];
-  // The x operands of a k-step are read from LDS two k-steps before their
-  // products; the scheduling barriers keep the compiler from moving the reads
-  // back next to their use, where every pair of products would wait out the
-  // full latency of LDS (this made the kernel's time grow with the rows of x).
-  auto multiply = [&](int buf, const bf16x8 (&a)[NT][KC]) {
-    bf16x8 bv[2][MB];
+  // The chunk loop, written once for a wavefront with all NT tiles and once for one with fewer
+  // (the last workgroups of an uneven share): a wavefront takes the branch as a whole, so each
+  // form is straight-line code whose loads the compiler can count, and a wavefront without a
+  // second tile neither loads nor multiplies for it (its loads would take places in the CU's
+  // queue of outstanding requests, which is what limits these kernels).
+  auto run = [&](auto ntl_tag) {
+    constexpr int NTL = decltype(ntl_tag)::value;
+    auto load_w = [&](int c, bf16x8 (&a)[NT][KC]) {
 #pragma unroll
-    for (int u = 0; u < 2 && u < KC; ++u)
+      for (int u = 0; u < KC; ++u) {
+        int ks = kbeg + c * KC + u;
+        if (ks >= kend) ks = kend - 1;               // its x is zero
 #pragma unroll
-      for (int b = 0; b < MB; ++b) bv[u][b] = xs[buf][u][b][lane];
+        for (int t = 0; t < NTL; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)ks);
+      }
+    };
+    // The x operands of a k-step are read from LDS two k-steps before their
+    // products; the scheduling barriers keep the compiler from moving the reads
+    // back next to their use, where every pair of products would wait out the
+    // full latency of LDS (this made the kernel's time grow with the rows of x).
+    auto multiply = [&](int buf, const bf16x8 (&a)[NT][KC]) {
+      bf16x8 bv[2][MB];
 #pragma unroll
-    for (int u = 0; u < KC; ++u) {
-      __builtin_amdgcn_sched_barrier(0);
+      for (int u = 0; u < 2 && u < KC; ++u)
 #pragma unroll
-      for (int b = 0; b < MB; ++b)
+        for (int b = 0; b < MB; ++b) bv[u][b] = xs[buf][u][b][lane];
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv[u & 1][b], acc[t][b], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (u + 2 < KC) {
+      for (int u = 0; u < KC; ++u) {
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int b = 0; b < MB; ++b) bv[u & 1][b] = xs[buf][u + 2][b][lane];
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+          for (int t = 0; t < NTL; ++t)
+            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv[u & 1][b], acc[t][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (u + 2 < KC) {
+#pragma unroll
+          for (int b = 0; b < MB; ++b) bv[u & 1][b] = xs[buf][u + 2][b][lane];
+        }
+      }
+    };
+    // Sets of W registers, the chunk loop unrolled over them: the loads of the chunks ahead stay
+    // in flight until their own products need them (a copy from one set into another would wait
+    // for them at once).
+    bf16x8 a0[NT][KC], a1[NT][KC], xr[XF];
+    if constexpr (DEPTH == 3) {
+      // W and x are asked for two chunks ahead (x into registers, stored to LDS one chunk ahead).
+      // Loads return in order, so a wait for a chunk's x must not have a later chunk's W before
+      // it: every step asks for x, then W, of the chunk two ahead, and waits only for what is older.
+      bf16x8 a2[NT][KC], xr1[XF], xr2[XF];
+      load_x(0, xr);
+      load_w(0, a0);
+      load_x(1, xr1);                              // (past the end: the last k-step again; stored as zeros)
+      load_w(1, a1);
+      store_x(0, 0, xr);
+      int c = 0;
+      for (; c + 3 < nchunks; c += 3) {
+        __syncthreads();
+        load_x(c + 2, xr2);
+        load_w(c + 2, a2);
+        multiply(0, a0);
+        store_x(1, c + 1, xr1);
+        __syncthreads();
+        load_x(c + 3, xr);
+        load_w(c + 3, a0);
+        multiply(1, a1);
+        store_x(2, c + 2, xr2);
+        __syncthreads();
+        load_x(c + 4, xr1);
+        load_w(c + 4, a1);
+        multiply(2, a2);
+        store_x(0, c + 3, xr);
+      }
+      // the last one to three chunks: W of c in a0 and of c + 1 in a1, x of c in LDS and of c + 1 in xr1
+      __syncthreads();
+      if (c + 2 < nchunks) {
+        load_x(c + 2, xr2);
+        load_w(c + 2, a2);
+      }
+      multiply(0, a0);
+      if (c + 1 < nchunks) {
+        store_x(1, c + 1, xr1);
+        __syncthreads();
+        multiply(1, a1);
+        if (c + 2 < nchunks) {
+          store_x(2, c + 2, xr2);
+          __syncthreads();
+          multiply(2, a2);
+        }
+      }
+    } else {
+      load_x(0, xr);
+      load_w(0, a0);
+      store_x(0, 0, xr);
+      int c = 0;
+      for (; c + 2 < nchunks; c += 2) {
+        __syncthreads();
+        load_x(c + 1, xr);
+        load_w(c + 1, a1);
+        multiply(0, a0);
+        store_x(1, c + 1, xr);
+        __syncthreads();
+        load_x(c + 2, xr);
+        load_w(c + 2, a0);
+        multiply(1, a1);
+        store_x(0, c + 2, xr);
+      }
+      // the last one or two chunks
+      __syncthreads();
+      if (c + 1 < nchunks) {
+        load_x(c + 1, xr);
+        load_w(c + 1, a1);
+      }
+      multiply(0, a0);
+      if (c + 1 < nchunks) {
+        store_x(1, c + 1, xr);
+        __syncthreads();
+        multiply(1, a1);
       }
     }
   };
-  load_x(0, xr);
-  load_w(0, a0);
-  store_x(0, 0, xr);
-  int c = 0;
-  for (; c + 2 < nchunks; c += 2) {
-    __syncthreads();
-    load_x(c + 1, xr);
-    load_w(c + 1, a1);
-    multiply(0, a0);
-    store_x(1, c + 1, xr);
-    __syncthreads();
-    load_x(c + 2, xr);
-    load_w(c + 2, a0);
-    multiply(1, a1);
-    store_x(0, c + 2, xr);
-  }
-  // the last one or two chunks
-  __syncthreads();
-  if (c + 1 < nchunks) {
-    load_x(c + 1, xr);
-    load_w(c + 1, a1);
-  }
-  multiply(0, a0);
-  if (c + 1 < nchunks) {
-    store_x(1, c + 1, xr);
-    __syncthreads();
-    multiply(1, a1);
-  }
+  // (live[t] comes from the wavefront's index and the workgroup's: a scalar, so this is a real branch)
+  if (live[NT - 1]) run(std::integral_constant<int, NT>{});
+  else run(std::integral_constant<int, (NT > 1 ? NT - 1 : 1)>{});
   // lane: column m = 16 b + i of x, rows n = 16 tile + 4 gq + r of W
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
