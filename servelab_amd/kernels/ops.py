@@ -80,6 +80,20 @@ class Deferred:
         self.x, self.weight, self.bias = x, weight, bias
 
 
+class TiledRows:
+    """Few rows of activations [M, K] laid out by k-step (element (m, k) at
+    (k // 32) * (M * 32) + m * 32 + k % 32): what a gated product writes for the
+    product that reads it (``HipOps.gated_mlp``).  Never leaves the kernel table."""
+    __slots__ = ("data", "shape")
+
+    def __init__(self, data, shape):
+        self.data, self.shape = data, tuple(shape)
+
+    def rows(self):
+        M, K = self.shape
+        return self.data.view(K // 32, M, 32).permute(1, 0, 2).reshape(M, K)
+
+
 class PartialSums:
     """A product whose K was split over workgroups, left as float partial sums
     ``parts`` [ks, T, N] with the bias not yet added, for a reader that adds
@@ -97,14 +111,22 @@ class ScaledRows:
     sums of squares of the stream by row.  Only ``linear`` and ``gated_linear``
     read them: they scale their result rows instead.  ``rows`` optionally
     selects which rows take part."""
-    __slots__ = ("x", "parts", "eps", "rows")
+    __slots__ = ("x", "parts", "eps", "rows", "tiled")
 
-    def __init__(self, x, parts, eps, rows=None):
+    def __init__(self, x, parts, eps, rows=None, tiled=0):
         self.x, self.parts, self.eps, self.rows = x, parts, eps, rows
+        self.tiled = tiled          # x is laid out by k-step (see TiledRows) with this many rows; 0: plain rows
 
     @property
     def shape(self):
         return (self.rows.shape[0] if self.rows is not None else self.x.shape[0], self.x.shape[1])
+
+    def plain_x(self):
+        """``x`` as plain rows (a copy when it is laid out by k-step)."""
+        if not self.tiled:
+            return self.x
+        T, K = self.x.shape
+        return self.x.reshape(K // 32, T, 32).permute(1, 0, 2).reshape(T, K)
 
 
 class HipOps:
@@ -149,6 +171,7 @@ class HipOps:
         self._resident_k = {}
         self.fuse_norms = act_dtype == torch.bfloat16
         self.fuse_rope = act_dtype == torch.bfloat16
+        self.tile_few_rows = act_dtype == torch.bfloat16      # gated_mlp keeps few rows tiled by k-step
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
         self._untiled = None          # scratch for "tiled": the row-major form of one matrix
         # Up to this many rows no product of a prepared weight goes to the library
@@ -203,15 +226,18 @@ class HipOps:
         return two < 0.97 * one
 
     def _skinny(self, x, weight, bias, y, M, N, K, out_f32=False, gated=False, scaled=None,
-                resid=None, next_gain=None, out_parts=None, rope=None):
+                resid=None, next_gain=None, out_parts=None, rope=None, y_tiled=False):
         """One call of the few-rows kernel (at most 16 rows) in any of its forms."""
         parts = scaled.parts if scaled is not None else None
+        x_tiled = scaled.tiled if scaled is not None else 0
+        if isinstance(x, TiledRows):
+            x_tiled, x = x.shape[0], x.data
         self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                    int(out_f32), int(gated), _p(parts), parts.shape[0] if parts is not None else 0,
                    _c_float(scaled.eps if scaled is not None else 0.0),
                    _p(scaled.rows) if scaled is not None else None, _p(resid), _p(next_gain),
                    _p(out_parts), ctypes.byref(rope) if rope is not None else None,
-                   int(self._pair_tiles(M, N, K)))
+                   int(self._pair_tiles(M, N, K)), int(x_tiled), int(y_tiled))
 
     # ------------------------------------------------------------ embedding
     def embed(self, ids, table):
@@ -288,13 +314,15 @@ class HipOps:
         N = weight.shape[0]
         if tuple(resid.shape) != (M, N):
             raise KernelError(f"a delta of shape {[M, N]} does not fit the stream {list(resid.shape)}")
-        self._check(x, self.act_dtype, None, "x")
+        self._check(x.data if isinstance(x, TiledRows) else x, self.act_dtype, None, "x")
         if d.bias is not None:
             self._check(d.bias, torch.float32, (N,), "bias")
         out = self._new((M, N))
         parts = self._new((-(-N // 16), 16), torch.float32)
-        self._skinny(x, weight, d.bias, out, M, N, K, resid=resid, next_gain=gain, out_parts=parts)
-        return ScaledRows(out, parts, eps)
+        tiled = M if self.tile_few_rows and M > 1 and N % 32 == 0 else 0     # for the products that read the rows
+        self._skinny(x, weight, d.bias, out, M, N, K, resid=resid, next_gain=gain, out_parts=parts,
+                     y_tiled=bool(tiled))
+        return ScaledRows(out, parts, eps, tiled=tiled)
 
     # --------------------------------------------------------------- linear
     def plan_weights(self, total_bytes: int) -> str:
@@ -358,6 +386,13 @@ class HipOps:
             return self._linear_scaled(x, weight, bias, out_f32, False)
         M, K = x.shape
         N = weight.shape[0]
+        if isinstance(x, TiledRows) and not (defer and self.fuse_norms and not out_f32 and N <= 8192):
+            # (rows by k-step are read by the few-rows kernel only, which is where they come from)
+            if weight.shape != (N, K):
+                raise KernelError(f"weight has shape {list(weight.shape)}, x has {K} columns")
+            y = self._new((M, N), torch.float32 if out_f32 else None)
+            self._skinny(x, weight, bias, y, M, N, K, out_f32)
+            return y
         if (defer and self.fuse_norms and not out_f32 and 0 < M <= self.FUSED_NORM_MAX_M
                 and weight.tiled is not None and weight.shape == (N, K) and N <= 8192):
             return Deferred(x, weight, bias)
@@ -460,7 +495,7 @@ class HipOps:
         self._skinny(x, weight, bias, y, M, N, K, out_f32)
         return y
 
-    def _linear_scaled(self, xs, weight, bias, out_f32, gated):
+    def _linear_scaled(self, xs, weight, bias, out_f32, gated, y_tiled=False):
         """The consumer of un-normalised rows: one few-rows product that scales
         its result rows by rsqrt(mean x^2 + eps)."""
         M, K = xs.shape
@@ -473,10 +508,10 @@ class HipOps:
         if self._takes_resident(N, K):
             self._call("gemm", "sl_gemm_resident", _p(xs.x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                        int(out_f32), int(gated), _p(xs.parts), xs.parts.shape[0], _c_float(xs.eps),
-                       _p(xs.rows))
+                       _p(xs.rows), int(xs.tiled), int(y_tiled))
         else:
-            self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs)
-        return y
+            self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs, y_tiled=y_tiled)
+        return TiledRows(y, (M, N // 2)) if y_tiled else y
 
     def _takes_resident(self, N, K) -> bool:
         """Whether a consumer product runs on the workgroups that stay and walk the tiles
@@ -491,7 +526,7 @@ class HipOps:
 
     GATE_BLOCK = 8                # gate and up rows alternate in blocks of 8 (half an MFMA tile)
 
-    def gated_linear(self, x, weight, block):
+    def gated_linear(self, x, weight, block, _tiled_out=False):
         """silu(x Wg^T) * (x Wu^T) for a weight whose rows hold gate and up
         interleaved in blocks of ``block`` rows (``block`` = I: plain [Wg; Wu]).
         Few rows and a tiled weight with blocks of 8: one fused kernel."""
@@ -500,9 +535,15 @@ class HipOps:
         if isinstance(x, ScaledRows):
             if block != self.GATE_BLOCK or weight.shape[0] % 16:
                 raise KernelError("un-normalised rows need gate and up in blocks of 8")
-            return self._linear_scaled(x, weight, None, False, True)
+            return self._linear_scaled(x, weight, None, False, True, y_tiled=_tiled_out)
         M, K = x.shape
         N = weight.shape[0]
+        if (_tiled_out and M < self.WIDE_MIN_M and M <= self._few_rows_limit(weight)
+                and block == self.GATE_BLOCK and N % 16 == 0):
+            self._check(x, self.act_dtype, None, "x")
+            y = self._new((M, N // 2))
+            self._skinny(x, weight, None, y, M, N, K, gated=True, y_tiled=True)
+            return TiledRows(y, (M, N // 2))
         if M <= self._few_rows_limit(weight) and block == self.GATE_BLOCK and N % 16 == 0:
             self._check(x, self.act_dtype, None, "x")
             if M >= self.WIDE_MIN_M:
@@ -513,6 +554,23 @@ class HipOps:
             self._skinny(x, weight, None, y, M, N, K, gated=True)
             return y
         return self.silu_mul(self.linear(x, weight, None), block)
+
+    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False):
+        """down(silu(gate x) * (up x)): ``gated_linear`` followed by ``linear``.  With few rows the
+        kernel table keeps what lies between them in the layout its second kernel reads best
+        (rows by k-step: the eight rows of a decode step then cost the down product half as many
+        cache lines per load of x)."""
+        if not isinstance(w_gate_up, LinearWeight):
+            w_gate_up = LinearWeight(w_gate_up)
+        if not isinstance(w_down, LinearWeight):
+            w_down = LinearWeight(w_down)
+        M = x.shape[0]
+        inner = w_gate_up.shape[0] // 2
+        tiled = (self.act_dtype == torch.bfloat16 and self.tile_few_rows and 1 < M <= self.FUSED_NORM_MAX_M
+                 and block == self.GATE_BLOCK and inner % 32 == 0 and w_gate_up.tiled is not None
+                 and w_down.tiled is not None and w_down.shape[1] == inner and w_gate_up.shape[0] % 16 == 0)
+        h = self.gated_linear(x, w_gate_up, block, _tiled_out=tiled)
+        return self.linear(h, w_down, None, defer=defer)
 
     def linear_rows(self, x, w, bias, out_f32=False):
         M, K = x.shape

@@ -41,5 +41,4 @@ class GatedMLP(FeedForward):
 
     def forward(self, x):
         ops = self.rt.ops
-        return ops.linear(ops.gated_linear(x, self.w_gate_up, self.block), self.w_down, None,
-                          defer=True)
+        return ops.gated_mlp(x, self.w_gate_up, self.block, self.w_down, defer=True)

@@ -53,6 +53,9 @@ class EmulatedOps:
         g, u = gu[:, :, 0].reshape(T, inter), gu[:, :, 1].reshape(T, inter)
         return (g * torch.sigmoid(g) * u).to(self.act_dtype)
 
+    def gated_mlp(self, x, w_gate_up, block, w_down, defer=False):
+        return self.linear(self.gated_linear(x, w_gate_up, block), w_down, None, defer=defer)
+
     def gated_linear(self, x, w, block):
         return self.silu_mul(self.linear(x, w, None), block)
 

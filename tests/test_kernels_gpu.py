@@ -376,6 +376,45 @@ def test_consumer_products_on_workgroups_that_stay(M, H, N2):
         ops.linear(odd, ops.prepare_weight(randn(32, H + 32, dtype=torch.bfloat16, seed=3)), None)
 
 
+@pytest.mark.parametrize("M,H,I", [(2, 256, 64), (8, 3584, 18944), (16, 2048, 96), (5, 96, 160), (13, 512, 4128)])
+def test_gated_mlp_keeps_few_rows_by_k_step_between_its_two_products(M, H, I):
+    """gate/up and down in one call: with few rows what lies between them is laid out by k-step;
+    the numbers are those of the two calls with a plain tensor between them, bit for bit, from
+    plain rows and from un-normalised ones, as a finished tensor and as a product left to the norm."""
+    from servelab_amd.kernels import HipOps
+    from servelab_amd.kernels.ops import Deferred, ScaledRows, TiledRows
+    dt = torch.bfloat16
+    ops = HipOps(dt, "cuda:0")
+    gu = ops.prepare_weight(randn(2 * I, H, dtype=dt, scale=0.5 / H ** 0.5, seed=1))
+    down = ops.prepare_weight(randn(H, I, dtype=dt, scale=1.0 / I ** 0.5, seed=2))
+    x = randn(M, H, dtype=dt, seed=3)
+    parts = randn(-(-H // 16), 16, seed=4).abs().contiguous()
+    gain = 1 + 0.1 * randn(H, seed=5)
+    resid0 = randn(M, H, seed=6)
+    got = {}
+    for tiled in (False, True):
+        ops.tile_few_rows = tiled
+        out = []
+        for xin in (x, ScaledRows(x, parts, 1e-5)):
+            out.append(ops.gated_mlp(xin, gu, 8, down))
+            d = ops.gated_mlp(xin, gu, 8, down, defer=True)
+            assert isinstance(d, Deferred) and isinstance(d.x, TiledRows) == tiled
+            if tiled:                                   # what lies between is the plain tensor, rearranged
+                assert torch.equal(d.x.rows(), ops.gated_linear(xin, gu, 8))
+            out.append(ops.materialize(d))
+            resid = resid0.clone()
+            scaled = ops.add_rmsnorm(resid, d, gain, 1e-5, fuse=True)
+            assert bool(scaled.tiled) == (tiled and M > 1 and H % 32 == 0)
+            out += [resid, scaled.plain_x(), scaled.parts, ops.linear(scaled, gu, None)]
+        got[tiled] = out
+    for a, b in zip(got[False], got[True]):
+        assert a.shape == b.shape and torch.equal(a, b)
+    # against the formula: gate and up rows alternate in blocks of 8
+    w = gu.w.float().reshape(I // 8, 2, 8, H)
+    h = (torch.nn.functional.silu(x.float() @ w[:, 0].reshape(I, H).T) * (x.float() @ w[:, 1].reshape(I, H).T)).to(dt)
+    assert rel_err(got[True][0], h.float() @ down.w.float().T) < 2 ** -5
+
+
 def test_rope_tables(both):
     ops, emu, dt = both
     D, theta = 48, 1e6
