@@ -468,40 +468,47 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
   f32x4 acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  int ks = ks0;
-  for (; ks + U <= ks1; ks += U) {
-    bf16x8 a[NT][U];
+  // The K loop, written once for plain rows of x (a constant step from one k-step to the next,
+  // folded into the loads' offsets) and once for rows laid out by k-step.
+  auto stream_k = [&](auto tiled_tag) {
+    const size_t xs_ = decltype(tiled_tag)::value ? xstep : (size_t)32;
+    int ks = ks0;
+    for (; ks + U <= ks1; ks += U) {
+      bf16x8 a[NT][U];
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const bf16x8 bv = *(const bf16x8*)(xp + xstep * (size_t)(ks + u));
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv, acc[t], 0, 0, 0);
-    }
-  }
-  if (ks < ks1) {
-    // the last k-steps, fewer than U: all their loads are issued before the
-    // first product, so they cost one trip to memory, not one each
-    bf16x8 a[NT][U], bv[U];
-#pragma unroll
-    for (int u = 0; u < U - 1; ++u)
-      if (ks + u < ks1) {
+      for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
-        bv[u] = *(const bf16x8*)(xp + xstep * (size_t)(ks + u));
-      }
 #pragma unroll
-    for (int u = 0; u < U - 1; ++u)
-      if (ks + u < ks1) {
+      for (int u = 0; u < U; ++u) {
+        const bf16x8 bv = *(const bf16x8*)(xp + xs_ * (size_t)(ks + u));
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv[u], acc[t], 0, 0, 0);
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv, acc[t], 0, 0, 0);
       }
-  }
+    }
+    if (ks < ks1) {
+      // the last k-steps, fewer than U: all their loads are issued before the
+      // first product, so they cost one trip to memory, not one each
+      bf16x8 a[NT][U], bv[U];
+#pragma unroll
+      for (int u = 0; u < U - 1; ++u)
+        if (ks + u < ks1) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
+          bv[u] = *(const bf16x8*)(xp + xs_ * (size_t)(ks + u));
+        }
+#pragma unroll
+      for (int u = 0; u < U - 1; ++u)
+        if (ks + u < ks1) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], bv[u], acc[t], 0, 0, 0);
+        }
+    }
+  };
+  if (F.x_tiled) stream_k(std::true_type{});
+  else stream_k(std::false_type{});
 #pragma unroll
   for (int t = 0; t < NT; ++t) red[t][wave][lane] = acc[t];
   if (CONSUMER) {            // this wavefront's share of the sums of squares, by row
