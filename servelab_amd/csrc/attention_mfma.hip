@@ -97,7 +97,14 @@ struct AttnParams {
   float* part_ml;                // [rows, nh, nsplit, 2]
   int part_row0;                 // token index of partial row 0
   int pair;                      // prompt workgroups take a late tile and its early mirror
+  int out_rows;                  // 0: out is [T, nh * D]; else its rows are laid out by k-step for the few-rows
+                                 // product that reads them: element (t, c) at (c / 32) * (out_rows * 32) + t * 32 + c % 32
 };
+
+// where element (row, col) of the result goes (col = head * D + channel; runs of four channels stay together)
+__device__ __forceinline__ size_t out_index(int out_rows, int nh, size_t row, int col) {
+  return out_rows ? (size_t)(col / 32) * (out_rows * 32) + row * 32 + col % 32 : row * (size_t)(nh * D) + col;
+}
 
 // The columns of one wavefront: queries, reference points and sums, outputs.
 //
@@ -309,13 +316,12 @@ struct Columns {
         }
       } else {
         const float inv = 1.f / l;
-        __bf16* po = P.out + (row * P.nh + head[b]) * D + 4 * gq;
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd) {
           bf16x4 r;
 #pragma unroll
           for (int j = 0; j < 4; ++j) r[j] = (__bf16)(o[b][dd][j] * inv);
-          *(bf16x4*)(po + 16 * dd) = r;
+          *(bf16x4*)(P.out + out_index(P.out_rows, P.nh, row, head[b] * D + 16 * dd + 4 * gq)) = r;
         }
       }
     }
@@ -679,7 +685,7 @@ void attention_mfma_shared_kernel(const AttnParams P) {
 // of eight splits in flight at a time.
 __global__ __launch_bounds__(64) void attention_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int nsplit, int nh,
-    int part_row0, __bf16* __restrict__ out) {
+    int part_row0, __bf16* __restrict__ out, int out_rows) {
   __shared__ float ws[64];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)r * nh + h) * nsplit;
@@ -695,7 +701,6 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
   __syncthreads();
   const float inv = 1.f / denom;
   const float* po = part_o + base * D;
-  __bf16* o = out + ((size_t)(part_row0 + r) * nh + h) * D;
   for (int d = lane; d < D; d += 64) {
     float acc = 0.f;
     int j = 0;
@@ -707,7 +712,7 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
       for (int u = 0; u < 8; ++u) acc += ws[j + u] * v[u];
     }
     for (; j < nsplit; ++j) acc += ws[j] * po[(size_t)j * D + d];
-    o[d] = (__bf16)(acc * inv);
+    out[out_index(out_rows, nh, (size_t)(part_row0 + r), h * D + d)] = (__bf16)(acc * inv);
   }
 }
 
@@ -728,7 +733,7 @@ extern "C" const char* sl_attention_mfma(
     int max_pages, const int* cu_q, const int* positions, int seq_begin, int num_seqs,
     int max_q_len, int nh, int nkv, int head_dim, int page, float scale, int window, int nsplit,
     int shared_min_waves, int pair_tiles, void* out, float* part_o, float* part_ml, int part_row0, int part_rows,
-    int narrow_below, hipStream_t stream) {
+    int narrow_below, int out_rows, hipStream_t stream) {
   SL_CHECK(head_dim == D, "attention_mfma: built for another head size");
   SL_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: heads must be a multiple of kv heads");
   SL_CHECK(page == 16 || page == 32 || page == 64, "attention_mfma: page size must be 16, 32 or 64");
@@ -741,7 +746,9 @@ extern "C" const char* sl_attention_mfma(
   const int g = nh / nkv;
   AttnParams P{(const __bf16*)qkv, row_stride, (const __bf16*)kc, (const __bf16*)vc, block_tables,
                max_pages, cu_q, positions, seq_begin, nh, nkv, page, scale, window, nsplit,
-               (__bf16*)out, part_o, part_ml, part_row0, pair_tiles};
+               (__bf16*)out, part_o, part_ml, part_row0, pair_tiles, out_rows};
+  SL_CHECK(out_rows >= 0 && (out_rows == 0 || (max_q_len == 1 && seq_begin == 0 && out_rows == num_seqs)),
+           "attention_mfma: a result laid out by k-step is that of a step of single tokens, all of its rows");
   const long long cols = (long long)max_q_len * g;
   // scale * log2(e) == 1: the caller's q is already in units of log 2 (see Columns)
   const bool fold = fabsf(scale * 1.4426950408889634f - 1.f) < 1e-6f;
@@ -763,7 +770,7 @@ extern "C" const char* sl_attention_mfma(
     const char* e = sl_launch_status();
     if (e) return e;
     attention_combine_kernel<<<dim3(num_seqs, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh,
-                                                                  part_row0, (__bf16*)out);
+                                                                  part_row0, (__bf16*)out, out_rows);
     return sl_launch_status();
   }
   // Prompt portions.  One wavefront per 32 columns, each reading its keys
@@ -806,7 +813,7 @@ extern "C" const char* sl_attention_mfma(
       const char* e = sl_launch_status();
       if (e) return e;
       attention_combine_kernel<<<dim3(part_rows, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh,
-                                                                    part_row0, (__bf16*)out);
+                                                                    part_row0, (__bf16*)out, out_rows);
     }
   }
   return sl_launch_status();

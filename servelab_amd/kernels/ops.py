@@ -851,8 +851,24 @@ class HipOps:
         return qkv
 
     # ------------------------------------------------------------ attention
+    def attend_and_project(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                           batch, scale, window, w_out, bias=None, defer=False):
+        """``paged_attention`` followed by ``linear`` with the output projection.  For a step of a few
+        single tokens the kernel table keeps what lies between them laid out by k-step, as
+        ``gated_mlp`` does (at 16 rows the projection reads as many bytes of x as of W)."""
+        if not isinstance(w_out, LinearWeight):
+            w_out = LinearWeight(w_out)
+        T = qkv.shape[0]
+        tiled = (self.tile_few_rows and 1 < T <= self.FUSED_NORM_MAX_M and batch.max_q_len == 1
+                 and batch.num_prefill_seqs == 0 and batch.num_seqs == T and w_out.tiled is not None
+                 and w_out.shape[1] == nh * D
+                 and self._mfma_attention_fits(D, nh // nkv, block_tables.shape[1], page_size, batch))
+        attn = self.paged_attention(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                                    batch, scale, window, _tiled_out=tiled)
+        return self.linear(attn, w_out, bias, defer=defer)
+
     def paged_attention(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
-                        batch, scale, window):
+                        batch, scale, window, _tiled_out=False):
         T = qkv.shape[0]
         S, max_pages = block_tables.shape
         self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
@@ -867,8 +883,8 @@ class HipOps:
         out = self._new((T, nh * D))
         if self._mfma_attention_fits(D, nh // nkv, max_pages, page_size, batch):
             self._attention_mfma(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
-                                 batch, scale, window, out)
-            return out
+                                 batch, scale, window, out, out_rows=T if _tiled_out else 0)
+            return TiledRows(out, (T, nh * D)) if _tiled_out else out
         stride = (nh + 2 * nkv) * D
         first = 0                         # tokens before this one are done
         n_pre, n_pre_tok = batch.num_prefill_seqs, batch.num_prefill_tokens
@@ -920,7 +936,7 @@ class HipOps:
         return key
 
     def _attention_mfma(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables, batch,
-                        scale, window, out):
+                        scale, window, out, out_rows=0):
         lib = self._attention_lib(D)
         self._check(batch.cu_q, torch.int32, (batch.num_seqs + 1,), "cu_q")
         max_pages = block_tables.shape[1]
@@ -955,7 +971,7 @@ class HipOps:
                 part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
                        0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
-                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS)
+                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
@@ -966,7 +982,7 @@ class HipOps:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, 0, _p(out),
-                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0, 0)
+                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0, 0, int(out_rows))
 
     # ------------------------------------------------------------- sampling
     SAMPLE_SLICE = 2048           # logits per workgroup of the two-stage argmax and draw (at most 64 slices)

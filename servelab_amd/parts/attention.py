@@ -88,7 +88,7 @@ class PagedAttention(Mixer):
         qkv = ops.project_qkv(x, self.w_qkv, self.b_qkv, self.num_heads, self.num_kv_heads,
                               self.head_dim, self.rotation, self.position.tables(batch, shared),
                               slots, kc, vc, cache.page_size, q_scale=self.q_scale)
-        attn = ops.paged_attention(
+        return ops.attend_and_project(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
-            cache.page_size, group.block_tables, batch, self.score_scale, self.window)
-        return ops.linear(attn, self.w_o, None, defer=True)
+            cache.page_size, group.block_tables, batch, self.score_scale, self.window,
+            self.w_o, None, defer=True)

@@ -53,6 +53,12 @@ class EmulatedOps:
         g, u = gu[:, :, 0].reshape(T, inter), gu[:, :, 1].reshape(T, inter)
         return (g * torch.sigmoid(g) * u).to(self.act_dtype)
 
+    def attend_and_project(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                           batch, scale, window, w_out, bias=None, defer=False):
+        attn = self.paged_attention(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                                    batch, scale, window)
+        return self.linear(attn, w_out, bias, defer=defer)
+
     def gated_mlp(self, x, w_gate_up, block, w_down, defer=False):
         return self.linear(self.gated_linear(x, w_gate_up, block), w_down, None, defer=defer)
 

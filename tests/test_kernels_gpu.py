@@ -796,6 +796,40 @@ def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window, un
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+@pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 32, 16), (28, 4, 128, 16), (6, 3, 64, 64), (5, 5, 96, 32)])
+@pytest.mark.parametrize("contexts", [(700, 333, 5, 64, 65, 1, 129), (3, 2), (40,) * 16, (2000, 7, 300)])
+def test_attention_and_its_projection_in_one_call(nh, nkv, D, page, contexts):
+    """A step of a few single tokens through attend_and_project: what lies between the attention
+    and the output projection is laid out by k-step (split contexts merged by the combine kernel,
+    short ones written by the attention kernel itself); the result is that of the two calls with a
+    plain tensor between them, bit for bit, finished or left to the norm."""
+    from servelab_amd.kernels import HipOps
+    from servelab_amd.kernels.ops import Deferred, TiledRows
+    dt = torch.bfloat16
+    ops = HipOps(dt, "cuda:0")
+    seqs = [(c, 1) for c in contexts]
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=11)
+    T, H = len(seqs), 160
+    w_o = ops.prepare_weight(randn(H, nh * D, dtype=dt, scale=1.0 / (nh * D) ** 0.5, seed=12))
+    gain = 1 + 0.1 * randn(H, seed=13)
+    resid0 = randn(T, H, seed=14)
+    args = (qkv, nh, nkv, D, kc, vc, page, tables, batch, 1.0 / math.sqrt(D), None)
+    plain = ops.paged_attention(*args)
+    got = {}
+    for tiled in (False, True):
+        ops.tile_few_rows = tiled
+        d = ops.attend_and_project(*args, w_o, None, defer=True)
+        assert isinstance(d, Deferred) and isinstance(d.x, TiledRows) == tiled
+        if tiled:
+            assert torch.equal(d.x.rows(), plain)
+        resid = resid0.clone()
+        scaled = ops.add_rmsnorm(resid, d, gain, 1e-5, fuse=True)
+        got[tiled] = [ops.attend_and_project(*args, w_o, None), ops.materialize(d), resid, scaled.plain_x()]
+    for a, b in zip(got[False], got[True]):
+        assert torch.equal(a, b)
+    assert rel_err(got[True][0], plain.float() @ w_o.w.float().T) < 2 ** -6
+
+
 @pytest.mark.parametrize("D,page", [(16, 16), (32, 16), (128, 32)])
 @pytest.mark.parametrize("q_len", [1, 5])
 @pytest.mark.parametrize("units", UNITS)
