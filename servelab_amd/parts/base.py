@@ -91,7 +91,7 @@ class Norm(Part):
     ``delta`` is what the part before returned: a tensor, or a product the
     kernel table deferred (``ops.linear(..., defer=True)``), which the norm's
     kernel call runs.  ``fuse`` says that the reader of the normed rows passes
-    them only to ``ops.linear`` / ``ops.gated_linear`` (it has
+    them only to ``ops.linear`` / ``ops.gated_linear`` / ``ops.gated_mlp`` (it has
     ``takes_scaled_rows``); the kernel table may then hand it rows whose
     normalisation the reader's product completes."""
 
