@@ -99,13 +99,14 @@ def time_decode(cfg, model, batch, ctx_end, steps, warmup, page, seed=0):
     total = warmup + steps
     budget = 8192
     prompt_len = ctx_end - total - 1
-    prompt_len -= -(-batch * prompt_len // budget) - 1   # the first request decodes while the others prefill
+    prefill_steps = -(-batch * prompt_len // budget)
+    prompt_len -= prefill_steps - 1                      # the first request decodes while the others prefill
     pages = batch * (-(-(ctx_end + 2) // page)) + 16
     engine = LLMEngine(cfg, CacheConfig(block_size=page, num_blocks=pages),
                        SchedulerConfig(max_num_seqs=max(batch, 1), max_num_batched_tokens=budget),
                        model=model)
     gen = torch.Generator().manual_seed(seed)
-    params = SamplingParams(temperature=0.0, max_tokens=total + 64, ignore_eos=True)
+    params = SamplingParams(temperature=0.0, max_tokens=total + prefill_steps + 64, ignore_eos=True)
     for _ in range(batch):
         engine.add_request(prompt_token_ids=torch.randint(0, cfg.vocab_size, (prompt_len,),
                                                           generator=gen).tolist(),

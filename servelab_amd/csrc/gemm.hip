@@ -1093,18 +1093,25 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
     tile_of[t] = live[t] ? tbeg + WAVES * t + wave : (t > 0 && live[0] ? tile_of[0] : tbeg);
     wp[t] = wt + ((size_t)tile_of[t] * KT * 64 + lane) * 8;
   }
-  // this thread's share of a chunk of x: XF fragments (ks, mb, lane) = (idx / (MB * 64), idx / 64 % MB, idx % 64)
+  // This thread's share of a chunk of x: XF fragments of 16 bytes.  A wavefront's load takes 8 rows
+  // and, of each, 8 pieces (two k-steps: a whole 128-byte line; with one k-step a load touched 16
+  // lines and used half of each, and x is a third to a half of what these kernels pull through L1);
+  // lanes 0..7 take the 8 rows of one piece, so that they store to neighbouring places in LDS.
   constexpr int XF = MB * KC * 64 / THREADS;
-  static_assert(XF * THREADS == MB * KC * 64, "a chunk of x must divide evenly over the threads");
+  static_assert(XF * THREADS == MB * KC * 64 && KC % 2 == 0, "a chunk of x must divide evenly over the threads");
   const __bf16* xsrc[XF];
-  int xks[XF];
+  int xks[XF], xmb[XF], xfl[XF];
 #pragma unroll
   for (int j = 0; j < XF; ++j) {
     const int idx = threadIdx.x + THREADS * j;
-    const int fl = idx % 64, mb = idx / 64 % MB;
-    xks[j] = idx / (MB * 64);
-    const int m = 16 * mb + (fl & 15) < M ? 16 * mb + (fl & 15) : M - 1;
-    xsrc[j] = x + (size_t)m * K + 8 * (fl >> 4);
+    const int l = idx % 64, blk = idx / 64;
+    const int r = 8 * (blk % (MB * 2)) + l % 8;           // row of the chunk
+    const int p = 8 * (blk / (MB * 2)) + l / 8;           // piece of the row: k-step p / 4 of the chunk, channels 8 (p % 4)..
+    xks[j] = p / 4;
+    xmb[j] = r / 16;
+    xfl[j] = 16 * (p % 4) + r % 16;                        // the lane whose B operand this is
+    const int m = r < M ? r : M - 1;
+    xsrc[j] = x + (size_t)m * K + 8 * (p % 4);
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   // Every load of the main loop is issued unconditionally (past the end: from
@@ -1120,10 +1127,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_mid_kernel(
   };
   auto store_x = [&](int buf, int c, const bf16x8 (&xr)[XF]) {
 #pragma unroll
-    for (int j = 0; j < XF; ++j) {
-      const int idx = threadIdx.x + THREADS * j;
-      xs[buf][idx / (MB * 64)][idx / 64 % MB][idx % 64] = kbeg + c * KC + xks[j] < kend ? xr[j] : zero;
-    }
+    for (int j = 0; j < XF; ++j)
+      xs[buf][xks[j]][xmb[j]][xfl[j]] = kbeg + c * KC + xks[j] < kend ? xr[j] : zero;
   };
   f32x4 acc[NT][MB];
 #pragma unroll
