@@ -445,11 +445,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 25
 // time at 8,192 tokens, the loads and the writes about equally.)
 //
 // A stage holds K as 32 rows of D / 8 units of 16 bytes, in the order the
-// score product wants its rows (tile m, row i), and then V^T as D rows of 4
-// units.  No padding: a lane can put any unit anywhere at no cost, so the units
+// score product wants its rows (tile m, row i), and then V^T as D / 16 tiles of
+// 64 units.  No padding: a lane can put any unit anywhere at no cost, so the units
 // of K row r are rotated by r % 16 places, which spreads the 16 lanes that read one
-// operand column of a tile (rows r..r+15, same channel) over the banks; V^T's
-// reads cover 1 KB side by side as they are.
+// operand column of a tile (rows r..r+15, same channel) over the banks; the units
+// of V^T lie in the order of the lanes that read them (tile dd: 1 KB, unit 16 q + i =
+// keys 8 q.. of channel 16 dd + i).
 typedef const __attribute__((address_space(4))) int* ConstInts;
 constexpr int SHARED_WAVES = 4;
 constexpr int KU = D / 8;                          // 16-byte units in a row of K
@@ -513,7 +514,8 @@ void attention_mfma_shared_kernel(const AttnParams P) {
 
   // What a lane fetches is fixed for the whole kernel: unit u = 64 chunk + lane of a stage.
   // K unit (row r = 16 m + i, place s) holds channels 8 ((s - i) mod KU) of key
-  // 8 (i / 4) + 4 m + i % 4; V^T unit (row d, place q) holds keys 8 q .. 8 q + 7 of channel d.
+  // 8 (i / 4) + 4 m + i % 4; V^T unit 64 dd + 16 q + i holds keys 8 q .. 8 q + 7 of channel 16 dd + i: the place
+  // of the lane that reads it as its operand of tile dd, so that a read takes 1 KB in the order of the lanes.
   int src[LOADS];                                    // offset inside the page's slice of this kv head, elements
   bool second[LOADS];                                // the unit lies in the second page of the block (16-key pages)
 #pragma unroll
@@ -525,7 +527,7 @@ void attention_mfma_shared_kernel(const AttnParams P) {
       src[i] = (ko & (page - 1)) * D + 8 * c;
       second[i] = ko >= 16;
     } else {
-      const int d = (u - 32 * KU) >> 2, q = u & 3;
+      const int w = (u - 32 * KU) & 63, d = 16 * ((u - 32 * KU) >> 6) + (w & 15), q = w >> 4;
       src[i] = d * page + ((8 * q) & (page - 1));
       second[i] = q >= 2;
     }
@@ -536,7 +538,7 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   int k_at[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) k_at[kk] = 16 * (n * KU + (4 * kk + gq + n) % KU);
-  const int v_at = 16 * 32 * KU + 64 * n + 16 * gq;
+  const int v_at = 16 * 32 * KU + 16 * lane;
 
   auto ring = [&](auto stage) -> char* {
     constexpr int S = decltype(stage)::value;
