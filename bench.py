@@ -97,7 +97,7 @@ def time_decode(cfg, model, batch, ctx_end, steps, warmup, page, seed=0):
     import torch
     from servelab_amd import CacheConfig, LLMEngine, SamplingParams, SchedulerConfig
     total = warmup + steps
-    budget = 8192
+    budget = max(8192, ctx_end)                          # a prompt fits one step, so requests start a step apart
     prompt_len = ctx_end - total - 1
     prefill_steps = -(-batch * prompt_len // budget)
     prompt_len -= prefill_steps - 1                      # the first request decodes while the others prefill

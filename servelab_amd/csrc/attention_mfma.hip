@@ -682,24 +682,37 @@ void attention_mfma_shared_kernel(const AttnParams P) {
 }
 
 // out[row, head, :] = sum_j w_j o_j / sum_j w_j l_j,  w_j = exp(m_j - max m).
-// One wavefront per (row, head); lane j takes split j's (m, l), so nsplit <= 64;
-// then the lanes split the channels and sum the partial outputs with the loads
-// of eight splits in flight at a time.
+// One wavefront per (row, head); lane j takes the (m, l) of splits j, j + 64, ..., so
+// nsplit <= 64 * COMBINE_PER_LANE; then the lanes split the channels and sum the partial
+// outputs with the loads of eight splits in flight at a time.
+constexpr int COMBINE_PER_LANE = 4;
 __global__ __launch_bounds__(64) void attention_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int nsplit, int nh,
     int part_row0, __bf16* __restrict__ out, int out_rows) {
-  __shared__ float ws[64];
+  __shared__ float ws[64 * COMBINE_PER_LANE];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t base = ((size_t)r * nh + h) * nsplit;
-  float m = -INFINITY, l = 0.f;
-  if (lane < nsplit) {
-    m = part_ml[(base + lane) * 2];
-    l = part_ml[(base + lane) * 2 + 1];
+  float m[COMBINE_PER_LANE], l[COMBINE_PER_LANE], top = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < COMBINE_PER_LANE; ++i) {
+    const int j = lane + 64 * i;
+    m[i] = -INFINITY;
+    l[i] = 0.f;
+    if (j < nsplit) {
+      m[i] = part_ml[(base + j) * 2];
+      l[i] = part_ml[(base + j) * 2 + 1];
+    }
+    top = fmaxf(top, m[i]);
   }
-  const float mx = wave_max(m);
-  const float w = m == -INFINITY ? 0.f : fast_exp2(m - mx);     // maxima are in units of log 2
-  const float denom = wave_sum(w * l);
-  ws[lane] = w;
+  const float mx = wave_max(top);
+  float mine = 0.f;
+#pragma unroll
+  for (int i = 0; i < COMBINE_PER_LANE; ++i) {
+    const float w = m[i] == -INFINITY ? 0.f : fast_exp2(m[i] - mx);     // maxima are in units of log 2
+    mine += w * l[i];
+    ws[lane + 64 * i] = w;
+  }
+  const float denom = wave_sum(mine);
   __syncthreads();
   const float inv = 1.f / denom;
   const float* po = part_o + base * D;
@@ -718,6 +731,7 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
   }
 }
 
+extern "C" int sl_attention_mfma_max_splits() { return 64 * COMBINE_PER_LANE; }
 extern "C" int sl_attention_mfma_head_dim() { return D; }
 // whether this head size has the prompt kernel that shares keys through LDS (its buffers fit)
 extern "C" int sl_attention_mfma_shares_keys() { return SHARED_FITS ? 1 : 0; }
@@ -758,7 +772,7 @@ extern "C" const char* sl_attention_mfma(
     SL_CHECK(part_o != nullptr && part_ml != nullptr && part_rows == num_seqs,
              "attention_mfma: a split launch needs partial buffers for its rows");
     SL_CHECK(g <= 64, "attention_mfma: more than 64 query heads per kv head");
-    SL_CHECK(nsplit <= 64, "attention_mfma: at most 64 splits of the context");
+    SL_CHECK(nsplit <= 64 * COMBINE_PER_LANE, "attention_mfma: too many splits of the context");
     const dim3 grid(nsplit, nkv, num_seqs);
     if (fold) {
       if (g <= 16) attention_mfma_kernel<1, true, true, true><<<grid, 64, 0, stream>>>(P);
@@ -787,8 +801,8 @@ extern "C" const char* sl_attention_mfma(
   const bool shared = cols > 16 && SHARED_FITS && tiles * nkv * num_seqs >= shared_min_waves;
   if (nsplit > 1) {
     SL_CHECK(shared && !pair_tiles, "attention_mfma: prompt portions are split only as unpaired tiles through LDS");
-    SL_CHECK(nsplit <= 64 && part_o != nullptr && part_ml != nullptr && part_rows > 0,
-             "attention_mfma: a split launch needs partial buffers for its rows and at most 64 splits");
+    SL_CHECK(nsplit <= 64 * COMBINE_PER_LANE && part_o != nullptr && part_ml != nullptr && part_rows > 0,
+             "attention_mfma: a split launch needs partial buffers for its rows and not too many splits");
   }
   if (cols <= 16) {
     if (fold) attention_mfma_kernel<1, false, true><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);

@@ -976,7 +976,10 @@ class HipOps:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
                 blocks = min(blocks, -(-int(window) // 32) + 1)
-            nsplit = max(1, min(64, blocks // 2, -(-self.TARGET_WAVES // (n_dec * nkv))))
+            # (a few requests with long contexts: up to 256 shares, so that the launch still has TARGET_WAVES
+            # wavefronts; 7B shape, one request at 32,000 tokens: 64 shares leave one wavefront per CU)
+            most = int(self._lib[lib].sl_attention_mfma_max_splits())
+            nsplit = max(1, min(most, blocks // 2, -(-self.TARGET_WAVES // (n_dec * nkv))))
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)

@@ -796,6 +796,31 @@ def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window, un
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+@pytest.mark.parametrize("nh,nkv,D,page", [(28, 4, 128, 16), (8, 1, 64, 32)])
+@pytest.mark.parametrize("contexts", [(9000,), (9000, 5000)])
+def test_decode_attention_with_more_shares_than_lanes(nh, nkv, D, page, contexts):
+    """One or two requests with long contexts are cut into more than 64 shares (141 here, with a launch
+    that aims at 2,048 wavefronts), of which a lane of the merging wavefront takes several; the key that
+    carries the weight of request 0 lies in a late share."""
+    from servelab_amd.kernels import HipOps, Tuning
+    dt = torch.bfloat16
+    ops, emu = HipOps(dt, "cuda:0", tuning=Tuning(target_waves=2048)), EmulatedOps(dt)
+    blocks = -(-max(contexts) // 32)
+    assert min(256, blocks // 2, -(-ops.TARGET_WAVES // (len(contexts) * nkv))) == 141
+    seqs = [(c, 1) for c in contexts]
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=21)
+    at = 8000
+    kc[int(tables[0, at // page]), :, at % page] = 4 * qkv[0, :D].float().sign().to(dt)     # head 0's query picks it
+    qkv, scale = in_units(UNITS[1], qkv, nh, D, 1.0 / math.sqrt(D))
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, None)
+    ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                              types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                       for k, v in vars(batch).items()}), scale, None)
+    assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+    picked = vc[int(tables[0, at // page]), 0, :, at % page].float()
+    assert (got[0, :D].float() - picked).abs().max() < 0.05 * picked.abs().max()
+
+
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 32, 16), (28, 4, 128, 16), (6, 3, 64, 64), (5, 5, 96, 32)])
 @pytest.mark.parametrize("contexts", [(700, 333, 5, 64, 65, 1, 129), (3, 2), (40,) * 16, (2000, 7, 300)])
 def test_attention_and_its_projection_in_one_call(nh, nkv, D, page, contexts):
