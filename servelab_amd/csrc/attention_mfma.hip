@@ -117,15 +117,21 @@ __device__ __forceinline__ size_t out_index(int out_rows, int nh, size_t row, in
 //     s * scale * log2(e) - m, ready for exp2, with no multiply-add per score;
 //   - the sums of the probabilities come from the matrix cores as well (one
 //     more product of P with a tile of ones), not from an add per score;
-//   - a lane compares only its own largest score with the threshold; the
-//     maximum over the lanes of a column is taken only when some lane's has
-//     crossed it and the reference point has to move, which is rare.
+//   - a lane compares only its own largest score with the threshold, and takes
+//     that largest over the scores' bit patterns as integers (v_max3_i32: no
+//     quieting of NaNs around every maximum; above a positive threshold the
+//     order of the patterns is the order of the floats); the maximum over the
+//     lanes of a column is taken only when some lane's has crossed it and the
+//     reference point has to move, which is rare.
 template <int NB, bool FOLD>
 struct Columns {
   int tok[NB], head[NB], pos_c[NB], lo_c[NB];
   bf16x8 qf[NB][KK];
-  float thr[NB];                 // a score (less the reference) above this moves the reference; -inf
-                                 // before the column's first visible key, when there is no reference yet
+  int thr[NB];                   // bit pattern of the score (less the reference) above which the reference moves;
+                                 // UNSET before the column's first visible key, when there is no reference yet:
+                                 // every pattern but that of -0 lies above it, and -0 no score is (the products
+                                 // are added to an accumulator that starts at +0 then)
+  static constexpr int UNSET = -2147483647 - 1;
   f32x4 negm[NB];                // -reference point (units of log 2) in all four entries; 0 before there is one
   f32x4 l_acc[NB];               // sum of the probabilities, every entry the same
   f32x4 o[NB][DD];
@@ -147,7 +153,7 @@ struct Columns {
       const __bf16* q = P.qkv + (size_t)(q0 + tok[b]) * P.row_stride + (size_t)head[b] * D + 8 * gq;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) qf[b][kk] = *(const bf16x8*)(q + 32 * kk);
-      thr[b] = -INFINITY;
+      thr[b] = UNSET;
       negm[b] = f32x4{0.f, 0.f, 0.f, 0.f};
       l_acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -190,9 +196,9 @@ struct Columns {
   }
 
   // From the products to what exp2 takes, with the keys a column does not see
-  // masked out on edge blocks; returns this lane's largest.
-  __device__ __forceinline__ float settle(int b, const f32x4& s0, const f32x4& s1, bool edge, int kbase,
-                                          int gq, float (&s)[8]) const {
+  // masked out on edge blocks; returns the largest of this lane's bit patterns.
+  __device__ __forceinline__ int settle(int b, const f32x4& s0, const f32x4& s1, bool edge, int kbase,
+                                        int gq, float (&s)[8]) const {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float raw = j < 4 ? s0[j] : s1[j - 4];
@@ -205,7 +211,10 @@ struct Columns {
         if (key > pos_c[b] || key < lo_c[b]) s[j] = -INFINITY;
       }
     }
-    return fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    int top = __float_as_int(s[0]);
+#pragma unroll
+    for (int j = 1; j < 8; ++j) top = max(top, __float_as_int(s[j]));
+    return top;
   }
 
   // The reference point of a column moves up to its largest score so far (and
@@ -214,7 +223,8 @@ struct Columns {
   // maximum: until a score exceeds it by LAZY (in units of log 2) it stays, so
   // probabilities reach 2^LAZY at most, far from any overflow, with the same
   // relative rounding, and this path is rare.
-  __device__ __forceinline__ void move(int b, float lane_max, float (&s)[8]) {
+  __device__ __forceinline__ void move(int b, float (&s)[8]) {
+    const float lane_max = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
     const float top = column_max(lane_max) - negm[b][0];          // back in absolute units
     const float m_old = reference(b);
     if (!(top > m_old)) return;
@@ -222,7 +232,7 @@ struct Columns {
     const float shift = -top - negm[b][0];
 #pragma unroll
     for (int j = 0; j < 8; ++j) s[j] += shift;
-    thr[b] = LAZY;
+    thr[b] = __float_as_int(LAZY);
     negm[b] = f32x4{-top, -top, -top, -top};
     l_acc[b] *= alpha;
 #pragma unroll
@@ -230,7 +240,7 @@ struct Columns {
   }
 
   __device__ __forceinline__ float reference(int b) const {
-    return thr[b] == -INFINITY ? -INFINITY : -negm[b][0];
+    return thr[b] == UNSET ? -INFINITY : -negm[b][0];
   }
 
   __device__ __forceinline__ bf16x8 probabilities(const float (&s)[8]) const {
@@ -260,8 +270,8 @@ struct Columns {
       f32x4 s0, s1;
       float s[8];
       scores(b, kf, s0, s1);
-      const float lane_max = settle(b, s0, s1, edge, kbase, gq, s);
-      if (__builtin_expect(__any(lane_max > thr[b]), 0)) move(b, lane_max, s);
+      const int lane_top = settle(b, s0, s1, edge, kbase, gq, s);
+      if (__builtin_expect(__any(lane_top > thr[b]), 0)) move(b, s);
       weigh(b, vf, probabilities(s));
     }
   }
@@ -275,18 +285,18 @@ struct Columns {
     const int kbase = kb * 32;
     const bool edge = kb >= full_end || kb < full_begin;
     f32x4 s0[NB], s1[NB];
-    float s[NB][8], lane_max[NB];
+    float s[NB][8];
     bool crossed = false;
 #pragma unroll
     for (int b = 0; b < NB; ++b) scores(b, kf, s0[b], s1[b]);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      lane_max[b] = settle(b, s0[b], s1[b], edge, kbase, gq, s[b]);
-      crossed = crossed || lane_max[b] > thr[b];
+      const int lane_top = settle(b, s0[b], s1[b], edge, kbase, gq, s[b]);
+      crossed = crossed || lane_top > thr[b];
     }
     if (__builtin_expect(__any(crossed), 0)) {
 #pragma unroll
-      for (int b = 0; b < NB; ++b) move(b, lane_max[b], s[b]);
+      for (int b = 0; b < NB; ++b) move(b, s[b]);
     }
     bf16x8 pb[NB];
     pb[0] = probabilities(s[0]);
