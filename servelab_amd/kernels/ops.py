@@ -935,6 +935,22 @@ class HipOps:
             self._lib[key] = lib
         return key
 
+    def _pair_prompt_tiles(self, tiles, prompts_and_heads) -> bool:
+        """Whether the workgroups of a whole prompt's attention take a late tile of the causal triangle and
+        its early mirror (equal work for all, half as many workgroups) or a tile each, long ones first.
+        Equal workgroups fill the chip in rounds of two per CU, and the last round may be nearly empty;
+        tiles of their own leave the balance to the order in which workgroups start, at the price of
+        twice the prologues.  7B shape, one prompt, pairs against a tile each: 4,096 tokens (448 pairs, one
+        round) 175 against 223 us, 5,120 (560) 335 against 270, 7,168 (784) 546 against 461, 8,192 (896) 615
+        against 572, 10,240 (1,120) 972 against 880, 14,336 (1,568) 1,842 against 1,618, 16,384 (1,792: three
+        and a half rounds) 2,040 either way."""
+        if not self.PAIR_PROMPT_TILES:
+            return False
+        pairs = -(-tiles // 2) * prompts_and_heads
+        slots = 2 * self._num_cus
+        rounds = -(-pairs // slots)
+        return rounds == 1 or pairs >= self.UNPAIRED_BELOW_FILL * rounds * slots
+
     def _attention_mfma(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables, batch,
                         scale, window, out, out_rows=0):
         lib = self._attention_lib(D)
@@ -959,10 +975,11 @@ class HipOps:
                       bool(self._lib[lib].sl_attention_mfma_shares_keys()))
             # tiles of a causal triangle differ in length and are paired; those of a portion
             # that starts deeper in its context than it is long do not
-            pair = batch.max_ctx_len < 2 * batch.max_q_len
+            triangle = batch.max_ctx_len < 2 * batch.max_q_len
+            pair = triangle and self._pair_prompt_tiles(-(-batch.max_q_len * (nh // nkv) // 128), nkv * n_pre)
             # few unpaired tiles over a long context: each is cut into shares of its keys
             nsplit, part_o, part_ml = 1, None, None
-            if shared and not pair:
+            if shared and not triangle:
                 nsplit = max(1, min(self.PROMPT_SPLIT_MAX, batch.max_ctx_len // 32 // self.PROMPT_SPLIT_MIN_BLOCKS,
                                     -(-self.PROMPT_SPLIT_WORKGROUPS // -(-waves // 4)),
                                     self.PROMPT_SPLIT_BYTES // (n_pre_tok * nh * D * 4)))

@@ -67,6 +67,11 @@ class Tuning:
     # workgroups of 64 columns: a wavefront then holds 16 columns and three fit a SIMD
     # (2,048 tokens of the 7B shape: 77 against 88 us)
     narrow_attention_workgroups: int = 400
+    # a workgroup of a whole prompt's launch takes a late tile of the causal triangle and its early mirror,
+    # unless the pairs would fill the chip (two workgroups a CU) in several rounds, the last of them
+    # mostly empty: below this share of the slots of all rounds, every tile gets a workgroup of its own
+    pair_prompt_tiles: bool = True
+    unpaired_below_fill: float = 0.9
 
     def apply(self, table) -> None:
         """Sets every field on ``table`` under its upper-case name."""

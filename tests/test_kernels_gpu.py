@@ -719,19 +719,21 @@ def test_paged_attention(both, nh, nkv, D, page, window, units):
                                            (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16),
                                            (4, 2, 256, 16)])     # 256: no LDS form; the same calls take the other kernel
 @pytest.mark.parametrize("window", [None, 16, 50])
-@pytest.mark.parametrize("form", ["paired", "unpaired", "shares"])
+@pytest.mark.parametrize("form", ["paired", "a tile each", "unpaired", "shares"])
 @pytest.mark.parametrize("units", UNITS)
 def test_prompt_attention_through_lds(nh, nkv, D, page, window, form, units):
     """The prompt kernel whose wavefronts share each block of keys through LDS,
     forced at sizes far below its crossover: portions that end inside a
     workgroup's 128 columns, that start deep in a context, and one-token rows;
-    whole prompts with late and early tiles paired in a workgroup; tiles cut
-    into shares of their keys (down to one block, some shares empty)."""
-    from servelab_amd.kernels import HipOps
+    whole prompts with late and early tiles paired in a workgroup, and with a
+    workgroup for every tile (what launches of two or three uneven rounds of
+    pairs take); tiles cut into shares of their keys (down to one block, some
+    shares empty)."""
+    from servelab_amd.kernels import HipOps, Tuning
     dt = torch.bfloat16
-    ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+    ops, emu = HipOps(dt, "cuda:0", tuning=Tuning(pair_prompt_tiles=form != "a tile each")), EmulatedOps(dt)
     ops.SHARED_ATTENTION_MIN_CONTEXT = ops.SHARED_ATTENTION_MIN_WAVES = 0
-    if form == "paired":
+    if form in ("paired", "a tile each"):
         seqs = [(130, 130), (64, 64), (97, 97), (333, 333), (2, 2), (1, 1)]
     else:
         seqs = [(130, 130), (277, 45), (64, 64), (200, 2), (333, 97), (16, 1), (145, 1)]
@@ -745,6 +747,19 @@ def test_prompt_attention_through_lds(nh, nkv, D, page, window, form, units):
                                                        for k, v in vars(batch).items()}),
                               scale, window)
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+
+
+def test_whole_prompts_pair_their_tiles_unless_the_rounds_are_uneven():
+    """The choice between a late tile with its early mirror per workgroup and a workgroup per tile, at the
+    sizes it was measured at (7B shape: 7 columns a token, 4 kv heads, 256 CUs)."""
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.bfloat16, "cuda:0")
+    ops._num_cus = 256
+    paired = {T: ops._pair_prompt_tiles(-(-T * 7 // 128), 4) for T in (2048, 4096, 4608, 5120, 8192, 14336, 32768)}
+    assert paired == {2048: True, 4096: True, 4608: True, 5120: False, 8192: False, 14336: False, 32768: True}
+    assert ops._pair_prompt_tiles(-(-4096 * 7 // 128), 4 * 8)          # eight prompts of 4,096: seven full rounds
+    ops.PAIR_PROMPT_TILES = False
+    assert not ops._pair_prompt_tiles(10, 4)
 
 
 @pytest.mark.parametrize("units", UNITS)
