@@ -367,6 +367,11 @@ struct NormFusion {
   // for the product that reads it (x_tiled: the number of rows M the tensor was written with, 0 = plain rows).
   int x_tiled;
   int y_tiled;
+  // PRODUCER: rows of W per tile, 8..16 and even (W then lies as [ceil(N / th)][K / 32][4][th][8], see
+  // sl_tile_weight).  A product of few rows takes as long as its busiest CU needs to pull its tiles of W
+  // and its re-read of x, so a matrix whose 16-row tiles do not go round the CUs evenly gets lower tiles
+  // that do (N = 3584 on 256 CUs: 256 tiles of 14 rows instead of 224 of 16).  Other forms: 16.
+  int th;
 };
 
 // Rotary embedding and the write to the cache pages fused into the q/k/v
@@ -407,14 +412,16 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
   // condition the compiler takes for divergent and may turn into masking
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int lane = threadIdx.x % 64, i = lane & 15, gq = lane >> 4;
-  const int ntiles = (N + 15) / 16;
+  const int th = PRODUCER ? F.th : 16;
+  const int ntiles = (N + th - 1) / th;
   const int KT = K / 32;
   const int ks0 = (int)((long long)KT * wave / WAVES), ks1 = (int)((long long)KT * (wave + 1) / WAVES);
   const __bf16* wp[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const int tile = blockIdx.x * NT + t < ntiles ? blockIdx.x * NT + t : ntiles - 1;
-    wp[t] = wt + ((size_t)tile * KT * 64 + lane) * 8;
+    // (lanes of rows a lower tile does not have read its last row; their columns of the result are dropped)
+    wp[t] = wt + ((size_t)tile * KT * (4 * th) + gq * th + (i < th ? i : th - 1)) * 8;
   }
   int xrow = i < M ? i : M - 1;
   if (CONSUMER && F.rows != nullptr) xrow = F.rows[xrow];
@@ -436,9 +443,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
   float r_old[NT], g_next[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int en = (blockIdx.x * NT + t) * 16 + threadIdx.x % 16;
+    const int en = (blockIdx.x * NT + t) * th + threadIdx.x % 16;
     r_old[t] = g_next[t] = 0.f;
-    if (PRODUCER && threadIdx.x < 256 && em < M && en < N) {
+    if (PRODUCER && threadIdx.x < 256 && em < M && (int)(threadIdx.x % 16) < th && en < N) {
       r_old[t] = F.resid[(size_t)em * N + en];
       g_next[t] = F.next_w[en];
     }
@@ -470,15 +477,16 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
   for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   // The K loop, written once for plain rows of x (a constant step from one k-step to the next,
   // folded into the loads' offsets) and once for rows laid out by k-step.
-  auto stream_k = [&](auto tiled_tag) {
+  auto stream_k = [&](auto tiled_tag, auto th_tag) {
     const size_t xs_ = decltype(tiled_tag)::value ? xstep : (size_t)32;
+    constexpr size_t WS = 32 * decltype(th_tag)::value;             // elements of W from one k-step of a tile to the next
     int ks = ks0;
     for (; ks + U <= ks1; ks += U) {
       bf16x8 a[NT][U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
+        for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + WS * (size_t)(ks + u));
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const bf16x8 bv = *(const bf16x8*)(xp + xs_ * (size_t)(ks + u));
@@ -495,7 +503,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
       for (int u = 0; u < U - 1; ++u)
         if (ks + u < ks1) {
 #pragma unroll
-          for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + 512 * (size_t)(ks + u));
+          for (int t = 0; t < NT; ++t) a[t][u] = stream_load(wp[t] + WS * (size_t)(ks + u));
           bv[u] = *(const bf16x8*)(xp + xs_ * (size_t)(ks + u));
         }
 #pragma unroll
@@ -507,8 +515,21 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
         }
     }
   };
-  if (F.x_tiled) stream_k(std::true_type{});
-  else stream_k(std::false_type{});
+  // (each form of the loop is straight-line code with constant steps; the tile height is a run-time
+  // choice only for producers)
+  auto stream_th = [&](auto th_tag) {
+    if (F.x_tiled) stream_k(std::true_type{}, th_tag);
+    else stream_k(std::false_type{}, th_tag);
+  };
+  if constexpr (!PRODUCER) {
+    stream_th(std::integral_constant<int, 16>{});
+  } else {
+    if (th == 16) stream_th(std::integral_constant<int, 16>{});
+    else if (th == 14) stream_th(std::integral_constant<int, 14>{});
+    else if (th == 12) stream_th(std::integral_constant<int, 12>{});
+    else if (th == 10) stream_th(std::integral_constant<int, 10>{});
+    else stream_th(std::integral_constant<int, 8>{});
+  }
 #pragma unroll
   for (int t = 0; t < NT; ++t) red[t][wave][lane] = acc[t];
   if (CONSUMER) {            // this wavefront's share of the sums of squares, by row
@@ -531,7 +552,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
   for (int t = 0; t < NT; ++t) {
     const int tile = blockIdx.x * NT + t;
     if (tile >= ntiles) break;
-    const int n0 = tile * 16;
+    const int n0 = tile * th;
     // lane (m + 16 (n_local / 4)) holds y[m, n_local] in element n_local % 4
     if (GATED) {
       if (threadIdx.x < 128) {
@@ -557,7 +578,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
     }
     if (threadIdx.x < 256) {
       const int m = em, n_local = threadIdx.x % 16, n = n0 + n_local;
-      const bool live = m < M && n < N;
+      const bool live = m < M && n_local < th && n < N;
       float s = 0.f;
 #pragma unroll
       for (int wv = 0; wv < WAVES; ++wv) s += red[t][wv][m + 16 * (n_local / 4)][n_local % 4];
@@ -616,13 +637,14 @@ static int device_cus() {
 // wt: W in the tiled layout, ceil(N / 16) * 16 rows (rows beyond N are zero).
 // At most 16 rows.  Fusion: in_parts != nullptr makes x un-normalised rows
 // (consumer), resid != nullptr makes the result a delta of the stream (producer).
-// pair_tiles: two tiles of W per workgroup.
+// pair_tiles: two tiles of W per workgroup.  th: rows of W per tile (16, or what sl_tile_weight was given
+// for a producer's matrix).
 extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float* bias, void* y,
                                       int M, int N, int K, int out_f32, int gated,
                                       const float* in_parts, int in_nparts, float eps,
                                       const int* rows, float* resid, const float* next_w,
                                       float* out_parts, const RopeStore* rope, int pair_tiles,
-                                      int x_tiled, int y_tiled, hipStream_t stream) {
+                                      int x_tiled, int y_tiled, int th, hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
   SL_CHECK(M <= 16, "gemm_skinny: at most 16 rows");
   SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
@@ -638,15 +660,17 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
   SL_CHECK(rows == nullptr || consumer, "gemm_skinny: a row gather belongs to a consumer");
   SL_CHECK(!producer || (next_w != nullptr && out_parts != nullptr && !gated && !out_f32),
            "gemm_skinny: a producer needs the next gain and a parts buffer, and is neither gated nor float");
+  SL_CHECK(th == 16 || (producer && th >= 8 && th < 16 && th % 2 == 0),
+           "gemm_skinny: tiles of 16 rows, or of 8, 10, 12 or 14 for a producer");
   if (M == 0) return nullptr;
-  const dim3 grid((N + 15) / 16);
+  const dim3 grid((N + th - 1) / th);
   const __bf16* xx = (const __bf16*)x;
   const __bf16* ww = (const __bf16*)wt;
   SL_CHECK(x_tiled >= 0 && (x_tiled == 0 || rows != nullptr || x_tiled == M),
            "gemm_skinny: x tiled by k-step has as many rows as the product, or rows are picked from it");
   SL_CHECK(!y_tiled || (gated && (N / 2) % 32 == 0) || (resid != nullptr && N % 32 == 0),
            "gemm_skinny: a tiled result is a gated one or a producer's, of a multiple of 32 columns");
-  const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts, x_tiled, y_tiled};
+  const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts, x_tiled, y_tiled, th};
   const bool few = in_nparts <= 32 * 8;
   if (rope != nullptr) {
     const RopeStore R = *rope;
@@ -672,7 +696,7 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
   }
   const RopeStore none{};
   if (pair_tiles) {                              // two tiles per workgroup
-    const dim3 grid2(((N + 15) / 16 + 1) / 2);
+    const dim3 grid2((grid.x + 1) / 2);
     if (producer) gemm_skinny_kernel<false, false, true, 1, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
     else if (consumer && gated && few) gemm_skinny_kernel<true, true, false, 8, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
     else if (consumer && gated) gemm_skinny_kernel<true, true, false, 16, false, 2><<<grid2, 512, 0, stream>>>(xx, ww, bias, y, M, N, K, 0, F, none);
@@ -852,7 +876,8 @@ extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const flo
   const __bf16* ww = (const __bf16*)wt;
 #define SL_RESIDENT(G, NS, R)                                                                   \
   do {                                                                                          \
-    constexpr int PARTS = NS <= 16 ? 8 : 16;          /* K / 16 parts, 32 per pass */           \
+    constexpr int PARTS = NS <= 16 ? 8 : 16;          /* K / 16 parts or more, 32 per pass */   \
+    SL_CHECK(in_nparts <= 32 * PARTS, "gemm_resident: more sums of squares a row than this form adds up"); \
     static int slots = 0;                                                                       \
     if (slots == 0) slots = resident_workgroups(gemm_resident_kernel<G, PARTS, NS, R>);         \
     SL_CHECK(slots > 0, "gemm_resident: the device holds no workgroup of this kernel");         \
@@ -1386,37 +1411,40 @@ extern "C" const char* sl_splitk_reduce(const float* part, const float* bias, vo
   return sl_launch_status();
 }
 
-// Row-major W [N, K] -> tiled [ceil(N / 16)][K / 32][64][8]; rows beyond N are zero.
+// Row-major W [N, K] -> tiled [ceil(N / th)][K / 32][4][th][8] (th = 16: [..][64][8], the matrix
+// instruction's A operand as it sits in registers); rows beyond N are zero.
 __global__ void tile_weight_kernel(const __bf16* __restrict__ w, __bf16* __restrict__ wt, int N,
-                                   int K, size_t total_vec) {
+                                   int K, int th, size_t total_vec) {
   const int KT = K / 32;
   for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec;
        v += (size_t)gridDim.x * blockDim.x) {
-    const int lane = (int)(v % 64);
-    const size_t t = v / 64;
+    const int at = (int)(v % (4 * th));                  // place inside the tile's k-step: quarter of k, row
+    const size_t t = v / (4 * th);
     const int ks = (int)(t % KT);
     const size_t tile = t / KT;
-    const size_t n = tile * 16 + (lane & 15);
-    const int k = ks * 32 + 8 * (lane >> 4);
+    const size_t n = tile * th + at % th;
+    const int k = ks * 32 + 8 * (at / th);
     bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
     if (n < (size_t)N) val = *(const bf16x8*)(w + n * K + k);
     *(bf16x8*)(wt + v * 8) = val;
   }
 }
 
-extern "C" const char* sl_tile_weight(const void* w, void* wt, int N, int K, hipStream_t stream) {
+// wt: ceil(N / th) * th * K elements.
+extern "C" const char* sl_tile_weight(const void* w, void* wt, int N, int K, int th, hipStream_t stream) {
   SL_CHECK(N > 0 && K > 0 && K % 32 == 0, "tile_weight: K must be a positive multiple of 32");
+  SL_CHECK(th >= 8 && th <= 16 && th % 2 == 0, "tile_weight: tiles of 8, 10, 12, 14 or 16 rows");
   SL_CHECK(((uintptr_t)w % 16) == 0 && ((uintptr_t)wt % 16) == 0, "tile_weight: 16-byte alignment");
-  const size_t total_vec = (size_t)((N + 15) / 16) * (K / 32) * 64;
+  const size_t total_vec = (size_t)((N + th - 1) / th) * (K / 32) * 4 * th;
   const size_t blocks = (total_vec + 255) / 256;
   tile_weight_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>(
-      (const __bf16*)w, (__bf16*)wt, N, K, total_vec);
+      (const __bf16*)w, (__bf16*)wt, N, K, th, total_vec);
   return sl_launch_status();
 }
 // Tiled -> row-major [N, K] (the inverse), for products with many rows when only
 // the tiled copy is kept.
 __global__ void untile_weight_kernel(const __bf16* __restrict__ wt, __bf16* __restrict__ w, int N,
-                                     int K, size_t total_vec) {
+                                     int K, int th, size_t total_vec) {
   const int KT = K / 32;
   for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec;
        v += (size_t)gridDim.x * blockDim.x) {
@@ -1424,18 +1452,19 @@ __global__ void untile_weight_kernel(const __bf16* __restrict__ wt, __bf16* __re
     const size_t n = v / (K / 8);
     const int k8 = (int)(v % (K / 8));
     const int ks = k8 / 4, gq = k8 % 4;
-    const size_t src = (((n / 16) * KT + ks) * 64 + 16 * gq + (n % 16)) * 8;
+    const size_t src = (((n / th) * KT + ks) * (4 * th) + gq * th + (n % th)) * 8;
     *(bf16x8*)(w + v * 8) = *(const bf16x8*)(wt + src);
   }
 }
 
-extern "C" const char* sl_untile_weight(const void* wt, void* w, int N, int K, hipStream_t stream) {
+extern "C" const char* sl_untile_weight(const void* wt, void* w, int N, int K, int th, hipStream_t stream) {
   SL_CHECK(N > 0 && K > 0 && K % 32 == 0, "untile_weight: K must be a positive multiple of 32");
+  SL_CHECK(th >= 8 && th <= 16 && th % 2 == 0, "untile_weight: tiles of 8, 10, 12, 14 or 16 rows");
   SL_CHECK(((uintptr_t)w % 16) == 0 && ((uintptr_t)wt % 16) == 0, "untile_weight: 16-byte alignment");
   const size_t total_vec = (size_t)N * (K / 8);
   const size_t blocks = (total_vec + 255) / 256;
   untile_weight_kernel<<<(unsigned)(blocks < 262144 ? blocks : 262144), 256, 0, stream>>>(
-      (const __bf16*)wt, (__bf16*)w, N, K, total_vec);
+      (const __bf16*)wt, (__bf16*)w, N, K, th, total_vec);
   return sl_launch_status();
 }
 #endif

@@ -62,12 +62,15 @@ class RotationPlan:
 class LinearWeight:
     """A weight matrix [N, K] as the products read it: row-major (``w``) for
     products with many rows, tiled (``tiled``, bfloat16 only) for the few-rows
-    kernels that decode steps use.  Both, or one of them."""
-    __slots__ = ("w", "tiled", "shape")
+    kernels that decode steps use.  Both, or one of them.  ``lower``: a further
+    tiled copy in tiles of ``th`` < 16 rows, for the few-rows product that adds
+    to the residual stream (see ``HipOps.producer_tile_height``)."""
+    __slots__ = ("w", "tiled", "shape", "lower", "th", "lower_from")
 
     def __init__(self, w, tiled=None, shape=None):
         self.w, self.tiled = w, tiled
         self.shape = tuple(w.shape) if w is not None else tuple(shape)
+        self.lower, self.th, self.lower_from = None, 16, 1          # lower_from: rows from which ``lower`` is read
 
 
 class Deferred:
@@ -173,6 +176,7 @@ class HipOps:
         self.fuse_rope = act_dtype == torch.bfloat16
         self.tile_few_rows = act_dtype == torch.bfloat16      # gated_mlp keeps few rows tiled by k-step
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
+        self.lower_tiles = act_dtype == torch.bfloat16        # see plan_weights
         self._untiled = None          # scratch for "tiled": the row-major form of one matrix
         # Up to this many rows no product of a prepared weight goes to the library
         # (whose kernels may record memsets, which HIP graphs replay wrongly here):
@@ -207,7 +211,7 @@ class HipOps:
     def _new(self, shape, dtype=None):
         return torch.empty(shape, dtype=dtype or self.act_dtype, device=self.device)
 
-    def _pair_tiles(self, M, N, K) -> bool:
+    def _pair_tiles(self, M, N, K, th=16) -> bool:
         """Whether a few-rows product gives its workgroups two tiles of W (16
         rows each) instead of one.  Two tiles share one pass over x; these
         kernels are bound by what the busiest CU has to pull through its L1
@@ -217,10 +221,10 @@ class HipOps:
         two forms measured within a few per cent of each other on the 7B, 32B
         and 72B shapes (pairs lose 7 % where K = 8192), so one tile stays; at 16
         rows pairs gain 15-25 % on the large matrices."""
-        tiles = -(-N // 16)
+        tiles = -(-N // th)
         if tiles < 2 or M <= 8:
             return False
-        w, x = 16 * K, min(M, 16) * K                     # bytes / 2 of a tile of W and of x
+        w, x = th * K, min(M, 16) * K                     # bytes / 2 of a tile of W and of x
         one = -(-tiles // self._num_cus) * (w + x)
         two = -(-(-(-tiles // 2)) // self._num_cus) * (2 * w + x)
         return two < 0.97 * one
@@ -232,12 +236,14 @@ class HipOps:
         x_tiled = scaled.tiled if scaled is not None else 0
         if isinstance(x, TiledRows):
             x_tiled, x = x.shape[0], x.data
-        self._call("gemm", "sl_gemm_skinny", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
+        # (the product that adds to the stream reads the copy in lower tiles, where the matrix has one)
+        wt, th = self._producer_copy(weight, M) if resid is not None else (weight.tiled, 16)
+        self._call("gemm", "sl_gemm_skinny", _p(x), _p(wt), _p(bias), _p(y), M, N, K,
                    int(out_f32), int(gated), _p(parts), parts.shape[0] if parts is not None else 0,
                    _c_float(scaled.eps if scaled is not None else 0.0),
                    _p(scaled.rows) if scaled is not None else None, _p(resid), _p(next_gain),
                    _p(out_parts), ctypes.byref(rope) if rope is not None else None,
-                   int(self._pair_tiles(M, N, K)), int(x_tiled), int(y_tiled))
+                   int(self._pair_tiles(M, N, K, th)), int(x_tiled), int(y_tiled), th)
 
     # ------------------------------------------------------------ embedding
     def embed(self, ids, table):
@@ -318,7 +324,8 @@ class HipOps:
         if d.bias is not None:
             self._check(d.bias, torch.float32, (N,), "bias")
         out = self._new((M, N))
-        parts = self._new((-(-N // 16), 16), torch.float32)
+        th = self._producer_copy(weight, M)[1]
+        parts = self._new((-(-N // th), 16), torch.float32)
         tiled = M if self.tile_few_rows and M > 1 and N % 32 == 0 else 0     # for the products that read the rows
         self._skinny(x, weight, d.bias, out, M, N, K, resid=resid, next_gain=gain, out_parts=parts,
                      y_tiled=bool(tiled))
@@ -331,12 +338,47 @@ class HipOps:
         if self.act_dtype == torch.bfloat16:
             total = torch.cuda.get_device_properties(self.device).total_memory
             self.weight_layout = "dual" if 2 * total_bytes <= self.DUAL_MEMORY_SHARE * total else "tiled"
+            # a third copy of the matrices that add to the stream (about a third of all), in lower tiles
+            self.lower_tiles = self.weight_layout == "dual" and 2.35 * total_bytes <= self.LOWER_TILES_MEMORY_SHARE * total
         return self.weight_layout
 
-    def prepare_weight(self, w, keep_rows=False):
+    def producer_tile_height(self, N, K, rows=8):
+        """(rows per tile, rows of x from which it pays) for the few-rows product of an [N, K] matrix that
+        adds to the residual stream.  At 8 rows and more such a product takes as long as its busiest CU needs
+        to pull its tiles of W and its re-read of x, so the tiles should go round the CUs evenly: of 16, 14,
+        12, 10 and 8 rows the height is taken whose busiest CU pulls least; 16 unless another saves
+        LOWER_TILES_MIN_GAIN of it.  Measured on MI355X (us at 1 / 4 / 8 / 16 rows, tiles of 16 against the
+        choice): 3584 x 18944, 14 rows (256 tiles on 256 CUs instead of 224): 23.8 / 25.7 / 29.4 / 38.6 against
+        25.8 / 26.2 / 28.0 / 33.8; 5120 x 27648, 10 rows (512 tiles instead of 320, two on a quarter of the
+        CUs): 57.6 / 61.2 / 68.9 against 54.1 / 52.6 / 56.1; 2048 x 11008, 8 rows (256 tiles instead of 128):
+        12.3 / 13.5 / 15.5 against 12.1 / 12.6 / 13.7.  Where the busiest CU pulls less W (fewer rounds, or
+        idle CUs put to work at half the tile) the lower tiles win from one row on; where only the re-read
+        of x per tile of W shrinks (3584), from 8 rows on: below, HBM is the limit, and it streams tiles of
+        1 KB a k-step a little faster.  (Timed with x in plain rows; with x laid out by k-step, as the engine
+        hands it over, the 3584 case gains nothing end to end, which is why the default minimum gain leaves
+        it at 16 rows.)"""
+        def busiest(th, x):
+            return -(-(-(-N // th)) // self._num_cus) * (th + x)
+        # (a tile is one sum of squares a row for the products that read the stream next: the kernel that keeps
+        # x in registers adds up 256 of them, 512 for rows of more than 4,096 values, as the others do)
+        most = 256 if N <= 4096 else 512
+        heights = [th for th in (16, 14, 12, 10, 8) if th == 16 or -(-N // th) <= most]
+        best = min(heights, key=lambda th: (busiest(th, rows), -th))
+        if busiest(best, rows) > (1 - self.LOWER_TILES_MIN_GAIN) * busiest(16, rows):
+            return 16, 1
+        return best, (1 if busiest(best, 0) <= 0.8 * busiest(16, 0) else 8)
+
+    def _producer_copy(self, weight, M):
+        """(tiled copy, its tile height) that the product adding ``M`` rows to the stream reads."""
+        if weight.lower is not None and M >= weight.lower_from:
+            return weight.lower, weight.th
+        return weight.tiled, 16
+
+    def prepare_weight(self, w, keep_rows=False, residual_delta=False, _th=None):
         """Called once per matrix at load: returns what ``linear`` takes.
         ``keep_rows``: the caller holds the row-major tensor anyway (a tied
-        embedding table), so keeping it costs nothing."""
+        embedding table), so keeping it costs nothing.  ``residual_delta``: the
+        matrix's products are only ever added to the residual stream."""
         N, K = w.shape
         self._check(w, self.act_dtype, None, "weight")
         if self.act_dtype != torch.bfloat16:
@@ -345,11 +387,17 @@ class HipOps:
             self.graph_rows_limit = min(self.graph_rows_limit, self.ROWS_KERNEL_MAX_M)
             return LinearWeight(w)
         tiled = torch.empty(-(-N // 16) * 16 * K, dtype=torch.bfloat16, device=self.device)
-        self._call("gemm", "sl_tile_weight", _p(w), _p(tiled), N, K)
+        self._call("gemm", "sl_tile_weight", _p(w), _p(tiled), N, K, 16)
         if self.weight_layout == "tiled" and not keep_rows:
             weight = LinearWeight(None, tiled, (N, K))
         else:
             weight = LinearWeight(w, tiled)
+        if residual_delta and self.fuse_norms and self.lower_tiles:
+            th, lower_from = (_th, 1) if _th is not None else self.producer_tile_height(N, K)
+            if th != 16:
+                weight.lower = torch.empty(-(-N // th) * th * K, dtype=torch.bfloat16, device=self.device)
+                weight.th, weight.lower_from = th, lower_from
+                self._call("gemm", "sl_tile_weight", _p(w), _p(weight.lower), N, K, th)
         self.graph_rows_limit = min(self.graph_rows_limit, self._few_rows_limit(weight))
         return weight
 
@@ -363,7 +411,7 @@ class HipOps:
             self._untiled = None
             self._untiled = torch.empty(N * K, dtype=torch.bfloat16, device=self.device)
         out = self._untiled[:N * K].view(N, K)
-        self._call("gemm", "sl_untile_weight", _p(weight.tiled), _p(out), N, K)
+        self._call("gemm", "sl_untile_weight", _p(weight.tiled), _p(out), N, K, 16)
         return out
 
     FUSED_NORM_MAX_M = 16         # the fused add + norm lives in the kernel for up to 16 rows
@@ -505,7 +553,7 @@ class HipOps:
         if bias is not None:
             self._check(bias, torch.float32, (N,), "bias")
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
-        if self._takes_resident(N, K):
+        if self._takes_resident(N, K) and xs.parts.shape[0] <= 32 * (8 if K <= 4096 else 16):
             self._call("gemm", "sl_gemm_resident", _p(xs.x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                        int(out_f32), int(gated), _p(xs.parts), xs.parts.shape[0], _c_float(xs.eps),
                        _p(xs.rows), int(xs.tiled), int(y_tiled))

@@ -17,6 +17,13 @@ class Tuning:
     # both copies of a matrix (row-major for the library, tiled for the few-rows kernels) are kept
     # while they stay below this share of the device's memory; beyond it only the tiled copy
     dual_memory_share: float = 0.45
+    # the matrices whose few-rows products add to the residual stream get a further copy in tiles of fewer
+    # than 16 rows where those go round the CUs more evenly (HipOps.producer_tile_height), while all copies
+    # stay below this share of the device's memory and the busiest CU pulls at least min_gain less (32B shape,
+    # 5120 columns, 512 tiles of 10 rows for 320 of 16: a quarter less, +6 % tokens/s at batch 8, +2 % at batch 1;
+    # 7B shape, 3584 columns, 256 tiles of 14 for 224 of 16: a twelfth less and nothing gained end to end)
+    lower_tiles_memory_share: float = 0.55
+    lower_tiles_min_gain: float = 0.15
 
     # ---- products of 17 and more rows over the tiled copy
     # from this many rows on two tiles of W share one read of x (gemm_wide / gemm_mid)

@@ -75,7 +75,7 @@ class PagedAttention(Mixer):
                 [reorder(tensors("q_proj.bias").float(), self.num_heads),
                  reorder(tensors("k_proj.bias").float(), self.num_kv_heads),
                  tensors("v_proj.bias").float()], 0))
-        self.w_o = rt.linear_weight(tensors("o_proj.weight"))
+        self.w_o = rt.linear_weight(tensors("o_proj.weight"), delta=True)
         # a kernel table may want part of the score scale applied to q where q is made
         split = getattr(rt.ops, "split_attention_scale", None)
         self.q_scale, self.score_scale = split(self.scale) if split is not None else (1.0, self.scale)

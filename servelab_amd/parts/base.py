@@ -47,12 +47,13 @@ class Runtime:
         """A matrix or table in the activation dtype, on the device."""
         return t.to(device=self.device, dtype=self.act_dtype).contiguous()
 
-    def linear_weight(self, t: torch.Tensor, shared: bool = False):
+    def linear_weight(self, t: torch.Tensor, shared: bool = False, delta: bool = False):
         """A matrix that only ``ops.linear`` reads, in whatever form the kernel
-        table wants it.  ``shared``: another part keeps ``t`` itself as well."""
+        table wants it.  ``shared``: another part keeps ``t`` itself as well.
+        ``delta``: its products are only ever added to the residual stream."""
         m = self.matrix(t)
         prepare = getattr(self.ops, "prepare_weight", None)
-        return prepare(m, keep_rows=shared) if prepare is not None else m
+        return prepare(m, keep_rows=shared, residual_delta=delta) if prepare is not None else m
 
     def vector(self, t: torch.Tensor) -> torch.Tensor:
         """A gain or bias: always float32 on the device (they enter float32 math)."""

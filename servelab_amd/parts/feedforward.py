@@ -37,7 +37,7 @@ class GatedMLP(FeedForward):
         b = self.block
         self.w_gate_up = rt.linear_weight(torch.stack(
             [gate.reshape(i // b, b, h), up.reshape(i // b, b, h)], 1).reshape(2 * i, h))
-        self.w_down = rt.linear_weight(tensors("down_proj.weight"))
+        self.w_down = rt.linear_weight(tensors("down_proj.weight"), delta=True)
 
     def forward(self, x):
         ops = self.rt.ops

@@ -163,7 +163,7 @@ def test_linear_skinny(M, N, K, pairs):
     from servelab_amd.kernels import HipOps
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
     if pairs:
-        ops._pair_tiles = lambda M, N, K: True
+        ops._pair_tiles = lambda M, N, K, th=16: True
     x = randn(M, K, dtype=torch.bfloat16, seed=4)
     w = randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5)
     b = randn(N, seed=6)
@@ -275,7 +275,7 @@ def test_gated_linear(both, M, I, K, pairs):
             pytest.skip("tiles of W are a matter of the bfloat16 kernels")
         from servelab_amd.kernels import HipOps
         ops = HipOps(dt, "cuda:0")
-        ops._pair_tiles = lambda M, N, K: True
+        ops._pair_tiles = lambda M, N, K, th=16: True
     x = randn(M, K, dtype=dt, seed=1)
     gate, up = randn(I, K, dtype=dt, scale=0.2, seed=2), randn(I, K, dtype=dt, scale=0.2, seed=3)
     ref = emu.silu_mul(emu.linear(x, torch.cat([gate, up]), None))
@@ -291,20 +291,26 @@ def test_gated_linear(both, M, I, K, pairs):
 
 @pytest.mark.parametrize("M,H,N2", [(1, 64, 96), (8, 3584, 4608), (16, 200 * 32, 48), (5, 96, 1000)])
 @pytest.mark.parametrize("pairs", [False, True])
-def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs):
+@pytest.mark.parametrize("th", [16, 14, 10, 8])
+def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs, th):
     """A deferred product run by the norm that adds it (stream += x W1^T, rows
     left un-normalised, sums of squares by workgroup) and the products that
     read such rows (plain with bias, gated, float output with a row gather):
     same results as product, add, norm and product one after the other; with
-    one tile of W per workgroup and with two."""
+    one tile of W per workgroup and with two; with the first matrix in tiles
+    of 16 rows and in a further copy of lower tiles (the last tile partly empty)."""
     from servelab_amd.kernels import HipOps
     from servelab_amd.kernels.ops import Deferred, ScaledRows
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
     if pairs:
-        ops._pair_tiles = lambda M, N, K: True
+        ops._pair_tiles = lambda M, N, K, th=16: True
     K1 = 128 if H != 3584 else 4160       # (the long one: 224 tiles, sixteen wavefronts a workgroup)
     x = randn(M, K1, dtype=torch.bfloat16, seed=1)
-    w1 = ops.prepare_weight(randn(H, K1, dtype=torch.bfloat16, scale=0.1 * (128 / K1) ** 0.5, seed=2))
+    if -(-H // th) > 512:
+        pytest.skip("more tiles than the readers of the stream add up sums of squares for")
+    w1 = ops.prepare_weight(randn(H, K1, dtype=torch.bfloat16, scale=0.1 * (128 / K1) ** 0.5, seed=2),
+                            residual_delta=th != 16, _th=th)
+    assert (w1.lower is None) == (th == 16) and ops._producer_copy(w1, M)[1] == th
     gain = 1 + 0.1 * randn(H, seed=3)
     resid0 = randn(M, H, seed=4)
     eps = 1e-5
@@ -338,6 +344,42 @@ def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs):
     # more rows than the fused kernels take: the product is simply done
     big = randn(17, K1, dtype=torch.bfloat16, seed=7)
     assert torch.is_tensor(ops.linear(big, w1, None, defer=True))
+
+
+def test_lower_tiles_for_the_products_that_add_to_the_stream():
+    """Which matrices get a copy in tiles of fewer than 16 rows (sizes and CU count of the measurements), from
+    how many rows of x it is read, and that the layout is what the inverse kernel undoes."""
+    from servelab_amd.kernels import HipOps, Tuning
+    from servelab_amd.kernels.ops import _p
+    ops = HipOps(torch.bfloat16, "cuda:0")
+    ops._num_cus = 256
+    chosen = {N: ops.producer_tile_height(N, 4096) for N in (2048, 3072, 3584, 4096, 5120, 6400, 8192)}
+    assert chosen == {2048: (8, 1), 3072: (12, 1), 3584: (16, 1), 4096: (16, 1), 5120: (10, 1), 6400: (16, 1),
+                      8192: (16, 1)}
+    w = randn(5120, 64, dtype=torch.bfloat16, seed=1)
+    weight = ops.prepare_weight(w, residual_delta=True)
+    assert weight.th == 10 and weight.lower.numel() == 5120 * 64 and weight.tiled.numel() == 5120 * 64
+    assert ops._producer_copy(weight, 1) == (weight.lower, 10)
+    assert ops.prepare_weight(w).lower is None                       # other matrices: tiles of 16 only
+    # a smaller gain is taken with another setting, and then only from 8 rows of x on (see the rule)
+    keen = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(lower_tiles_min_gain=0.05))
+    keen._num_cus = 256
+    assert keen.producer_tile_height(3584, 4096) == (14, 8)
+    weight = keen.prepare_weight(randn(3584, 64, dtype=torch.bfloat16, seed=1), residual_delta=True)
+    assert keen._producer_copy(weight, 7) == (weight.tiled, 16) and keen._producer_copy(weight, 8) == (weight.lower, 14)
+    for th in (16, 14, 12, 10, 8):
+        N, K = 100, 96
+        w = randn(N, K, dtype=torch.bfloat16, seed=th)
+        tiled = torch.full((-(-N // th) * th * K,), 7.0, dtype=torch.bfloat16, device="cuda")
+        back = torch.empty(N, K, dtype=torch.bfloat16, device="cuda")
+        ops._call("gemm", "sl_tile_weight", _p(w), _p(tiled), N, K, th)
+        ops._call("gemm", "sl_untile_weight", _p(tiled), _p(back), N, K, th)
+        assert torch.equal(back, w)
+        blocks = tiled.view(-(-N // th), K // 32, 4, th, 8)              # [tile][k-step][quarter of k][row][8]
+        assert torch.equal(blocks[2, 1, 3, 5], w[2 * th + 5, 32 + 24:32 + 32])
+        assert not blocks[-1, :, :, N - (N // th) * th:].any() or N % th == 0   # rows beyond N are zero
+    off = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(lower_tiles_min_gain=1.0))
+    assert off.prepare_weight(randn(5120, 64, dtype=torch.bfloat16, seed=1), residual_delta=True).lower is None
 
 
 @pytest.mark.parametrize("M,H,N2", [(1, 1536, 96), (8, 3584, 4608), (16, 5120, 1008), (5, 2048, 1000),
@@ -572,7 +614,7 @@ def test_qkv_rope_store(M, nh, nkv, D, page, H, rot, pairs):
     dt = torch.bfloat16
     ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
     if pairs:
-        ops._pair_tiles = lambda M, N, K: True
+        ops._pair_tiles = lambda M, N, K, th=16: True
     N = (nh + 2 * nkv) * D
     x = randn(M, H, dtype=dt, seed=1)
     w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.1 * min(1.0, (256 / H) ** 0.5), seed=2))
