@@ -370,7 +370,7 @@ struct NormFusion {
   // PRODUCER: rows of W per tile, 8..16 and even (W then lies as [ceil(N / th)][K / 32][4][th][8], see
   // sl_tile_weight).  A product of few rows takes as long as its busiest CU needs to pull its tiles of W
   // and its re-read of x, so a matrix whose 16-row tiles do not go round the CUs evenly gets lower tiles
-  // that do (N = 3584 on 256 CUs: 256 tiles of 14 rows instead of 224 of 16).  Other forms: 16.
+  // that do (N = 5120 on 256 CUs: 512 tiles of 10 rows instead of 320 of 16).  Other forms: 16.
   int th;
 };
 
