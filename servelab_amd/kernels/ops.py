@@ -342,8 +342,8 @@ class HipOps:
             self.lower_tiles = self.weight_layout == "dual" and 2.35 * total_bytes <= self.LOWER_TILES_MEMORY_SHARE * total
         return self.weight_layout
 
-    def producer_tile_height(self, N, K, rows=8):
-        """(rows per tile, rows of x from which it pays) for the few-rows product of an [N, K] matrix that
+    def producer_tile_height(self, N, rows=8):
+        """(rows per tile, rows of x from which it pays) for the few-rows product of a matrix of N rows that
         adds to the residual stream.  At 8 rows and more such a product takes as long as its busiest CU needs
         to pull its tiles of W and its re-read of x, so the tiles should go round the CUs evenly: of 16, 14,
         12, 10 and 8 rows the height is taken whose busiest CU pulls least; 16 unless another saves
@@ -393,7 +393,7 @@ class HipOps:
         else:
             weight = LinearWeight(w, tiled)
         if residual_delta and self.fuse_norms and self.lower_tiles:
-            th, lower_from = (_th, 1) if _th is not None else self.producer_tile_height(N, K)
+            th, lower_from = (_th, 1) if _th is not None else self.producer_tile_height(N)
             if th != 16:
                 weight.lower = torch.empty(-(-N // th) * th * K, dtype=torch.bfloat16, device=self.device)
                 weight.th, weight.lower_from = th, lower_from

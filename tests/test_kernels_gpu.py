@@ -353,7 +353,7 @@ def test_lower_tiles_for_the_products_that_add_to_the_stream():
     from servelab_amd.kernels.ops import _p
     ops = HipOps(torch.bfloat16, "cuda:0")
     ops._num_cus = 256
-    chosen = {N: ops.producer_tile_height(N, 4096) for N in (2048, 3072, 3584, 4096, 5120, 6400, 8192)}
+    chosen = {N: ops.producer_tile_height(N) for N in (2048, 3072, 3584, 4096, 5120, 6400, 8192)}
     assert chosen == {2048: (8, 1), 3072: (12, 1), 3584: (16, 1), 4096: (16, 1), 5120: (10, 1), 6400: (16, 1),
                       8192: (16, 1)}
     w = randn(5120, 64, dtype=torch.bfloat16, seed=1)
@@ -364,7 +364,7 @@ def test_lower_tiles_for_the_products_that_add_to_the_stream():
     # a smaller gain is taken with another setting, and then only from 8 rows of x on (see the rule)
     keen = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(lower_tiles_min_gain=0.05))
     keen._num_cus = 256
-    assert keen.producer_tile_height(3584, 4096) == (14, 8)
+    assert keen.producer_tile_height(3584) == (14, 8)
     weight = keen.prepare_weight(randn(3584, 64, dtype=torch.bfloat16, seed=1), residual_delta=True)
     assert keen._producer_copy(weight, 7) == (weight.tiled, 16) and keen._producer_copy(weight, 8) == (weight.lower, 14)
     for th in (16, 14, 12, 10, 8):
