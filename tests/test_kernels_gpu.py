@@ -289,7 +289,7 @@ def test_gated_linear(both, M, I, K, pairs):
         assert rel_err(ops.silu_mul(ops.linear(x, w, None), block), ref) < tol
 
 
-@pytest.mark.parametrize("M,H,N2", [(1, 64, 96), (8, 3584, 4608), (16, 200 * 32, 48), (5, 96, 1000)])
+@pytest.mark.parametrize("M,H,N2", [(1, 64, 96), (8, 3584, 4608), (16, 200 * 32, 48), (5, 96, 1000), (9, 5120, 80)])
 @pytest.mark.parametrize("pairs", [False, True])
 @pytest.mark.parametrize("th", [16, 14, 10, 8])
 def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs, th):
