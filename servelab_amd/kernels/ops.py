@@ -983,6 +983,24 @@ class HipOps:
             self._lib[key] = lib
         return key
 
+    def _decode_shares(self, units, most) -> int:
+        """Into how many shares the keys of each of ``units`` (request, kv head) pairs are cut, ``most`` at
+        most.  A share is a wavefront, and a wavefront streams its keys at the pace of its round trips to
+        memory, so the launch takes what its busiest CU holds: TARGET_WAVES wavefronts (two a CU) are best,
+        and a launch slightly above a whole number of wavefronts per CU is the worst (7B shape, contexts of
+        4,096: 14 requests in 10 shares, 560 wavefronts: 30.6 us a layer; in 9, 504 wavefronts: about 22 us;
+        24 requests 576 against 480 wavefronts: 4.73 against 4.40 ms a step; 48 requests 384 / 576 / 768
+        wavefronts: 5.62 / 5.77 / 5.49 ms).  Taken: the count whose wavefronts fill their rounds over the CUs
+        best, less a fifth of its relative distance from the target; no more than half again the target."""
+        cus, target = self._num_cus, self.TARGET_WAVES
+        best, best_score = 1, None
+        for shares in range(1, max(1, min(most, (3 * target // 2) // units)) + 1):
+            waves = units * shares
+            score = waves / (-(-waves // cus) * cus) - 0.2 * abs(waves - target) / target
+            if best_score is None or score > best_score + 1e-9:
+                best, best_score = shares, score
+        return best
+
     def _pair_prompt_tiles(self, tiles, prompts_and_heads) -> bool:
         """Whether the workgroups of a whole prompt's attention take a late tile of the causal triangle and
         its early mirror (equal work for all, half as many workgroups) or a tile each, long ones first.
@@ -1044,7 +1062,7 @@ class HipOps:
             # (a few requests with long contexts: up to 256 shares, so that the launch still has TARGET_WAVES
             # wavefronts; 7B shape, one request at 32,000 tokens: 64 shares leave one wavefront per CU)
             most = int(self._lib[lib].sl_attention_mfma_max_splits())
-            nsplit = max(1, min(most, blocks // 2, -(-self.TARGET_WAVES // (n_dec * nkv))))
+            nsplit = self._decode_shares(n_dec * nkv, min(most, blocks // 2))
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)

@@ -791,6 +791,17 @@ def test_prompt_attention_through_lds(nh, nkv, D, page, window, form, units):
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+def test_decode_shares_fill_whole_rounds_over_the_cus():
+    """The number of shares of a request's keys at the batch sizes it was measured at (4 kv heads, 256 CUs,
+    contexts of 4,096: 64 shares at most): never slightly more wavefronts than a whole number per CU."""
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.bfloat16, "cuda:0")
+    ops._num_cus = 256
+    shares = {b: ops._decode_shares(4 * b, 64) for b in (1, 8, 14, 16, 17, 24, 48, 64, 128, 200)}
+    assert shares == {1: 64, 8: 16, 14: 9, 16: 8, 17: 7, 24: 5, 48: 4, 64: 2, 128: 1, 200: 1}
+    assert ops._decode_shares(4, 1) == 1 and ops._decode_shares(4, 256) == 128
+
+
 def test_whole_prompts_pair_their_tiles_unless_the_rounds_are_uneven():
     """The choice between a late tile with its early mirror per workgroup and a workgroup per tile, at the
     sizes it was measured at (7B shape: 7 columns a token, 4 kv heads, 256 CUs)."""
@@ -856,14 +867,14 @@ def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window, un
 @pytest.mark.parametrize("nh,nkv,D,page", [(28, 4, 128, 16), (8, 1, 64, 32)])
 @pytest.mark.parametrize("contexts", [(9000,), (9000, 5000)])
 def test_decode_attention_with_more_shares_than_lanes(nh, nkv, D, page, contexts):
-    """One or two requests with long contexts are cut into more than 64 shares (141 here, with a launch
-    that aims at 2,048 wavefronts), of which a lane of the merging wavefront takes several; the key that
-    carries the weight of request 0 lies in a late share."""
+    """One or two requests with long contexts are cut into more than 64 shares (up to 141 here, with a
+    launch that aims at 2,048 wavefronts), of which a lane of the merging wavefront takes several; the key
+    that carries the weight of request 0 lies in a late share."""
     from servelab_amd.kernels import HipOps, Tuning
     dt = torch.bfloat16
     ops, emu = HipOps(dt, "cuda:0", tuning=Tuning(target_waves=2048)), EmulatedOps(dt)
     blocks = -(-max(contexts) // 32)
-    assert min(256, blocks // 2, -(-ops.TARGET_WAVES // (len(contexts) * nkv))) == 141
+    assert 64 < ops._decode_shares(len(contexts) * nkv, min(256, blocks // 2)) <= 141
     seqs = [(c, 1) for c in contexts]
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=21)
     at = 8000
