@@ -372,6 +372,7 @@ struct NormFusion {
   // and its re-read of x, so a matrix whose 16-row tiles do not go round the CUs evenly gets lower tiles
   // that do (N = 5120 on 256 CUs: 512 tiles of 10 rows instead of 320 of 16).  Other forms: 16.
   int th;
+  int pair_x;                // at most 8 rows and one tile a workgroup: a load of x takes two k-steps (see stream_k2)
 };
 
 // Rotary embedding and the write to the cache pages fused into the q/k/v
@@ -515,9 +516,71 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
         }
     }
   };
+  // The same loop for at most 8 rows of x and one tile: a load of x takes two k-steps.  The matrix
+  // instruction has 16 columns for the rows of x; with at most 8 rows the lanes of columns 8..15 load the
+  // same rows one k-step further on, the products of even k-steps go to one accumulator (columns 0..7
+  // valid) and those of odd k-steps to a second (columns 8..15 valid), and the second is added to the
+  // first at the end.  Half as many loads of x: a load takes a place in the CU's queue of outstanding
+  // requests whatever its size, and that queue is what these kernels run on.
+  f32x4 acc_odd = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto stream_k2 = [&](auto tiled_tag, auto th_tag) {
+    static_assert(NT == 1 && U % 2 == 0, "two k-steps a load of x: one tile, an even number of loads in flight");
+    const size_t xs_ = decltype(tiled_tag)::value ? xstep : (size_t)32;
+    constexpr size_t WS = 32 * decltype(th_tag)::value;
+    int row = (i & 7) < M ? (i & 7) : M - 1;
+    if (CONSUMER && F.rows != nullptr) row = F.rows[row];
+    const __bf16* x0 = (F.x_tiled ? x + (size_t)row * 32 + 8 * gq : x + (size_t)row * K + 8 * gq);
+    const __bf16* x2 = x0 + (i >= 8 ? xs_ : 0);          // columns 8..15: one k-step further
+    int ks = ks0;
+    for (; ks + U <= ks1; ks += U) {
+      bf16x8 a[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) a[u] = stream_load(wp[0] + WS * (size_t)(ks + u));
+#pragma unroll
+      for (int u = 0; u < U; u += 2) {
+        const bf16x8 bv = *(const bf16x8*)(x2 + xs_ * (size_t)(ks + u));
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv, acc[0], 0, 0, 0);
+        acc_odd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u + 1], bv, acc_odd, 0, 0, 0);
+      }
+    }
+    if (ks < ks1) {
+      // the last k-steps, fewer than U, in one trip to memory; an odd one at the end has its x in all
+      // 16 columns (nothing lies one k-step further that would be this wavefront's, or the row's)
+      bf16x8 a[U], bv[U / 2], last;
+#pragma unroll
+      for (int u = 0; u < U - 1; ++u)
+        if (ks + u < ks1) a[u] = stream_load(wp[0] + WS * (size_t)(ks + u));
+#pragma unroll
+      for (int u = 0; u + 1 < U - 1; u += 2)
+        if (ks + u + 1 < ks1) bv[u / 2] = *(const bf16x8*)(x2 + xs_ * (size_t)(ks + u));
+      const bool odd = (ks1 - ks) & 1;
+      if (odd) last = *(const bf16x8*)(x0 + xs_ * (size_t)(ks1 - 1));
+#pragma unroll
+      for (int u = 0; u + 1 < U - 1; u += 2)
+        if (ks + u + 1 < ks1) {
+          acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], bv[u / 2], acc[0], 0, 0, 0);
+          acc_odd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u + 1], bv[u / 2], acc_odd, 0, 0, 0);
+        }
+      if (odd) {
+        // (its W is a[ks1 - 1 - ks]: picked by a chain of selects, the index is the same for the wavefront)
+        bf16x8 w_last = a[0];
+#pragma unroll
+        for (int u = 1; u < U - 1; ++u)
+          if (ks + u == ks1 - 1) w_last = a[u];
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_last, last, acc[0], 0, 0, 0);
+      }
+    }
+  };
   // (each form of the loop is straight-line code with constant steps; the tile height is a run-time
   // choice only for producers)
   auto stream_th = [&](auto th_tag) {
+    if constexpr (NT == 1) {
+      if (M <= 8 && F.pair_x) {
+        if (F.x_tiled) stream_k2(std::true_type{}, th_tag);
+        else stream_k2(std::false_type{}, th_tag);
+        return;
+      }
+    }
     if (F.x_tiled) stream_k(std::true_type{}, th_tag);
     else stream_k(std::false_type{}, th_tag);
   };
@@ -529,6 +592,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(
     else if (th == 12) stream_th(std::integral_constant<int, 12>{});
     else if (th == 10) stream_th(std::integral_constant<int, 10>{});
     else stream_th(std::integral_constant<int, 8>{});
+  }
+  if constexpr (NT == 1) {
+    if (M <= 8 && F.pair_x) {         // column m + 8 of the odd k-steps' sums belongs to column m
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[0][r] += __shfl(acc_odd[r], lane + 8, 64);
+    }
   }
 #pragma unroll
   for (int t = 0; t < NT; ++t) red[t][wave][lane] = acc[t];
@@ -644,7 +713,7 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
                                       const float* in_parts, int in_nparts, float eps,
                                       const int* rows, float* resid, const float* next_w,
                                       float* out_parts, const RopeStore* rope, int pair_tiles,
-                                      int x_tiled, int y_tiled, int th, hipStream_t stream) {
+                                      int x_tiled, int y_tiled, int th, int pair_x, hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_skinny: sizes must be positive");
   SL_CHECK(M <= 16, "gemm_skinny: at most 16 rows");
   SL_CHECK(K % 32 == 0, "gemm_skinny: K must be a multiple of 32");
@@ -670,7 +739,7 @@ extern "C" const char* sl_gemm_skinny(const void* x, const void* wt, const float
            "gemm_skinny: x tiled by k-step has as many rows as the product, or rows are picked from it");
   SL_CHECK(!y_tiled || (gated && (N / 2) % 32 == 0) || (resid != nullptr && N % 32 == 0),
            "gemm_skinny: a tiled result is a gated one or a producer's, of a multiple of 32 columns");
-  const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts, x_tiled, y_tiled, th};
+  const NormFusion F{in_parts, in_nparts, eps, rows, resid, next_w, out_parts, x_tiled, y_tiled, th, pair_x};
   const bool few = in_nparts <= 32 * 8;
   if (rope != nullptr) {
     const RopeStore R = *rope;

@@ -238,12 +238,13 @@ class HipOps:
             x_tiled, x = x.shape[0], x.data
         # (the product that adds to the stream reads the copy in lower tiles, where the matrix has one)
         wt, th = self._producer_copy(weight, M) if resid is not None else (weight.tiled, 16)
+        pair = self._pair_tiles(M, N, K, th)
         self._call("gemm", "sl_gemm_skinny", _p(x), _p(wt), _p(bias), _p(y), M, N, K,
                    int(out_f32), int(gated), _p(parts), parts.shape[0] if parts is not None else 0,
                    _c_float(scaled.eps if scaled is not None else 0.0),
                    _p(scaled.rows) if scaled is not None else None, _p(resid), _p(next_gain),
                    _p(out_parts), ctypes.byref(rope) if rope is not None else None,
-                   int(self._pair_tiles(M, N, K, th)), int(x_tiled), int(y_tiled), th)
+                   int(pair), int(x_tiled), int(y_tiled), th, int(M <= 8 and not pair and self.PAIR_X_LOADS))
 
     # ------------------------------------------------------------ embedding
     def embed(self, ids, table):

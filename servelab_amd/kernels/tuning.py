@@ -25,6 +25,9 @@ class Tuning:
     lower_tiles_memory_share: float = 0.55
     lower_tiles_min_gain: float = 0.15
 
+    # few-rows products of at most 8 rows load x for two k-steps at once (gemm.hip, stream_k2)
+    pair_x_loads: bool = True
+
     # ---- products of 17 and more rows over the tiled copy
     # from this many rows on two tiles of W share one read of x (gemm_wide / gemm_mid)
     wide_min_m: int = 17

@@ -387,8 +387,9 @@ def test_lower_tiles_for_the_products_that_add_to_the_stream():
 def test_consumer_products_on_workgroups_that_stay(M, H, N2):
     """The products that read un-normalised rows, on workgroups that keep x in registers and walk
     the tiles (several rounds where the matrix has more tiles than the chip holds workgroups):
-    the very numbers of the kernel with a workgroup per tile, which the test above holds to the
-    unfused sequence.  Row lengths the kernel is not built for are refused."""
+    the very numbers of the kernel with a workgroup per tile (the same but for a last bit of the
+    float32 sums at 8 rows and fewer, where that kernel loads x for two k-steps at once), which the
+    test above holds to the unfused sequence.  Row lengths the kernel is not built for are refused."""
     from servelab_amd.kernels import HipOps, KernelError
     from servelab_amd.kernels.ops import ScaledRows
     ops = HipOps(torch.bfloat16, "cuda:0")
@@ -408,7 +409,12 @@ def test_consumer_products_on_workgroups_that_stay(M, H, N2):
         if N2 % 16 == 0:
             got[stay].append(ops.gated_linear(ScaledRows(x, parts, 1e-5), w2, 8))
     for a, b in zip(got[False], got[True]):
-        assert a.shape == b.shape and torch.equal(a, b)
+        assert a.shape == b.shape
+        if a.shape[0] > 8:
+            assert torch.equal(a, b)
+        else:       # (at most 8 rows: the kernel with a workgroup per tile adds up even and odd k-steps apart)
+            assert rel_err(a, b) < (2e-6 if a.dtype == torch.float32 else 2 ** -8)
+            assert (a != b).float().mean() < (1.0 if a.dtype == torch.float32 else 0.02)
     # and against the formula
     inv = torch.rsqrt(parts.sum(0)[:M] / H + 1e-5)
     ref = (x.float() @ w2.w.float().T) * inv[:, None] + b2
