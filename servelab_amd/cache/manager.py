@@ -113,6 +113,14 @@ class CacheManager:
         (servelab/engine/scheduler.py:211-215)."""
         return self.pages_for(total_tokens) <= self.num_pages
 
+    def can_admit(self, total_tokens: int) -> bool:
+        """Whether a request that is not open yet could be opened and grown to
+        ``total_tokens`` right now (a state slot and the pages of every group
+        are free).  Takes nothing."""
+        need = self.pages_for(total_tokens)
+        return self.state_slots.num_free > 0 and \
+            all(need <= g.allocator.num_free for g in self.page_groups)
+
     def grow(self, request, total_tokens: int) -> bool:
         """Make room for tokens [0, total_tokens) in every group; all groups or
         none.  Already held pages are kept, so growing twice is harmless

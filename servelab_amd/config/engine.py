@@ -43,6 +43,8 @@ class SchedulerConfig:
 
 @dataclass
 class EngineConfig:
+    """Everything ``LLMEngine`` is built from beside the model, in one record
+    (``LLMEngine.from_engine_config``; servelab/config.py:98-107)."""
     cache: CacheConfig = field(default_factory=CacheConfig)
     scheduler: SchedulerConfig = field(default_factory=SchedulerConfig)
     seed: int = 1234
@@ -51,3 +53,4 @@ class EngineConfig:
     tune_products: object = False          # True, or further row counts: time the library's kernels at start-up
     capture_graphs_up_to: int = 0          # > 0: capture the decode graphs of 1..max_num_seqs requests for
                                            # contexts up to this many tokens at start-up (0: at first sight)
+    run_ahead: bool = True                 # queue the next decode step before this one's tokens are read

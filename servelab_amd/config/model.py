@@ -13,6 +13,13 @@ class ConfigError(ValueError):
     """config.json lacks a required key, or holds a value no model can have."""
 
 
+# what the attention kernels take (csrc/attention.hip, MAX_D): a head's channels
+# sit in the registers of one wavefront, 256 at most
+MAX_HEAD_DIM = 256
+# the layer kinds a ``layer_types`` list may name, and what they mean here
+LAYER_KINDS = {"full_attention": False, "sliding_attention": True}
+
+
 _MISSING = object()
 
 
@@ -32,6 +39,24 @@ def read_key(cfg: Dict[str, Any], key: str, default: Any = _MISSING, kind=None):
             raise ConfigError(
                 f"config.json: key '{key}' = {cfg[key]!r} is not a {kind.__name__}")
     return value
+
+
+def refuse_rope_scaling(cfg: Dict[str, Any]) -> None:
+    """The rotary angles here are position * theta^(-2j/D) and nothing else
+    (servelab/parallel/tp_model.py:94-96; servelab/config.py:48-72 reads no
+    scaling key).  A ``rope_scaling`` entry that asks for other angles (linear,
+    dynamic, yarn, ...) is refused rather than dropped: the model would run, with
+    other logits than its authors meant.  null and the type "default" ask for
+    the plain angles and pass."""
+    scaling = cfg.get("rope_scaling")
+    if scaling is None:
+        return
+    kind = scaling.get("rope_type", scaling.get("type")) if isinstance(scaling, dict) else scaling
+    if kind in (None, "default") and isinstance(scaling, dict) and \
+            float(scaling.get("factor", 1.0) or 1.0) == 1.0:
+        return
+    raise ConfigError(f"config.json: rope_scaling = {scaling!r} is not supported: this engine "
+                      f"computes plain rotary angles (no scaling of any kind)")
 
 
 @dataclass
@@ -99,6 +124,7 @@ class Qwen2Config:
             # servelab/engine/scheduler.py:336 compares with `==`; take the first
             eos = eos[0] if eos else 0
         archs = cfg.get("architectures") or ["Qwen2ForCausalLM"]
+        refuse_rope_scaling(cfg)
         out = cls(
             hidden_size=hidden,
             num_layers=read_key(cfg, "num_hidden_layers", kind=int),
@@ -123,6 +149,7 @@ class Qwen2Config:
             raw=dict(cfg),
         )
         out.validate()
+        out.check_layer_types(cfg.get("layer_types"))
         return out
 
     def validate(self) -> None:
@@ -139,6 +166,10 @@ class Qwen2Config:
                     f"num_key_value_heads {self.num_kv_heads}")
             if self.head_dim % 2:
                 problems.append(f"head_dim {self.head_dim} must be even for rotary pairs")
+            if self.head_dim > MAX_HEAD_DIM:
+                problems.append(
+                    f"head_dim {self.head_dim} is more than the attention kernels take "
+                    f"({MAX_HEAD_DIM}: a head's channels sit in one wavefront's registers)")
         if not self.rms_norm_eps > 0:
             problems.append(f"rms_norm_eps must be positive, is {self.rms_norm_eps}")
         if not self.rope_theta > 0:
@@ -151,6 +182,28 @@ class Qwen2Config:
             problems.append(f"torch_dtype '{self.dtype}' is not float16|bfloat16|float32")
         if problems:
             raise ConfigError("config.json: " + "; ".join(problems))
+
+    def check_layer_types(self, layer_types) -> None:
+        """A ``layer_types`` list in config.json must say, layer by layer, what
+        ``use_sliding_window`` / ``max_window_layers`` say: the window of a layer
+        is computed from those keys, and a list that contradicts them names
+        another model than the one that would be served."""
+        if layer_types is None:
+            return
+        if not isinstance(layer_types, (list, tuple)) or len(layer_types) != self.num_layers:
+            raise ConfigError(
+                f"config.json: layer_types must list {self.num_layers} layers, is {layer_types!r}")
+        for i, kind in enumerate(layer_types):
+            if kind not in LAYER_KINDS:
+                raise ConfigError(f"config.json: layer_types[{i}] = {kind!r} is not one of "
+                                  f"{sorted(LAYER_KINDS)}")
+            windowed = self.layer_window(i) is not None
+            if LAYER_KINDS[kind] != windowed:
+                raise ConfigError(
+                    f"config.json: layer_types[{i}] = {kind!r} contradicts use_sliding_window="
+                    f"{self.use_sliding_window}, sliding_window={self.sliding_window}, "
+                    f"max_window_layers={self.max_window_layers}, by which layer {i} "
+                    f"{'has a window' if windowed else 'sees all keys'}")
 
     def to_hf(self) -> Dict[str, Any]:
         """The config.json this configuration is read back from."""

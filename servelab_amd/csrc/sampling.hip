@@ -46,7 +46,10 @@ __device__ __forceinline__ float uniform01(uint64_t seed, uint64_t draw, uint32_
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
   z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
   z ^= z >> 31;
-  return ((float)(z >> 40) + 0.5f) * (1.0f / 16777216.0f);     // in (0, 1)
+  // 23 bits: k + 0.5 is then exact in float32, so u stays inside (0, 1).  (With 24 bits the largest
+  // k + 0.5 rounds up to 2^24, u becomes 1 and its Gumbel value infinite: once in 2^24 logits a
+  // token would be drawn whatever its logit.)
+  return ((float)(z >> 41) + 0.5f) * (1.0f / 8388608.0f);
 }
 
 // e^x for x <= 0 by the hardware's 2^x: the top-p search below evaluates it for

@@ -24,8 +24,7 @@ const char* sl_sample(const float* logits, int R, int V, const float* temperatur
 
 // sl_sample for callers that cannot allocate device memory: code under HIP
 // graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
-// no counterpart in the reference, whose sampler runs row by row on the host
-// (servelab/engine/sampler.py:10-45).  Same arguments and results as sl_sample,
+// no counterpart in the reference.  Same arguments and results as sl_sample,
 // but the scratch is a static device array of SL_SAMPLE_STATIC_BYTES inside the
 // library (each GPU the library runs on holds its own copy until the process
 // ends) and the split of a row into slices is chosen here.  Sizes whose scratch

@@ -20,12 +20,15 @@ from .session import load_model_on_device, make_runner, random_model_on_device
 
 
 class _TokenBuffers:
-    """Two pinned host buffers for sampled tokens, used in turn: the step ahead
-    copies into one while the host still reads the other."""
+    """Two pinned host buffers used in turn: for sampled tokens, the step ahead
+    copies into one while the host still reads the other; for the rows a step
+    ahead gathers, the host fills one while the copy out of the other may still
+    be queued."""
 
-    def __init__(self, rows: int, device):
+    def __init__(self, rows: int, device, dtype=torch.int32):
         self.cuda = torch.device(device).type == "cuda"
-        self.buffers = [torch.empty(max(1, rows), dtype=torch.int32) for _ in range(2)]
+        self.dtype = dtype
+        self.buffers = [torch.empty(max(1, rows), dtype=dtype) for _ in range(2)]
         if self.cuda:
             self.buffers = [b.pin_memory() for b in self.buffers]
         self.turn = 0
@@ -33,7 +36,7 @@ class _TokenBuffers:
     def take(self, n: int) -> torch.Tensor:
         self.turn ^= 1
         if self.buffers[self.turn].numel() < n:
-            grown = torch.empty(2 * n, dtype=torch.int32)
+            grown = torch.empty(2 * n, dtype=self.dtype)
             self.buffers[self.turn] = grown.pin_memory() if self.cuda else grown
         return self.buffers[self.turn][:n]
 
@@ -129,8 +132,21 @@ class LLMEngine:
         self.run_ahead = bool(run_ahead)
         self._flight: Optional[_Flight] = None
         self._token_buffers = _TokenBuffers(self.scheduler_config.max_num_seqs, self.device)
+        self._row_buffers = _TokenBuffers(self.scheduler_config.max_num_seqs, self.device, torch.int64)
+        self._aborted: List[RequestOutput] = []      # results of abort_request, returned by the next step
         self._submitted = 0
         self.num_steps = 0
+
+    @classmethod
+    def from_engine_config(cls, model_config, engine_config, **more) -> "LLMEngine":
+        """The engine that an ``EngineConfig`` describes (cache, scheduler, seed,
+        dtype, device and the start-up options in one record); ``more`` passes
+        on what the record does not hold (``model``, ``ops``, ``tokenizer``,
+        ``random_weights``, ...)."""
+        ec = engine_config
+        return cls(model_config, ec.cache, ec.scheduler, seed=ec.seed, device=ec.device,
+                   dtype=ec.dtype, tune_products=ec.tune_products,
+                   capture_graphs_up_to=ec.capture_graphs_up_to, run_ahead=ec.run_ahead, **more)
 
     # -------------------------------------------------------------- intake
     def add_request(self, prompt: Optional[str] = None,
@@ -170,10 +186,10 @@ class LLMEngine:
         two steps then costs no device time.  A request that a stop token ends
         has one wasted row in the step ahead; a newcomer waits for that step."""
         flight, self._flight = self._flight, None
-        outputs: List[RequestOutput] = []
+        outputs, self._aborted = self._aborted, []
         if flight is None:
             plan = self.scheduler.schedule()
-            outputs = [result_of(r, self._to_text) for r in plan.aborted]
+            outputs += [result_of(r, self._to_text) for r in plan.aborted]
             if plan.is_empty():
                 if not outputs and self.scheduler.has_unfinished():
                     raise RuntimeError("nothing can be scheduled although requests are unfinished")
@@ -207,7 +223,11 @@ class LLMEngine:
             rows = [row_of[it.request.request_id] for it in items]
             ids = after.device_tokens
             if rows != list(range(len(after.drawing))):
-                ids = ids[torch.tensor(rows, dtype=torch.long, device=ids.device)]
+                # requests have left since that step: gather the rows that stay (the index goes
+                # through pinned memory, so nothing here waits for the device)
+                index = self._row_buffers.take(len(rows))
+                index.copy_(torch.tensor(rows, dtype=torch.int64))
+                ids = ids.index_select(0, index.to(ids.device, non_blocking=True))
             logits = self.runner.step(entries, device_ids=ids)
         drawn_before = 1 if after is not None else 0     # the token of the step this one follows
         device_tokens = self.sampler.sample_on_device(
@@ -216,7 +236,18 @@ class LLMEngine:
         return _Flight(plan, drawing, device_tokens, self._token_buffers)
 
     def abort_request(self, request_id: str) -> bool:
-        return self.scheduler.abort_request(request_id)
+        """servelab/engine/engine.py:162-163.  The request's pages are free at
+        once (a step or a step ahead that is still queued on the device may
+        write its rows of them; whoever gets the pages next writes after that,
+        in stream order); its result, with finish reason "aborted", comes with
+        the next ``step``."""
+        req = self.scheduler.abort_request(request_id)
+        if req is None:
+            return False
+        self._aborted.append(result_of(req, self._to_text))
+        if self._flight is not None and all(it.request.done for it in self._flight.plan.items()):
+            self._flight = None                  # nobody is left to take the step ahead's tokens
+        return True
 
     @property
     def _to_text(self):
@@ -226,7 +257,7 @@ class LLMEngine:
     def run(self, on_step: Optional[Callable[[dict], None]] = None):
         """Steps until nothing is unfinished, yielding each result as its
         request ends; ``on_step`` is called with ``stats()`` after every step."""
-        while self.has_unfinished():
+        while self.has_unfinished() or self._aborted:
             yield from self.step()
             if on_step is not None:
                 on_step(self.stats())
@@ -252,5 +283,7 @@ class LLMEngine:
                 "num_blocks": self.num_blocks, "block_size": self.cache_config.block_size,
                 "dtype": str(self.dtype).replace("torch.", ""),
                 "checkpoint_dtype": getattr(self.model_config, "dtype", None),
+                "dtype_substituted": (getattr(self.model_config, "dtype", None) == "float16"
+                                      and self.dtype == torch.bfloat16),
                 "device": str(self.device),
                 "steps": self.num_steps}

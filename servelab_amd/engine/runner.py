@@ -130,13 +130,15 @@ class ModelRunner:
             cap *= 2
         return (B, cap)
 
-    def _step_graph(self, key, packed, starts, rows, device_ids=None):
+    def _step_graph(self, key, packed, starts, rows, device_ids=None, evict=True):
         """Decode step through a HIP graph.  The first step of a shape runs
         eagerly on a side stream (its result is returned) and is then captured;
         later steps overwrite the graph's metadata buffer and replay it.
         Everything a launch depends on besides device memory is fixed by the
         key: the number of sequences and the context capacity, which sets the
-        width of the block tables and how the decode attention splits."""
+        width of the block tables and how the decode attention splits.
+        ``evict=False``: a new graph that would not fit beside the others is
+        not made (None is returned and nothing ran)."""
         B, cap = key
         pages = cap // self.manager.page_size
         arr = build_arrays(packed, starts, rows, self.manager, fixed_pages=pages)
@@ -155,6 +157,9 @@ class ModelRunner:
             self.graph_replays += 1
             self._decoding = (key, arr)
             return logits
+        need = self._entry_bytes(host, B)
+        if not evict and self._graphs and self._graph_bytes + need > self.graph_memory_limit:
+            return None
         staging = torch.empty_like(host).pin_memory()
         staging.copy_(host)
         dev = staging.to(self.rt.device, non_blocking=True)
@@ -166,7 +171,6 @@ class ModelRunner:
         with torch.cuda.stream(side):
             eager = self.model.forward(batch, self.bindings)
         torch.cuda.current_stream().wait_stream(side)
-        need = self._entry_bytes(dev, B)
         self._make_room(need)
         if self._graph_pool is None:
             self._graph_pool = torch.cuda.graph_pool_handle()
@@ -196,7 +200,7 @@ class ModelRunner:
             if cap >= limit:
                 break
             cap *= 2
-        made = 0
+        made, full = 0, False
         for B in sorted({int(b) for b in batch_sizes if 1 <= int(b) <= self.graph_max_seqs}):
             tags = [("capture_graphs", i) for i in range(B)]
             opened = []
@@ -211,23 +215,25 @@ class ModelRunner:
                 for cap in caps:
                     if (B, cap) in self._graphs or cap // self.manager.page_size < 1:
                         continue
-                    need = B * self.model.spec.vocab_size * 4
-                    if self._graphs and self._graph_bytes + need > self.graph_memory_limit:
-                        return made
-                    self._step_graph((B, cap), packed, [0] * B, list(range(B)))
+                    if self._step_graph((B, cap), packed, [0] * B, list(range(B)), evict=False) is None:
+                        full = True
+                        break
                     made += 1
             finally:
                 for t in opened:
                     self.close(t)
                 self._decoding = None
+            if full:
+                break
         if made:
             torch.cuda.synchronize(self.rt.device)
         return made
 
-    def _entry_bytes(self, dev, B) -> int:
+    def _entry_bytes(self, meta, B) -> int:
         """What a captured graph keeps alive beside the shared pool of
-        intermediates: its logits and its metadata buffer."""
-        return B * self.model.spec.vocab_size * 4 + dev.numel() * dev.element_size()
+        intermediates: its logits and its metadata buffer (``meta``: that
+        buffer, or the host array it is made from)."""
+        return B * self.model.spec.vocab_size * 4 + meta.numel() * meta.element_size()
 
     def _make_room(self, need: int) -> None:
         """Drop the graphs used longest ago until ``need`` more bytes fit the

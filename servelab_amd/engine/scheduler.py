@@ -105,16 +105,17 @@ class Scheduler:
     def add_request(self, req: Request) -> None:
         self.queue.append(req)
 
-    def abort_request(self, request_id: str) -> bool:
-        """servelab/engine/scheduler.py:132-144."""
+    def abort_request(self, request_id: str) -> Optional[Request]:
+        """servelab/engine/scheduler.py:132-144; the aborted request, or None
+        when no unfinished request has that id."""
         for held in (self.queue, self.active):
             for i, r in enumerate(held):
                 if r.request_id == request_id:
                     held.pop(i)
                     self.manager.close(request_id)
                     r.finish("aborted", self.clock())
-                    return True
-        return False
+                    return r
+        return None
 
     def has_unfinished(self) -> bool:
         return bool(self.queue or self.active)
@@ -187,12 +188,16 @@ class Scheduler:
         """The step after ``plan``, planned while ``plan`` still runs and its
         sampled tokens are not known: one more token for every request of
         ``plan`` that cannot end with this step by its length.  Possible only
-        when ``plan`` samples for every active request and nothing waits for
-        admission (so the step after it would be exactly this one, unless a
-        stop token ends a request: its row of the step ahead is then wasted and
-        ignored).  Pages are reserved; None when the step cannot be planned
-        ahead.  ``complete`` must see ``plan`` before the plan ahead."""
-        if self.queue or not plan.items() or len(plan.items()) != len(self.active):
+        when ``plan`` samples for every active request and the step after it
+        would be exactly this one, unless a stop token ends a request (its row
+        of the step ahead is then wasted and ignored).  That holds when nothing
+        waits for admission, and also under a standing queue as long as nobody
+        can be admitted in the next step: every slot is taken and stays taken,
+        the token budget is used up by the decode tokens, or the head of the
+        queue does not fit the pages that the step ahead leaves free.  Pages
+        are reserved; None when the step cannot be planned ahead.  ``complete``
+        must see ``plan`` before the plan ahead."""
+        if not plan.items() or len(plan.items()) != len(self.active):
             return None
         if not all(item.samples and item.request.phase == ACTIVE for item in plan.items()):
             return None
@@ -207,10 +212,26 @@ class Scheduler:
             ahead.decodes.append(Planned(req, item.start + item.count, 1))
         if not ahead.decodes or len(ahead.decodes) > self.cfg.max_num_batched_tokens:
             return None
+        if self.queue and len(ahead.decodes) < len(plan.items()):
+            return None                                       # a request ends: its slot and pages go to the queue
         for item in ahead.decodes:
             if not self.manager.grow(item.request.request_id, item.start + 1):
                 return None                                   # (pages taken so far stay with their requests)
+        if self.queue and self._could_admit(len(ahead.decodes)):
+            return None                                       # (likewise: the next step asks for the same pages)
         return ahead
+
+    def _could_admit(self, decodes: int) -> bool:
+        """Whether the next ``schedule`` would take (or abort) the head of the
+        queue beside ``decodes`` decode tokens, as the pool stands now."""
+        budget = self.cfg.max_num_batched_tokens - decodes
+        if len(self.active) >= self.cfg.max_num_seqs or budget <= 0:
+            return False
+        head = min(self.queue, key=self.key)
+        too_long = self.max_positions is not None and len(head.tokens) > self.max_positions
+        if too_long or not self.manager.can_ever_hold(len(head.tokens)):
+            return True                                       # it is aborted there, and the next one is looked at
+        return self.manager.can_admit(head.cached + self._portion(head, budget))
 
     # ------------------------------------------------------------- helpers
     def _portion(self, req: Request, budget: int) -> int:

@@ -26,15 +26,27 @@ FLOAT16_NOTICE = ("config.json says torch_dtype float16: this engine has bfloat1
                   "Pass dtype float32 for the exact path.")
 
 
+_noticed = set()
+
+
+def notice_once(text: str) -> None:
+    """A line on standard error, once per process."""
+    if text not in _noticed:
+        _noticed.add(text)
+        print(f"[servelab_amd] {text}", file=sys.stderr, flush=True)
+
+
 def resolve_dtype(name: str, config=None) -> torch.dtype:
     """'auto' takes config.json's torch_dtype.  There are no float16 kernels: a
     float16 checkpoint under 'auto' is served in bfloat16 and says so on
-    standard error (the reference serves it as float16,
-    servelab/engine/engine.py:35-39); float16 asked for by name is refused."""
+    standard error, once per process, and in the engine's ``stats()``
+    (``dtype_substituted``); the reference serves it as float16
+    (servelab/engine/engine.py:35-39), so logits of float16 checkpoints are
+    held to no reference figure.  float16 asked for by name is refused."""
     if name in (None, "auto"):
         name = getattr(config, "dtype", "bfloat16")
         if name in ("float16", "fp16", "half"):
-            print(f"[servelab_amd] {FLOAT16_NOTICE}", file=sys.stderr, flush=True)
+            notice_once(FLOAT16_NOTICE)
             name = "bfloat16"
     if name not in _DTYPES:
         raise ValueError(f"dtype must be bfloat16 or float32 (or auto), is {name!r}: "

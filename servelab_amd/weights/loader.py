@@ -85,7 +85,14 @@ def check_tensors(expected: Dict[str, Tuple[int, ...]],
     """One error that lists every missing tensor, every unexpected tensor and
     every wrong shape.  ``optional`` names may be present without being used
     (a stray lm_head.weight beside tied embeddings,
-    servelab/parallel/tp_model.py:112-113)."""
+    servelab/parallel/tp_model.py:112-113).
+
+    Decision: an unexpected tensor is fatal, like a missing one.  The reference
+    prints the names it did not use and goes on (servelab/engine/engine.py:88-90);
+    here a tensor that no part owns means the folder holds another model than
+    config.json describes (further layers, an adapter, a bias the configuration
+    switched off), and serving it would give logits nobody asked for.  The only
+    names let through are those of ``ignorable`` and ``optional``."""
     missing = sorted(n for n in expected if n not in found)
     unexpected = sorted(n for n in found
                         if n not in expected and n not in optional and not ignorable(n))

@@ -9,6 +9,7 @@ scheduler) runs without a GPU.  Nothing in ``servelab_amd`` imports this file.
 Layouts: K pages [pages, nkv, page_size, D]; V pages [pages, nkv, D, page_size];
 qkv rows [T, (nh + 2 nkv) D] with q first, then k, then v, head-major.
 """
+import numpy as np
 import torch
 
 
@@ -163,3 +164,60 @@ class EmulatedOps:
     # ------------------------------------------------------------- sampling
     def argmax(self, logits):
         return torch.argmax(logits, dim=-1).to(torch.int32)
+
+    def sample(self, logits, temperature, top_k, top_p, seeds, draws):
+        """One token per row: the argmax where temperature is 0, else the largest
+        of ``perturbed_scores`` among the logits the row's cut keeps."""
+        out = []
+        for r in range(logits.shape[0]):
+            T = float(temperature[r])
+            if T == 0.0:
+                out.append(int(torch.argmax(logits[r])))
+                continue
+            k = int(top_k[r]) if top_k is not None else -1
+            p = float(top_p[r]) if top_p is not None else 1.0
+            scores = perturbed_scores(logits[r], T, int(seeds[r]), int(draws[r]))
+            scores[~kept_by_cut(logits[r], T, k, p)] = -np.inf
+            out.append(int(np.argmax(scores)))
+        return torch.tensor(out, dtype=torch.int32, device=logits.device)
+
+
+def uniform01(seed: int, draw: int, n: int) -> np.ndarray:
+    """u_i in (0, 1) for i in [0, n): a counter-based 64-bit mix of (seed, draw, i)
+    whose top 23 bits become (bits + 0.5) / 2^23."""
+    one = np.ones(n, dtype=np.uint64)
+    i = np.arange(n, dtype=np.uint64)
+    z = one * np.uint64(seed % (1 << 64)) + np.uint64(0x9E3779B97F4A7C15) * (
+        one * np.uint64(draw) * np.uint64(0x100000001B3) + i + np.uint64(1))
+    z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    z ^= z >> np.uint64(31)
+    return ((z >> np.uint64(41)).astype(np.float64) + 0.5) / 8388608.0
+
+
+def perturbed_scores(row, T: float, seed: int, draw: int) -> np.ndarray:
+    """logit_i / max(T, 1e-6) + g_i with g_i = -ln(-ln u_i): the index of the
+    largest one is an exact draw from softmax(logits / T) (Gumbel-max)."""
+    x = row.detach().double().cpu().numpy() / max(T, 1e-6)
+    u = uniform01(seed, draw, x.shape[0])
+    return x - np.log(-np.log(u))
+
+
+def kept_by_cut(row, T: float, top_k: int, top_p: float) -> np.ndarray:
+    """Which logits a row's cut keeps: the top_k largest when top_k > 0 (top_p is
+    then ignored); else the sorted prefix whose cumulative probability stays
+    <= top_p, the first always kept (servelab/engine/sampler.py:30-44)."""
+    x = row.detach().double().cpu().numpy() / max(T, 1e-6)
+    keep = np.ones(x.shape[0], dtype=bool)
+    if top_k > 0:
+        keep[:] = False
+        keep[np.argsort(-x, kind="stable")[:top_k]] = True
+    elif top_p < 1.0:
+        order = np.argsort(-x, kind="stable")
+        probs = np.exp(x[order] - x[order[0]])
+        cum = np.cumsum(probs / probs.sum())
+        inside = cum <= top_p
+        inside[0] = True
+        keep[:] = False
+        keep[order[inside]] = True
+    return keep

@@ -46,12 +46,33 @@ def test_missing_required_key_is_named(key):
     ({"num_key_value_heads": 3}, "multiple"), ({"head_dim": 15}, "even"),
     ({"rms_norm_eps": 0.0}, "rms_norm_eps"), ({"hidden_act": "gelu"}, "hidden_act"),
     ({"use_sliding_window": True, "sliding_window": None}, "sliding_window"),
-    ({"torch_dtype": "int8"}, "torch_dtype"), ({"vocab_size": "many"}, "vocab_size")])
+    ({"torch_dtype": "int8"}, "torch_dtype"), ({"vocab_size": "many"}, "vocab_size"),
+    ({"rope_scaling": {"type": "yarn", "factor": 4.0,
+                       "original_max_position_embeddings": 32768}}, "rope_scaling"),
+    ({"rope_scaling": {"rope_type": "linear", "factor": 2.0}}, "rope_scaling"),
+    ({"layer_types": ["full_attention", "sliding_attention"]}, r"layer_types\[1\]"),
+    ({"layer_types": ["full_attention"]}, "layer_types must list 2"),
+    ({"layer_types": ["full_attention", "chunked_attention"]}, "chunked_attention"),
+    ({"head_dim": 320}, "head_dim 320 is more than the attention kernels take")])
 def test_impossible_values_are_refused(change, word):
     raw = dict(TINY_A)
     raw.update(change)
     with pytest.raises(ConfigError, match=word):
         Qwen2Config.from_hf(raw)
+
+
+def test_keys_that_ask_for_what_is_computed_pass():
+    raw = dict(TINY_B, rope_scaling=None,
+               layer_types=["full_attention", "full_attention", "sliding_attention"])
+    assert Qwen2Config.from_hf(raw) == Qwen2Config.from_hf(TINY_B)
+    raw = dict(TINY_A, rope_scaling={"rope_type": "default"},
+               layer_types=["full_attention", "full_attention"])
+    assert Qwen2Config.from_hf(raw) == Qwen2Config.from_hf(TINY_A)
+    # a window that use_sliding_window switches off is no window, whatever sliding_window says
+    raw = dict(TINY_B, use_sliding_window=False, layer_types=["full_attention"] * 3)
+    assert [Qwen2Config.from_hf(raw).layer_window(i) for i in range(3)] == [None] * 3
+    with pytest.raises(ConfigError, match="contradicts"):
+        Qwen2Config.from_hf(dict(TINY_B, layer_types=["full_attention"] * 3))
 
 
 def test_round_trip_and_param_count():

@@ -48,6 +48,17 @@ def test_any_cutting_gives_the_same_tokens(folder_and_plain, max_batched, max_se
     assert [o.outputs[0].token_ids for o in outs] == want
 
 
+def test_engine_from_one_record(folder_and_plain):
+    from servelab_amd import EngineConfig
+    folder, want = folder_and_plain
+    ec = EngineConfig(cache=CacheConfig(num_blocks=32), scheduler=SchedulerConfig(max_num_seqs=2),
+                      seed=5, dtype="float32", device="cpu", run_ahead=False)
+    eng = LLMEngine.from_engine_config(load_config(folder), ec, ops=EmulatedOps())
+    assert (eng.num_blocks, eng.scheduler.cfg.max_num_seqs, eng.sampler.seed, eng.run_ahead) == (32, 2, 5, False)
+    outs = eng.generate(PROMPTS[:2], SamplingParams.greedy(12))
+    assert [o.outputs[0].token_ids for o in outs] == want[:2]
+
+
 def test_preemption_keeps_outputs_whole(folder_and_plain):
     folder, want = folder_and_plain
     eng = make_engine(folder, num_blocks=9, max_batched=64)      # 144 tokens of cache for 4 requests
@@ -206,3 +217,89 @@ def test_decoding_a_step_ahead_changes_nothing_but_the_number_of_model_steps(fol
     other = eng.generate([PROMPTS[1]], SamplingParams.greedy(12))[0]
     assert other.outputs[0].token_ids == want[1]
     eng.runner.manager.check()
+
+
+def test_decoding_runs_ahead_under_a_standing_queue(folder_and_plain):
+    """More requests than slots: while every slot decodes and nobody ends by length, the queue
+    cannot move, so the engine keeps a step ahead; the tokens are plain's, and the number of
+    model steps is the one without the step ahead (no stop tokens: no row is wasted)."""
+    folder, want = folder_and_plain
+    steps, ahead_seen = {}, 0
+    for ahead in (False, True):
+        eng = make_engine(folder, max_seqs=2, run_ahead=ahead)
+        for p in PROMPTS:
+            eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(12))
+        done = {}
+        while eng.has_unfinished():
+            for out in eng.step():
+                done[out.request_id] = out.outputs[0].token_ids
+            if eng._flight is not None and eng.scheduler.queue:
+                ahead_seen += 1
+        assert [done[f"req-{i + 1}"] for i in range(4)] == want
+        assert eng.runner.manager.num_free_pages() == 64 and eng._flight is None
+        eng.runner.manager.check()
+        steps[ahead] = eng.runner.steps
+    assert steps[True] == steps[False]
+    assert ahead_seen >= 8                       # the first pair's decode steps, with two requests waiting
+
+
+def test_seeded_draws_do_not_depend_on_the_step_ahead_or_the_batch(folder_and_plain):
+    """Temperature, top-k and top-p rows with different lengths and a stop token: the step ahead
+    draws with the counter of the token before it, gathers the rows of requests that stay, and
+    gives the tokens of the engine that waits for every step; so does every request alone."""
+    folder, _ = folder_and_plain
+    params = [SamplingParams(temperature=0.9, max_tokens=14, seed=11),
+              SamplingParams(temperature=1.3, top_k=5, max_tokens=5, seed=12),
+              SamplingParams(temperature=0.8, top_p=0.7, max_tokens=9, seed=13),
+              SamplingParams(temperature=0.0, max_tokens=11)]
+
+    def run(ahead, which, stop=()):
+        eng = make_engine(folder, run_ahead=ahead, max_seqs=3)
+        ids = []
+        for i in which:
+            sp = params[i]
+            sp = SamplingParams(temperature=sp.temperature, top_k=sp.top_k, top_p=sp.top_p,
+                                max_tokens=sp.max_tokens, seed=sp.seed, stop_token_ids=tuple(stop))
+            ids.append(eng.add_request(prompt_token_ids=PROMPTS[i], sampling_params=sp))
+        done = {o.request_id: o.outputs[0] for o in eng.run()}
+        assert eng.runner.manager.num_free_pages() == 64 and eng._flight is None
+        eng.runner.manager.check()
+        return [(done[i].token_ids, done[i].finish_reason) for i in ids]
+
+    waited = run(False, range(4))
+    assert run(True, range(4)) == waited
+    assert len({tuple(t) for t, _ in waited}) == 4 and waited[0][0] != waited[3][0]
+    for i in range(4):
+        assert run(True, [i]) == [waited[i]]
+    stop = waited[0][0][6]                       # ends request 0 part-way, in a step that has a step ahead
+    cut = run(False, range(4), stop=(stop,))
+    assert cut[0][1] == "eos" and len(cut[0][0]) <= 7
+    assert run(True, range(4), stop=(stop,)) == cut
+
+
+def test_an_aborted_request_is_reported_and_leaves_no_step_behind(folder_and_plain):
+    folder, want = folder_and_plain
+    eng = make_engine(folder)
+    rid = eng.add_request(prompt_token_ids=PROMPTS[0], sampling_params=SamplingParams.greedy(12))
+    eng.step(), eng.step()
+    assert eng._flight is not None and eng.abort_request(rid)
+    assert eng._flight is None                   # the step ahead has nobody left to take its tokens
+    assert not eng.abort_request(rid)
+    steps = eng.runner.steps
+    other = eng.add_request(prompt_token_ids=PROMPTS[1], sampling_params=SamplingParams.greedy(12))
+    outs = eng.step()                            # the newcomer's prompt runs in this very step
+    assert eng.runner.steps == steps + 2         # (and its first decode step is queued behind it)
+    assert [(o.request_id, o.outputs[0].finish_reason) for o in outs] == [(rid, "aborted")]
+    assert outs[0].outputs[0].token_ids == want[0][:len(outs[0].outputs[0].token_ids)]
+    done = {o.request_id: o.outputs[0].token_ids for o in eng.run()}
+    assert done == {other: want[1]}
+    # aborts while others go on, through run(): everything is reported once
+    eng = make_engine(folder)
+    ids = [eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(12)) for p in PROMPTS]
+    for _ in range(4):
+        eng.step()
+    assert eng.abort_request(ids[2])
+    got = {o.request_id: o.outputs[0] for o in eng.run()}
+    assert got[ids[2]].finish_reason == "aborted"
+    assert [got[i].token_ids for i in (ids[0], ids[1], ids[3])] == [want[0], want[1], want[3]]
+    assert eng.runner.manager.num_free_pages() == 64

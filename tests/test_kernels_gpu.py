@@ -1013,6 +1013,58 @@ def test_argmax_and_sampling():
     assert (freq - wantp).abs().max().item() < 0.015
 
 
+def assert_plain_draws(tokens, logits, temperature, top_k, top_p, seeds, draws, slack=2e-3):
+    """Every token is the plain Gumbel-max draw of its row (tests/emulated_ops.py: the same
+    counter-based uniforms, logarithms in float64), or ties with it within ``slack`` (the kernels
+    take their logarithms from the hardware's log2)."""
+    from emulated_ops import kept_by_cut, perturbed_scores
+    import numpy as np
+    for r, tok in enumerate(tokens.tolist()):
+        T = float(temperature[r])
+        if T == 0.0:
+            assert tok == int(logits[r].argmax()), f"row {r}"
+            continue
+        scores = perturbed_scores(logits[r], T, int(seeds[r]), int(draws[r]))
+        keep = kept_by_cut(logits[r], T, int(top_k[r]) if top_k is not None else -1,
+                           float(top_p[r]) if top_p is not None else 1.0)
+        assert keep[tok], f"row {r}: token {tok} lies outside the cut"
+        best = np.where(keep, scores, -np.inf).max()
+        assert scores[tok] >= best - slack, f"row {r}: token {tok} scores {scores[tok]}, best {best}"
+
+
+def test_draws_are_the_plain_gumbel_draws():
+    """Seeded draws over a wide row equal the plain ones, with and without cuts; the uniform that
+    the hash maps to its largest value (seed 1234, draw 1, index 58452: 1 - 2^-24) stays below 1,
+    so its Gumbel value is finite and a logit of -20 there is not drawn."""
+    from emulated_ops import uniform01
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.float32, "cuda:0")
+    R, V = 12, 152064
+    assert uniform01(1234, 1, V)[58452] == 1 - 2.0 ** -24 and uniform01(1234, 1, V).max() < 1.0
+    logits = 2.0 * randn(R, V, seed=17)
+    logits[0] = 0.0
+    logits[0, 58452] = -20.0
+    temp = torch.full((R,), 0.9).cuda()
+    temp[0], temp[5] = 1.0, 0.0
+    seeds = (torch.arange(R, dtype=torch.int64) * 977 + 3).cuda()
+    draws = (torch.arange(R, dtype=torch.int64) % 4).cuda()
+    seeds[0], draws[0] = 1234, 1
+    toks = ops.sample(logits, temp, None, None, seeds, draws)
+    assert toks[0].item() != 58452
+    assert_plain_draws(toks, logits, temp, None, None, seeds, draws)
+    top_k = torch.full((R,), -1, dtype=torch.int32).cuda()
+    top_k[1::3] = 50
+    top_p = torch.ones(R).cuda()
+    top_p[2::3] = 0.85
+    toks = ops.sample(logits, temp, top_k, top_p, seeds, draws)
+    # (the kernel finds the top-p cut with weights from the hardware's 2^x: a logit right at the cut
+    # may fall on either side, so the plain cut is taken a little wider)
+    assert_plain_draws(toks, logits, temp, top_k, torch.clamp(top_p + 1e-4, max=1.0), seeds, draws)
+    short = logits[:, :3000].contiguous()                     # one workgroup a row
+    toks = ops.sample(short, temp, top_k, top_p, seeds, draws)
+    assert_plain_draws(toks, short, temp, top_k, torch.clamp(top_p + 1e-4, max=1.0), seeds, draws)
+
+
 @pytest.mark.parametrize("V", [50000, 50001, 152064])
 def test_sampling_cuts_of_a_wide_vocabulary(V):
     """top-k and top-p over a wide row (vector loads when the row is 16-byte

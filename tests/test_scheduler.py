@@ -254,3 +254,116 @@ def test_window_groups_keep_few_pages_during_long_decoding():
     assert s.num_output == 40
     assert d.manager.page_groups[1].allocator.high_water <= 4
     assert d.manager.page_groups[0].allocator.high_water == 12
+
+
+def ahead_driver(**kw):
+    """A driver that does what the engine does around every step: ask for the
+    step ahead while the step's tokens are not known yet, and when there is one
+    run it as the next step."""
+    d = Driver(**kw)
+
+    def run_plan(out):
+        """Runs ``out``; returns the step ahead that was planned meanwhile."""
+        sampled = {}
+        for item in out.items():
+            if item.request.phase == "active":
+                d.manager.commit(item.request.request_id, item.start + item.count)
+            if item.samples:
+                sampled[item.request.request_id] = d.token
+        ahead = d.scheduler.plan_ahead(out)
+        d.finished += d.scheduler.complete(out, sampled)
+        d.aborted += out.aborted
+        d.manager.check()
+        return ahead
+
+    def step_and_ahead():
+        out = d.scheduler.schedule()
+        return out, run_plan(out)
+
+    def run_with_ahead(max_steps=500):
+        planned_ahead = steps = 0
+        while d.scheduler.has_unfinished():
+            steps += 1
+            assert steps < max_steps
+            out = d.scheduler.schedule()
+            while out is not None:
+                assert all(it.request.phase == "active" for it in out.items())   # (no stop tokens here)
+                out = run_plan(out)
+                planned_ahead += out is not None
+        assert d.manager.num_free_pages() == d.manager.num_pages
+        return planned_ahead
+    d.run_plan, d.step_and_ahead, d.run_with_ahead = run_plan, step_and_ahead, run_with_ahead
+    return d
+
+
+def test_the_step_ahead_is_planned_under_a_standing_queue_when_nobody_can_be_admitted():
+    # two slots, five requests: while both slots decode and nobody ends by length, the queue
+    # cannot move, so the next step is known
+    d = ahead_driver(max_seqs=2, num_pages=64)
+    reqs = [d.submit(f"r{i}", 6, 9) for i in range(5)]
+    out, ahead = d.step_and_ahead()            # r0, r1 admitted; three wait
+    assert len(d.scheduler.queue) == 3 and len(out.portions) == 2
+    assert ahead is not None and [x.request.request_id for x in ahead.decodes] == ["r0", "r1"]
+    # the pages of the step ahead are reserved: the ordinary plan of that step is the same one
+    free = d.manager.num_free_pages()
+    again = d.scheduler.schedule()
+    assert [(x.request.request_id, x.start) for x in again.decodes] == \
+        [(x.request.request_id, x.start) for x in ahead.decodes] and not again.portions
+    assert d.manager.num_free_pages() == free
+    d.run_plan(again)
+    planned = d.run_with_ahead()
+    assert all(r.num_output == 9 for r in reqs)
+    # of a request's 8 decode steps, all but the one in which it ends are planned ahead
+    assert planned >= 3 * 5
+
+
+def test_no_step_ahead_when_a_slot_or_the_pages_open_up_for_the_queue():
+    d = ahead_driver(max_seqs=2, num_pages=64)
+    d.submit("a", 6, 3), d.submit("b", 6, 8), d.submit("c", 6, 2)
+    assert d.step_and_ahead()[1] is not None   # a gets the first of its 3 tokens
+    assert d.step_and_ahead()[1] is not None   # ... its second
+    out, ahead = d.step_and_ahead()            # ... its third: it ends with this step
+    assert ahead is None                       # so c takes its slot in the next
+    # a free slot but no pages for the head of the queue: the active request decodes ahead
+    d = ahead_driver(max_seqs=4, num_pages=6, page_size=4)
+    d.submit("a", 9, 6)                        # 3 pages, grows into a fourth
+    d.step_and_ahead()
+    d.submit("big", 13, 2)                     # 4 pages: does not fit beside a
+    out, ahead = d.step_and_ahead()
+    assert [x.request.request_id for x in out.decodes] == ["a"] and not out.portions
+    assert ahead is not None
+    # a head that fits is admitted in the next step: no step ahead
+    d = ahead_driver(max_seqs=4, num_pages=16, page_size=4)
+    d.submit("a", 9, 6)
+    d.step_and_ahead()
+    d.submit("b", 5, 2)
+    out = d.scheduler.schedule()
+    assert [p.request.request_id for p in out.portions] == ["b"]
+    assert d.run_plan(out) is not None         # nothing waits any more
+    d.submit("c", 5, 2)
+    out = d.scheduler.schedule()
+    d.scheduler.queue.append(d.scheduler.active.pop())     # (as if c had come a moment later)
+    d.manager.close("c")
+    out.portions.clear()
+    assert d.run_plan(out) is None             # c fits: the next step admits it
+    # a head that can never be held is aborted by the next schedule: no step ahead either
+    d = ahead_driver(max_seqs=4, num_pages=6, page_size=4)
+    d.submit("a", 9, 6)
+    d.step_and_ahead()
+    out = d.scheduler.schedule()
+    d.submit("never", 40, 2)
+    assert d.run_plan(out) is None
+    d.run_with_ahead()
+    assert [r.request_id for r in d.aborted] == ["never"]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_steps_ahead_under_random_loads_lose_nothing(seed):
+    import random
+    rng = random.Random(seed)
+    d = ahead_driver(max_seqs=rng.choice([1, 2, 3]), num_pages=rng.choice([8, 12, 40]),
+                     page_size=4, max_batched=rng.choice([4, 16, 64]))
+    reqs = [d.submit(f"r{i}", rng.randint(1, 14), rng.randint(1, 12)) for i in range(9)]
+    d.run_with_ahead()
+    for r in reqs:
+        assert r.finish_reason == "length" and r.num_output == r.params.max_tokens

@@ -98,8 +98,10 @@ def test_wide_shape_long_prompt_and_growing_batches(tmp_path, crowd, dtype):
     out = str(tmp_path / "out")
     replay_in_process(folder, steps, out, dtype, rs.max_tokens_needed(steps), max_live=40)
     worst, where = compare(out, steps, reference, 152064)
-    print(f"wide, long prompt and batches, {dtype}: max abs err {worst:.3e} at {where}")
-    assert worst < tolerance(dtype, reference), f"max abs err {worst} at {where}"
+    bar = tolerance(dtype, reference) if dtype == "float32" else \
+        bfloat16_bar(folder, requests, reference, 152064, "crowd")
+    print(f"wide, long prompt and batches, {dtype}: max abs err {worst:.3e} at {where}, bar {bar:.3e}")
+    assert worst < bar, f"max abs err {worst} at {where}, bar {bar}"
 
 
 def test_float32_error_at_depth():

@@ -2,12 +2,15 @@
 static device scratch array inside the library), called through ctypes: its
 tokens equal those of ``sl_sample`` with a workspace, on two calls in a row of
 which the second has the smaller input, for greedy rows, plain draws and rows
-with top-k / top-p cuts; sizes beyond the static array are refused."""
+with top-k / top-p cuts; greedy rows are the argmax and drawn rows the plain
+Gumbel-max draw of tests/emulated_ops.py; sizes beyond the static array are
+refused."""
 import ctypes
 
 import pytest
 import torch
 
+from emulated_ops import perturbed_scores
 from servelab_amd.kernels import build
 
 pytestmark = pytest.mark.gpu
@@ -85,6 +88,14 @@ def test_static_scratch_sampling_equals_sampling_with_a_workspace(mode):
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"{mode} R={R} V={V}: {got.tolist()} vs {want.tolist()}"
         assert int(got.min()) >= 0 and int(got.max()) < V
+        if mode == "draw":                                    # held to the plain draw, not only to sl_sample
+            logits, temperature, _, _, seeds, draws = args
+            for r, tok in enumerate(got.tolist()):
+                if float(temperature[r]) == 0.0:
+                    assert tok == int(logits[r].argmax())
+                    continue
+                scores = perturbed_scores(logits[r], float(temperature[r]), int(seeds[r]), int(draws[r]))
+                assert scores[tok] >= scores.max() - 2e-3, f"R={R} V={V} row {r}"
     if mode == "greedy":
         logits = _inputs(3, 1000, "greedy", 3)[0]
         assert torch.equal(_static(lib, logits, None, None, None, None, None)[1].long(),
