@@ -91,7 +91,9 @@ def time_decode(cfg, model, batch, ctx_end, steps, warmup, page, seed=0):
     prefilled (untimed), then ``warmup`` untimed decode steps, then exactly
     ``steps`` steps between two synchronisations.  The longest context reaches
     ``ctx_end`` at the last step (requests whose prompts were prefilled a step
-    later are a token shorter each).  The engine keeps one decode step
+    later are a token shorter each).  Returns (seconds a step: the region over
+    ``steps``; mean context; the median of the times between the returns of
+    two engine steps, which in the steady state is the median step).  The engine keeps one decode step
     queued ahead of the host; the region starts with that step finished and not
     yet consumed, so exactly ``steps`` steps are queued and finished inside it."""
     import torch
@@ -118,24 +120,28 @@ def time_decode(cfg, model, batch, ctx_end, steps, warmup, page, seed=0):
         engine.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    marks = [t0]
     for _ in range(steps):
         engine.step()
+        marks.append(time.perf_counter())            # a step returns when the step before it has finished
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    gaps = sorted(b - a for a, b in zip(marks, marks[1:]))
     assert engine.num_steps - before == total and len(engine.scheduler.active) == batch
     lengths = [engine.runner.manager.length(r.request_id) for r in engine.scheduler.active]
     assert ctx_end - 2 <= max(lengths) <= ctx_end and min(lengths) >= ctx_end - 2 - batch, lengths
     mean_ctx = sum(lengths) / batch - (steps + 1) / 2.0
     del engine
     torch.cuda.empty_cache()
-    return dt / steps, mean_ctx
+    return dt / steps, mean_ctx, gaps[len(gaps) // 2]
 
 
 def time_prefill(model, T, page, repeats, max_chunk, seed=1, tune=True):
     """A prompt of T tokens from an empty cache, in portions of at most
     ``max_chunk`` tokens (one portion when T fits).  ``tune``: before the
     warm-up run the library's kernels are timed for a portion of that size, as
-    the engine does at start-up with ``tune_products``."""
+    the engine does at start-up with ``tune_products``.  Returns the median
+    and the best of ``repeats`` runs, each between two synchronisations."""
     import torch
     from servelab_amd.engine import ModelRunner, StepEntry
     runner = ModelRunner(model, -(-T // page) + 8, page, max_num_seqs=4)
@@ -157,15 +163,16 @@ def time_prefill(model, T, page, repeats, max_chunk, seed=1, tune=True):
 
     once("w")
     torch.cuda.synchronize()
-    best = float("inf")
+    times = []
     for i in range(repeats):
         t0 = time.perf_counter()
         once(f"p{i}")
         torch.cuda.synchronize()
-        best = min(best, time.perf_counter() - t0)
+        times.append(time.perf_counter() - t0)
     del runner
     torch.cuda.empty_cache()
-    return best
+    times.sort()
+    return times[len(times) // 2], times[0]
 
 
 def main():
@@ -196,7 +203,7 @@ def main():
     itemsize = 2 if short == "bf16" else 4
     page = args.block_size
 
-    step_s, mean_ctx = time_decode(cfg, model, args.batch, args.context, args.steps, args.warmup, page)
+    step_s, mean_ctx, median_s = time_decode(cfg, model, args.batch, args.context, args.steps, args.warmup, page)
     value = args.batch / step_s
     step_bytes = weight_bytes_per_step(cfg, itemsize) + \
         args.batch * mean_ctx * cache_bytes_per_token(cfg, itemsize)
@@ -205,6 +212,7 @@ def main():
     line = {
         "metric": "decode_tokens_per_s", "value": round(value, 2), "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
+        "ms_per_step_median": round(median_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short,
         "data": "synthetic: seeded random weights, prompts of uniform random token ids prefilled "
                 "by the engine up to the context",
@@ -224,14 +232,15 @@ def main():
     }
     if not args.no_prefill:
         T = args.prefill_tokens
-        pre_s = time_prefill(model, T, page, repeats=3, max_chunk=args.prefill_chunk,
-                             tune=not args.no_tune)
+        pre_s, best_s = time_prefill(model, T, page, repeats=5, max_chunk=args.prefill_chunk,
+                                     tune=not args.no_tune)
         line["prefill"] = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
-                           "frac": round(prefill_flops(cfg, T) / pre_s / PEAK_FLOPS[short], 4)}
+                           "frac": round(prefill_flops(cfg, T) / pre_s / PEAK_FLOPS[short], 4),
+                           "timing": "median of 5", "best_ms": round(best_s * 1e3, 3)}
     if not args.no_points:
         points = {}
         for b in (1, 64):
-            s, _ = time_decode(cfg, model, b, args.context, max(5, args.steps // 2), 2, page)
+            s, _, _ = time_decode(cfg, model, b, args.context, max(5, args.steps // 2), 2, page)
             points[f"decode_b{b}"] = round(b / s, 2)
         line["points"] = points
     print(json.dumps(line))

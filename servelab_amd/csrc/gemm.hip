@@ -99,6 +99,7 @@ extern "C" const char* sl_gemm_rows(const void* x, const void* w, const float* b
 #define TM 64
 #define TN 64
 #define TK 16
+#define SEGMENT_K 512      // terms a running sum takes before it is added to the total (a multiple of 16)
 
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(
     const act_t* __restrict__ x, const act_t* __restrict__ w, const float* __restrict__ bias,
@@ -109,13 +110,24 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
   const int tx = tid % 16, ty = tid / 16;          // 4 columns at tx*4, 4 rows at ty*4
   const int lr = tid / 4, lk = (tid % 4) * 4;      // loader: row lr, k offset lk..lk+3
-  float acc[4][4];
+  // Sums of K products in one running float32 sum lose with the length of the sum; the sum is kept
+  // in segments of SEGMENT_K terms, each started from zero and added to the total when it is full.
+  float acc[4][4], total[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = total[i][j] = 0.f;
 
   for (int k0 = 0; k0 < K; k0 += TK) {
+    if (k0 != 0 && k0 % SEGMENT_K == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          total[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = k0 + lk + j;
@@ -146,7 +158,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= N) continue;
-      const float r = acc[i][j] + (bias != nullptr ? bias[n] : 0.f);
+      const float r = total[i][j] + acc[i][j] + (bias != nullptr ? bias[n] : 0.f);
       if (out_f32) ((float*)y)[(size_t)m * N + n] = r;
       else ((act_t*)y)[(size_t)m * N + n] = from_f<act_t>(r);
     }
@@ -211,13 +223,15 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(
     const int n = n0 + r < N ? n0 + r : N - 1;
     wp[i] = w + (size_t)n * K + (idx & 3) * 4;
   }
-  f32x16 acc[TI][TJ];
+  // running sums of SEGMENT_K terms (acc) and the sums of the full ones (total): a sum of 18,944
+  // products in one float32 accumulator loses about six times what 37 sums of 512 lose
+  f32x16 acc[TI][TJ], total[TI][TJ];
 #pragma unroll
   for (int i = 0; i < TI; ++i)
 #pragma unroll
     for (int j = 0; j < TJ; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = total[i][j][r] = 0.f;
   float4 xr[XL], wr[WL];
   auto load = [&](int k0) {
 #pragma unroll
@@ -268,8 +282,22 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
     }
     if (c + 1 < nchunks) store(buf ^ 1);
+    if ((c + 1) % (SEGMENT_K / FK) == 0) {
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+          total[i][j] += acc[i][j];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        }
+    }
     __syncthreads();
   }
+#pragma unroll
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) acc[i][j] += total[i][j];
   // element r of a tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
 #pragma unroll
   for (int j = 0; j < TJ; ++j) {

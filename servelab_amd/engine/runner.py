@@ -39,7 +39,7 @@ class ModelRunner:
         self.manager = CacheManager(model.spec.stream_specs(), num_pages, page_size,
                                     num_state_slots=max_num_seqs)
         self.pool = CachePool(self.manager, self.rt.device, self.rt.act_dtype)
-        self.bindings = [self.pool.binding(c.stream, c.write) for c in model.spec.run]
+        self.bindings = [[self.pool.binding(s, c.write) for s in c.streams] for c in model.spec.run]
         self.max_positions = model.spec.max_position_embeddings
         self.steps = 0
         self.tokens_run = 0

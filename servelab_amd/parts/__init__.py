@@ -1,4 +1,4 @@
-from .base import (Block, FeedForward, Mixer, Norm, PagedKVSpec, ParamSpec, Part,
+from .base import (Block, Embedding, FeedForward, Mixer, Norm, PagedKVSpec, ParamSpec, Part,
                    PositionEncoding, RotaryLayout, RotaryTables, Runtime, StateSpec, prefixed)
 from .norm import RMSNorm
 from .position import NoPosition, RotaryPosition

@@ -164,12 +164,26 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """An arrangement of norms, a mixer and a feed-forward around the residual
-    stream.  ``forward(resid, delta, batch, cache, shared) -> delta``: ``resid``
-    is the float32 stream (updated in place), ``delta`` the not yet added
-    output of what ran before (None at the start)."""
+    """An arrangement of norms, mixers and a feed-forward around the residual
+    stream.  ``cache_specs()`` lists what the block needs cached per request,
+    one entry for each of its parts that caches (none, one, or several: an
+    attention and a state mixer side by side have two); a layer call names one
+    cache stream for each.  ``forward(resid, delta, batch, caches, shared) ->
+    delta``: ``resid`` is the float32 stream (updated in place), ``delta`` the
+    not yet added output of what ran before (None at the start), ``caches`` the
+    bindings of the call's streams in the order of ``cache_specs()``."""
 
-    mixer: Mixer
+    def cache_specs(self):
+        return []
 
-    def forward(self, resid, delta, batch, cache, shared):
+    def forward(self, resid, delta, batch, caches, shared):
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    """forward(batch) -> the float32 residual stream [T, H] of the step's
+    tokens.  The whole batch is at hand: ``batch.ids``, and ``batch.positions``
+    for an embedding that adds a table of absolute positions."""
+
+    def forward(self, batch):
         raise NotImplementedError

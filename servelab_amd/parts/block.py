@@ -21,6 +21,10 @@ class PreNormBlock(Block):
     def _children(self):
         return list(zip(self.names, (self.norm1, self.mixer, self.norm2, self.feedforward)))
 
+    def cache_specs(self):
+        spec = self.mixer.cache_spec()
+        return [] if spec is None else [spec]
+
     def param_specs(self):
         specs = {}
         for prefix, part in self._children():
@@ -33,8 +37,8 @@ class PreNormBlock(Block):
         for prefix, part in self._children():
             part.load(prefixed(prefix, tensors), rt)
 
-    def forward(self, resid, delta, batch, cache, shared):
+    def forward(self, resid, delta, batch, caches, shared):
         x = self.norm1.forward(resid, delta, fuse=self.mixer.takes_scaled_rows)
-        a = self.mixer.forward(x, batch, cache, shared)
+        a = self.mixer.forward(x, batch, caches[0] if caches else None, shared)
         x2 = self.norm2.forward(resid, a, fuse=self.feedforward.takes_scaled_rows)
         return self.feedforward.forward(x2)

@@ -4,10 +4,10 @@ Embedding lookup servelab/parallel/tp_model.py:123; head = embedding table when
 tied, else its own matrix, no bias, logits returned in float32
 (servelab/parallel/tp_model.py:115-119, servelab/engine/engine.py:218).
 """
-from .base import Part, ParamSpec
+from .base import Embedding, Part, ParamSpec
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int):
@@ -20,9 +20,10 @@ class TokenEmbedding(Part):
         self.rt = rt
         self.weight = rt.matrix(tensors("weight"))
 
-    def forward(self, ids):
-        """int32 ids [T] -> float32 residual stream [T, H]."""
-        return self.rt.ops.embed(ids, self.weight)
+    def forward(self, batch):
+        """The rows of the table at ``batch.ids`` (int32 [T]) as the float32
+        residual stream [T, H]."""
+        return self.rt.ops.embed(batch.ids, self.weight)
 
 
 class OutputHead(Part):

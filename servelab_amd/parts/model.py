@@ -9,7 +9,7 @@ twice (each call with a cache stream of its own) or let a call read the stream
 another call wrote.
 """
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, List, Optional, Tuple, Union
 
 import torch
 
@@ -19,11 +19,17 @@ from .base import PagedKVSpec, ParamSpec, Part, Runtime, StateSpec, prefixed
 @dataclass(frozen=True)
 class LayerCall:
     """One entry of the run list: run block ``layer`` against cache stream
-    ``stream``; ``write`` False reads a stream that an earlier call of this
-    step has written."""
+    ``stream``, or against several streams (a tuple) when the block declares
+    several cache needs, one stream for each in the order of its
+    ``cache_specs()``; ``()`` for a block that caches nothing.  ``write`` False
+    reads streams that an earlier call of this step has written."""
     layer: int
-    stream: int
+    stream: Union[int, Tuple[int, ...]] = ()
     write: bool = True
+
+    @property
+    def streams(self) -> Tuple[int, ...]:
+        return (self.stream,) if isinstance(self.stream, int) else tuple(self.stream)
 
 
 @dataclass
@@ -55,21 +61,29 @@ class ModelSpec:
         return specs
 
     def stream_specs(self) -> Dict[int, Any]:
-        """{cache stream: cache spec of the mixer that writes it}."""
+        """{cache stream: the cache need it serves}, from what the blocks of
+        the run list declare (``Block.cache_specs``)."""
+        def needs(call):
+            specs = list(self.layers[call.layer][1].cache_specs())
+            if len(specs) != len(call.streams):
+                raise ValueError(f"layer call of block {call.layer} names {len(call.streams)} cache "
+                                 f"streams, the block declares {len(specs)} cache needs")
+            return zip(call.streams, specs)
         out: Dict[int, Any] = {}
         for call in self.run:
-            spec = self.layers[call.layer][1].mixer.cache_spec()
             if call.write:
-                if call.stream in out:
-                    raise ValueError(f"cache stream {call.stream} is written by two layer calls")
-                out[call.stream] = spec
+                for stream, spec in needs(call):
+                    if stream in out:
+                        raise ValueError(f"cache stream {stream} is written by two layer calls")
+                    out[stream] = spec
         for call in self.run:
             if not call.write:
-                if call.stream not in out:
-                    raise ValueError(f"layer call reads stream {call.stream} that no call writes")
-                if self.layers[call.layer][1].mixer.cache_spec() != out[call.stream]:
-                    raise ValueError(
-                        f"layer {call.layer} reads stream {call.stream} of a different cache kind")
+                for stream, spec in needs(call):
+                    if stream not in out:
+                        raise ValueError(f"layer call reads stream {stream} that no call writes")
+                    if spec != out[stream]:
+                        raise ValueError(
+                            f"layer {call.layer} reads stream {stream} of a different cache kind")
         return out
 
 
@@ -114,14 +128,14 @@ class DecoderModel:
 
     def forward(self, batch, bindings) -> torch.Tensor:
         """Run the batch's tokens through the run list; returns float32 logits
-        [R, V] at ``batch.logit_rows``.  ``bindings[i]`` is the cache binding of
-        ``spec.run[i]``."""
+        [R, V] at ``batch.logit_rows``.  ``bindings[i]`` are the cache bindings of
+        ``spec.run[i]``, one for each of its streams."""
         spec = self.spec
         shared: Dict[Any, Any] = {}
-        resid = spec.embedding[1].forward(batch.ids)
+        resid = spec.embedding[1].forward(batch)
         delta = None
-        for call, binding in zip(spec.run, bindings):
-            delta = spec.layers[call.layer][1].forward(resid, delta, batch, binding, shared)
+        for call, caches in zip(spec.run, bindings):
+            delta = spec.layers[call.layer][1].forward(resid, delta, batch, caches, shared)
         if batch.num_logit_rows == 0:
             # the last block's output is never read; nothing to add
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.rt.device)

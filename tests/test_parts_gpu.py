@@ -90,7 +90,8 @@ def test_embedding_and_head_parts(rt):
     emb = TokenEmbedding(1000, 72)
     t = load(emb, {"weight": rand(1000, 72, seed=1)}, runtime)
     ids = torch.tensor([0, 999, 5], dtype=torch.int32).cuda()
-    assert torch.equal(emb.forward(ids).cpu(), t["weight"][[0, 999, 5]])
+    import types
+    assert torch.equal(emb.forward(types.SimpleNamespace(ids=ids)).cpu(), t["weight"][[0, 999, 5]])
     x = rand(4, 72, seed=2).to(runtime.act_dtype)
     tied = OutputHead(1000, 72, tied_to=emb)
     assert tied.param_specs() == {}
@@ -165,7 +166,7 @@ def test_block_part(rt):
                     "mlp.down_proj.weight": rand(H, I, scale=0.1, seed=13)})
     assert set(block.param_specs()) == set(tensors)
     t = load(block, tensors, runtime)
-    manager = CacheManager({0: block.mixer.cache_spec()}, num_pages=4, page_size=16)
+    manager = CacheManager({0: block.cache_specs()[0]}, num_pages=4, page_size=16)
     pool = CachePool(manager, runtime.device, runtime.act_dtype)
     manager.open("r")
     manager.grow("r", T)
@@ -173,7 +174,7 @@ def test_block_part(rt):
     h = rand(T, H, seed=20)
     pending = rand(T, H, scale=0.1, seed=21).to(runtime.act_dtype)
     resid = h.cuda()
-    delta = runtime.ops.materialize(block.forward(resid, pending.cuda(), batch, pool.binding(0, True), {}))
+    delta = runtime.ops.materialize(block.forward(resid, pending.cuda(), batch, [pool.binding(0, True)], {}))
     h0 = h + pending.float()
     att = {n[len("self_attn."):]: v for n, v in t.items() if n.startswith("self_attn.")}
     h1 = h0 + plain_attention_layer(plain.rms_norm(h0, t["input_layernorm.weight"], 1e-6), att,

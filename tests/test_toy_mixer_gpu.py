@@ -13,9 +13,9 @@ from servelab_amd import LLMEngine, CacheConfig, SamplingParams, SchedulerConfig
     register_architecture, write_random_model
 from servelab_amd.engine import ModelRunner, StepEntry
 from servelab_amd.engine.session import load_model_on_device
-from servelab_amd.parts import (GatedMLP, LayerCall, Mixer, ModelSpec, OutputHead, PagedAttention,
-                                ParamSpec, PreNormBlock, RMSNorm, RotaryPosition, StateSpec,
-                                TokenEmbedding)
+from servelab_amd.parts import (Block, Embedding, GatedMLP, LayerCall, Mixer, ModelSpec, NoPosition,
+                                OutputHead, PagedAttention, ParamSpec, PreNormBlock, RMSNorm,
+                                RotaryPosition, StateSpec, TokenEmbedding, prefixed)
 
 pytestmark = pytest.mark.gpu
 
@@ -63,7 +63,8 @@ class ToyConfig:
 
     @classmethod
     def from_hf(cls, raw, path=""):
-        return cls(raw["hidden_size"], raw["vocab_size"], raw["decay"], raw.get("torch_dtype", "float32"), path=path)
+        return cls(raw["hidden_size"], raw["vocab_size"], raw["decay"], raw.get("torch_dtype", "float32"),
+                   raw["architectures"][0], path=path)
 
     def to_hf(self):
         return {"architectures": [self.architecture], "hidden_size": self.hidden_size,
@@ -164,3 +165,134 @@ def test_toy_architecture_generates_through_the_engine(tmp_path):
         for t in o.outputs[0].token_ids:
             assert t == int(torch.argmax(plain_toy(cfg, w, toks)[-1]))
             toks.append(t)
+
+
+# ------------------------------------------------- two mixers in a block, positions at the embedding
+class PositionTableEmbedding(Embedding):
+    """Token row plus the row of a learned table at the token's absolute position."""
+
+    def __init__(self, vocab_size, hidden_size, positions):
+        self.vocab_size, self.hidden_size, self.positions = vocab_size, hidden_size, positions
+
+    def param_specs(self):
+        return {"tokens.weight": ParamSpec((self.vocab_size, self.hidden_size)),
+                "positions.weight": ParamSpec((self.positions, self.hidden_size))}
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        self.tokens = tensors("tokens.weight").to(rt.device, torch.float32)
+        self.table = tensors("positions.weight").to(rt.device, torch.float32)
+
+    def forward(self, batch):
+        return self.tokens[batch.ids.long()] + self.table[batch.positions.long()]
+
+
+class SideBySideBlock(Block):
+    """h += Attention(Norm(h)) + State(Norm(h)); h += FeedForward(Norm2(h)): two parts that
+    cache, a paged one and one with a state slot, in one layer."""
+
+    def __init__(self, norm1, attention, state, norm2, feedforward):
+        self.parts = [("norm1.", norm1), ("attn.", attention), ("state.", state), ("norm2.", norm2),
+                      ("ffn.", feedforward)]
+        self.norm1, self.attention, self.state, self.norm2, self.feedforward = \
+            norm1, attention, state, norm2, feedforward
+
+    def cache_specs(self):
+        return [self.attention.cache_spec(), self.state.cache_spec()]
+
+    def param_specs(self):
+        return {prefix + n: s for prefix, part in self.parts for n, s in part.param_specs().items()}
+
+    def load(self, tensors, rt):
+        self.rt = rt
+        for prefix, part in self.parts:
+            part.load(prefixed(prefix, tensors), rt)
+
+    def forward(self, resid, delta, batch, caches, shared):
+        pages, slots = caches
+        x = self.norm1.forward(resid, delta)
+        a = self.rt.ops.materialize(self.attention.forward(x, batch, pages, shared))
+        both = (a.float() + self.state.forward(x, batch, slots, shared).float()).to(x.dtype)
+        return self.feedforward.forward(self.norm2.forward(resid, both))
+
+
+@dataclass
+class SideBySideConfig(ToyConfig):
+    architecture: str = "ToySideBySideForCausalLM"
+
+
+def build_side_by_side(cfg):
+    h = cfg.hidden_size
+
+    def block(decay):
+        return SideBySideBlock(RMSNorm(h, 1e-6), PagedAttention(h, 3, 1, 16, NoPosition(), qkv_bias=False),
+                               DecayingSumMixer(h, decay), RMSNorm(h, 1e-6), GatedMLP(h, 80))
+    return ModelSpec(("emb.", PositionTableEmbedding(cfg.vocab_size, h, 128)),
+                     [("layers.0.", block(cfg.decay)), ("layers.1.", block(0.5))],
+                     [LayerCall(0, (0, 1)), LayerCall(1, (2, 3))],
+                     ("final_norm.", RMSNorm(h, 1e-6)), ("out.", OutputHead(cfg.vocab_size, h)),
+                     cfg.vocab_size, h, eos_token_id=-1, max_position_embeddings=128)
+
+
+def plain_side_by_side(cfg, w, toks):
+    import math
+    import plain_qwen2 as plain
+    T, h = len(toks), cfg.hidden_size
+    pos = torch.arange(T)
+    x = w["emb.tokens.weight"][toks] + w["emb.positions.weight"][:T]
+    for p, decay in (("layers.0.", cfg.decay), ("layers.1.", 0.5)):
+        n = plain.rms_norm(x, w[p + "norm1.weight"], 1e-6)
+        q = (n @ w[p + "attn.q_proj.weight"].T).view(T, 3, 16)
+        k = (n @ w[p + "attn.k_proj.weight"].T).view(T, 1, 16)
+        v = (n @ w[p + "attn.v_proj.weight"].T).view(T, 1, 16)
+        a = plain.attention(q, k, v, 1 / math.sqrt(16), pos, pos).reshape(T, 48) @ w[p + "attn.o_proj.weight"].T
+        u = n @ w[p + "state.in_proj.weight"].T
+        s, ys = torch.zeros(h), []
+        for t in range(T):
+            s = decay * s + u[t]
+            ys.append(s)
+        x = x + a + torch.stack(ys)
+        x = x + plain.swiglu(plain.rms_norm(x, w[p + "norm2.weight"], 1e-6), w[p + "ffn.gate_proj.weight"],
+                             w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+    return plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["out.weight"].T
+
+
+def test_a_block_with_two_caching_parts_and_an_embedding_that_reads_positions(tmp_path):
+    """Attention without position encoding and a state mixer side by side in every block (two cache
+    streams a layer call: pages and a state slot), positions added once at the embedding: registered,
+    built and stepped in portions, two requests side by side, with nothing changed in the framework."""
+    register_architecture("ToySideBySideForCausalLM", SideBySideConfig.from_hf, build_side_by_side)
+    folder = write_random_model(SideBySideConfig(), str(tmp_path / "toy"), seed=6, std=0.1)
+    cfg = load_config(folder)
+    assert cfg.architecture == "ToySideBySideForCausalLM"
+    _, model = load_model_on_device(folder, "float32")
+    assert sorted(model.spec.stream_specs()) == [0, 1, 2, 3]
+    runner = ModelRunner(model, num_pages=8, page_size=16, max_num_seqs=2)
+    m = runner.manager
+    assert len(m.page_groups) == 1 and m.page_groups[0].streams == [0, 2]
+    assert len(m.state_groups) == 1 and m.state_groups[0].streams == [1, 3]
+    from safetensors.torch import load_file
+    w = {k: v.float() for k, v in load_file(folder + "/model.safetensors").items()}
+    gen = torch.Generator().manual_seed(2)
+    seqs = {r: torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for r, n in (("a", 45), ("b", 28))}
+    ref = {r: plain_side_by_side(cfg, w, t) for r, t in seqs.items()}
+    plan = [[("a", 0, 19), ("b", 0, 3)], [("a", 19, 20), ("b", 3, 17)], [("a", 20, 45), ("b", 17, 18)],
+            [("b", 18, 28)]]
+    worst = 0.0
+    for step in plan:
+        out = runner.step([StepEntry(r, seqs[r][a:b], list(range(b - a))) for r, a, b in step])
+        row = 0
+        for r, a, b in step:
+            worst = max(worst, (out[row:row + b - a].cpu() - ref[r][a:b]).abs().max().item())
+            row += b - a
+    assert worst < 1e-4, worst
+    # a position the table does not hold is past max_position_embeddings: refused by the step function
+    runner.close("a")
+    with pytest.raises(ValueError, match="max_position_embeddings"):
+        runner.step([StepEntry("c", [1] * 129, [])])
+    runner.close("c"), runner.close("b")
+    m.check()
+    with pytest.raises(ValueError, match="names 1 cache streams, the block declares 2"):
+        spec = build_side_by_side(cfg)
+        spec.run[0] = LayerCall(0, 0)
+        spec.stream_specs()

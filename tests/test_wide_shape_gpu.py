@@ -110,9 +110,11 @@ def test_float32_error_at_depth():
     on the device and shared by both sides; the plain implementation runs on the device in float64
     and in float32 (library products, no reduced-precision mode), the latter to show what float32
     arithmetic itself costs at that depth.  Prompt of 48 tokens, then 16 tokens one by one.
-    Up to 8 layers the error stays below 1e-4; at every depth it stays within 1.5 times what the
-    plain implementation loses by computing in float32 itself (it grows like the square root of
-    the depth for both)."""
+    At every depth the error stays below 1e-4 (the bar of the reference's own cross-checks,
+    tests/test_parallel.py:103-104) and below what the plain implementation loses by computing
+    in float32 itself: the kernels keep their sums of products in segments of 512 terms (and a
+    wavefront's lanes each their own share), where a running sum over 3,584 to 18,944 terms
+    loses more.  The error grows like the square root of the depth for both."""
     import plain_qwen2 as plain
     from servelab_amd.engine import ModelRunner, StepEntry
     from servelab_amd.engine.session import random_model_on_device
@@ -139,5 +141,5 @@ def test_float32_error_at_depth():
     for layers, (engine, arithmetic, top) in report.items():
         print(f"float32 at {layers} layers of the 7B widths: engine {engine:.2e}, plain float32 "
               f"{arithmetic:.2e} off the float64 logits (largest {top:.2f})")
-    assert all(report[layers][0] <= 1e-4 for layers in (2, 4, 8)), report
-    assert all(engine <= 1.5 * arithmetic for engine, arithmetic, _ in report.values()), report
+    assert all(engine <= 1e-4 for engine, _, _ in report.values()), report
+    assert all(engine <= arithmetic for engine, arithmetic, _ in report.values()), report
