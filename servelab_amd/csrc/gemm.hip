@@ -263,41 +263,39 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(
   __syncthreads();
   // operand element of this lane in a 32 x 2 step: row lane % 32, k lane / 32
   const int orow = lane & 31, ok = lane >> 5;
-  for (int c = 0; c < nchunks; ++c) {
-    const int buf = c & 1;
-    if (c + 1 < nchunks) load((c + 1) * FK);
-    const float* xa = &xs[buf][(wm * 32 * TI + orow) * FS + ok];
-    const float* wb = &ws[buf][(wn * 32 * TJ + orow) * FS + ok];
+  constexpr int SEG = SEGMENT_K / FK;                 // chunks a running sum takes
+  for (int c0 = 0; c0 < nchunks; c0 += SEG) {
+    const int c1 = c0 + SEG < nchunks ? c0 + SEG : nchunks;
+    for (int c = c0; c < c1; ++c) {
+      const int buf = c & 1;
+      if (c + 1 < nchunks) load((c + 1) * FK);
+      const float* xa = &xs[buf][(wm * 32 * TI + orow) * FS + ok];
+      const float* wb = &ws[buf][(wn * 32 * TJ + orow) * FS + ok];
 #pragma unroll
-    for (int kk = 0; kk < FK; kk += 2) {
-      float a[TI], b[TJ];
+      for (int kk = 0; kk < FK; kk += 2) {
+        float a[TI], b[TJ];
 #pragma unroll
-      for (int i = 0; i < TI; ++i) a[i] = xa[32 * i * FS + kk];
+        for (int i = 0; i < TI; ++i) a[i] = xa[32 * i * FS + kk];
 #pragma unroll
-      for (int j = 0; j < TJ; ++j) b[j] = wb[32 * j * FS + kk];
+        for (int j = 0; j < TJ; ++j) b[j] = wb[32 * j * FS + kk];
 #pragma unroll
-      for (int i = 0; i < TI; ++i)
+        for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < TJ; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < TJ; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+      }
+      if (c + 1 < nchunks) store(buf ^ 1);
+      __syncthreads();
     }
-    if (c + 1 < nchunks) store(buf ^ 1);
-    if ((c + 1) % (SEGMENT_K / FK) == 0) {
 #pragma unroll
-      for (int i = 0; i < TI; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-          total[i][j] += acc[i][j];
+      for (int j = 0; j < TJ; ++j) {
+        total[i][j] += acc[i][j];
 #pragma unroll
-          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-        }
-    }
-    __syncthreads();
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      }
   }
-#pragma unroll
-  for (int i = 0; i < TI; ++i)
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) acc[i][j] += total[i][j];
   // element r of a tile: row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
 #pragma unroll
   for (int j = 0; j < TJ; ++j) {
@@ -309,7 +307,7 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + (wm * TI + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m < M) y[(size_t)m * N + n] = acc[i][j][r] + bv;
+        if (m < M) y[(size_t)m * N + n] = total[i][j][r] + bv;
       }
   }
 }
@@ -939,11 +937,22 @@ static int resident_workgroups(Kernel kernel) {
   return device_cus() * per_cu;
 }
 
-// Whether sl_gemm_resident has a kernel for rows of K values (K = 256 * steps for one of
-// the step counts it is built for).
-extern "C" int sl_gemm_resident_takes(int K) {
+// The row lengths sl_gemm_resident is built for (K = 256 * NS: the number of k-steps a
+// wavefront takes is a template argument, so that the compiler can count the loads in
+// flight), each with the number of k-steps R a wavefront asks for at once.  They are the
+// widths whose consumers have many tiles per CU among the models this was measured on
+// (1536, 2048, 3584, 4096, 5120); every other K, and K = 8192, where this form measured
+// slower, takes sl_gemm_skinny, which gives the same result bit for bit.
+#define SL_RESIDENT_WIDTHS(X) X(6, 6) X(8, 8) X(14, 14) X(16, 16) X(20, 10)
+constexpr int resident_parts_per_thread(int NS) { return NS <= 16 ? 8 : 16; }
+
+// How many sums of squares a row (K / 16 or more) the kernel for rows of K values adds up,
+// 0 when sl_gemm_resident has no kernel for that K.
+extern "C" int sl_gemm_resident_parts(int K) {
   switch (K) {
-    case 256 * 6: case 256 * 8: case 256 * 14: case 256 * 16: case 256 * 20: return 1;
+#define SL_CASE(NS, R) case 256 * NS: return 32 * resident_parts_per_thread(NS);
+    SL_RESIDENT_WIDTHS(SL_CASE)
+#undef SL_CASE
     default: return 0;
   }
 }
@@ -956,7 +965,7 @@ extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const flo
                                         const int* rows, int x_tiled, int y_tiled, hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_resident: sizes must be positive");
   SL_CHECK(M <= 16, "gemm_resident: at most 16 rows");
-  SL_CHECK(sl_gemm_resident_takes(K), "gemm_resident: no kernel for rows of this length");
+  SL_CHECK(sl_gemm_resident_parts(K) > 0, "gemm_resident: no kernel for rows of this length");
   SL_CHECK(!gated || (N % 16 == 0 && bias == nullptr && !out_f32),
            "gemm_resident: the gated form needs N % 16 == 0, no bias, activation output");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wt % 16) == 0,
@@ -973,7 +982,7 @@ extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const flo
   const __bf16* ww = (const __bf16*)wt;
 #define SL_RESIDENT(G, NS, R)                                                                   \
   do {                                                                                          \
-    constexpr int PARTS = NS <= 16 ? 8 : 16;          /* K / 16 parts or more, 32 per pass */   \
+    constexpr int PARTS = resident_parts_per_thread(NS);   /* K / 16 parts or more, 32 per pass */ \
     SL_CHECK(in_nparts <= 32 * PARTS, "gemm_resident: more sums of squares a row than this form adds up"); \
     static int slots = 0;                                                                       \
     if (slots == 0) slots = resident_workgroups(gemm_resident_kernel<G, PARTS, NS, R>);         \
@@ -986,14 +995,8 @@ extern "C" const char* sl_gemm_resident(const void* x, const void* wt, const flo
 #define SL_RESIDENT_CASE(NS, R)                                     \
   case 256 * NS:                                                    \
     if (gated) SL_RESIDENT(true, NS, R); else SL_RESIDENT(false, NS, R); \
-    break
-  switch (K) {
-    SL_RESIDENT_CASE(6, 6);
-    SL_RESIDENT_CASE(8, 8);
-    SL_RESIDENT_CASE(14, 14);
-    SL_RESIDENT_CASE(16, 16);
-    SL_RESIDENT_CASE(20, 10);
-  }
+    break;
+  switch (K) { SL_RESIDENT_WIDTHS(SL_RESIDENT_CASE) }
 #undef SL_RESIDENT_CASE
 #undef SL_RESIDENT
   return sl_launch_status();

@@ -554,7 +554,7 @@ class HipOps:
         if bias is not None:
             self._check(bias, torch.float32, (N,), "bias")
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
-        if self._takes_resident(N, K) and xs.parts.shape[0] <= 32 * (8 if K <= 4096 else 16):
+        if self._takes_resident(N, K, xs.parts.shape[0]):
             self._call("gemm", "sl_gemm_resident", _p(xs.x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                        int(out_f32), int(gated), _p(xs.parts), xs.parts.shape[0], _c_float(xs.eps),
                        _p(xs.rows), int(xs.tiled), int(y_tiled))
@@ -562,16 +562,18 @@ class HipOps:
             self._skinny(xs.x, weight, bias, y, M, N, K, out_f32, gated, scaled=xs, y_tiled=y_tiled)
         return TiledRows(y, (M, N // 2)) if y_tiled else y
 
-    def _takes_resident(self, N, K) -> bool:
+    def _takes_resident(self, N, K, parts) -> bool:
         """Whether a consumer product runs on the workgroups that stay and walk the tiles
         (x in registers, row scales computed once): matrices with several tiles per CU whose
-        row length the kernel is built for."""
+        row length the kernel is built for (the library says which: ``sl_gemm_resident_parts``,
+        the most sums of squares a row its kernel for K adds up, 0 for no kernel).  Every other
+        width takes the workgroup-per-tile kernel, which gives the same result bit for bit."""
         if -(-N // 16) < self.RESIDENT_MIN_ROUNDS * self._num_cus:
             return False
-        takes = self._resident_k.get(K)
-        if takes is None:
-            takes = self._resident_k[K] = bool(self._lib["gemm"].sl_gemm_resident_takes(K))
-        return takes
+        most = self._resident_k.get(K)
+        if most is None:
+            most = self._resident_k[K] = int(self._lib["gemm"].sl_gemm_resident_parts(K))
+        return 0 < parts <= most
 
     GATE_BLOCK = 8                # gate and up rows alternate in blocks of 8 (half an MFMA tile)
 

@@ -393,8 +393,11 @@ def test_consumer_products_on_workgroups_that_stay(M, H, N2):
     from servelab_amd.kernels import HipOps, KernelError
     from servelab_amd.kernels.ops import ScaledRows
     ops = HipOps(torch.bfloat16, "cuda:0")
-    assert ops._takes_resident(1 << 20, H) and not ops._takes_resident(1 << 20, H + 32)
-    assert not ops._takes_resident(16 * ops._num_cus, H)
+    np_ = -(-H // 16)
+    assert ops._takes_resident(1 << 20, H, np_) and not ops._takes_resident(1 << 20, H + 32, np_ + 2)
+    assert not ops._takes_resident(1 << 20, 8192, 512)        # measured slower there: not built
+    assert not ops._takes_resident(16 * ops._num_cus, H, np_) and not ops._takes_resident(1 << 20, H, 1 << 20)
+    routed = ops._takes_resident
     x = randn(M, H, dtype=torch.bfloat16, seed=1)
     parts = randn(-(-H // 16), 16, seed=2).abs().contiguous()
     w2 = ops.prepare_weight(randn(N2, H, dtype=torch.bfloat16, scale=0.05, seed=5))
@@ -404,7 +407,7 @@ def test_consumer_products_on_workgroups_that_stay(M, H, N2):
              (ScaledRows(x, parts, 1e-5, rows), None, True)]
     got = {}
     for stay in (False, True):
-        ops._takes_resident = lambda N, K, stay=stay: stay
+        ops._takes_resident = lambda N, K, parts, stay=stay: stay
         got[stay] = [ops.linear(xs, w2, b, out_f32=f32) for xs, b, f32 in cases]
         if N2 % 16 == 0:
             got[stay].append(ops.gated_linear(ScaledRows(x, parts, 1e-5), w2, 8))
@@ -420,8 +423,14 @@ def test_consumer_products_on_workgroups_that_stay(M, H, N2):
     ref = (x.float() @ w2.w.float().T) * inv[:, None] + b2
     assert rel_err(got[True][0], ref) < 2 ** -6
     odd = ScaledRows(randn(M, H + 32, dtype=torch.bfloat16, seed=1), randn(-(-(H + 32) // 16), 16, seed=2).abs(), 1e-5)
+    w_odd = ops.prepare_weight(randn(16 * 3 * ops._num_cus + 16, H + 32, dtype=torch.bfloat16, scale=0.05, seed=3))
     with pytest.raises(KernelError, match="no kernel for rows of this length"):
-        ops.linear(odd, ops.prepare_weight(randn(32, H + 32, dtype=torch.bfloat16, seed=3)), None)
+        ops.linear(odd, w_odd, None)
+    # left to itself the kernel table sends a width the kernel is not built for to the workgroup-per-tile
+    # kernel, however many tiles the matrix has
+    ops._takes_resident = routed
+    inv = torch.rsqrt(odd.parts.sum(0)[:M] / (H + 32) + 1e-5)
+    assert rel_err(ops.linear(odd, w_odd, None, out_f32=True), (odd.x.float() @ w_odd.w.float().T) * inv[:, None]) < 2 ** -6
 
 
 @pytest.mark.parametrize("M,H,I", [(2, 256, 64), (8, 3584, 18944), (16, 2048, 96), (5, 96, 160), (13, 512, 4128)])
