@@ -159,7 +159,8 @@ def build_engine(args):
                             max_num_batched_tokens=args.max_batched_tokens,
                             chunked_prefill=not args.no_chunked_prefill,
                             policy=args.scheduler_policy)
-    warm = dict(tune_products=tune_option(args), capture_graphs_up_to=args.capture_graphs_up_to)
+    warm = dict(tune_products=tune_option(args), capture_graphs_up_to=args.capture_graphs_up_to,
+                run_ahead=not args.no_run_ahead)
     if args.model:
         cfg = load_config(args.model)
         return cfg, LLMEngine(cfg, cache, sched, dtype=args.dtype, **warm)
@@ -200,7 +201,7 @@ def run(args) -> dict:
         "output_tokens": args.output_tokens, "max_num_seqs": args.max_num_seqs,
         "max_batched_tokens": args.max_batched_tokens, "block_size": args.block_size,
         "num_blocks": engine.num_blocks, "temperature": args.temperature, "top_p": args.top_p,
-        "top_k": args.top_k,
+        "top_k": args.top_k, "run_ahead": not args.no_run_ahead,
     }
     return res
 
@@ -238,6 +239,8 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--tune-products", action="store_true")
     ap.add_argument("--capture-graphs-up-to", type=int, default=0,
                     help="capture decode graphs for contexts up to this length before the clock starts")
+    ap.add_argument("--no-run-ahead", action="store_true",
+                    help="wait for every step's tokens before the next step is planned")
     ap.add_argument("--tune-rows", default="", help="further step sizes (rows) to tune the library products for")
     return ap
 
