@@ -1567,4 +1567,187 @@ extern "C" const char* sl_untile_weight(const void* wt, void* w, int N, int K, i
       (const __bf16*)wt, (__bf16*)w, N, K, th, total_vec);
   return sl_launch_status();
 }
+
+// ------------------------------------------------- 129 rows and more, matrix cores
+// y[M, N] = x[M, K] W[N, K]^T for steps of a few hundred rows (a newcomer's prompt beside decoded
+// tokens) and matrices of few rows (q/k/v, o, down), where the product is neither bound by
+// streaming W (the kernels above) nor large enough for the tiles of a library kernel to fill the
+// chip.  Both operands are row-major; a workgroup of WM x WN wavefronts owns a tile of 64 WM rows
+// of x by 64 WN rows of W over a share of K (grid.z shares write float partial sums [KS, M, N]
+// that the reader or splitk_reduce adds), a wavefront 64 x 64 of it (16 matrix instructions per
+// 8 operand reads).
+//
+// Chunks of 64 values of k travel from global memory straight into a ring of three LDS stages
+// (global_load_lds_dwordx4: a wavefront's 64 loads of 16 bytes land side by side in 1 KB), two
+// chunks in flight while the third is multiplied: at the 50 GB/s a CU pulls and 2 us of loaded
+// latency that is what keeps the stream going.  A stage holds the rows of x, then those of W, 8
+// units of 16 bytes a row; a lane can put any unit anywhere at no cost, so unit c of row r lies
+// at place c ^ f(r), f(r) = ((r >> 1) & 7) ^ 4 (r & 1): the 16 lanes that read one operand
+// column (rows r .. r + 15, same c) then touch 16 different 16-byte slots of a 256-byte line of
+// banks, and each half of them 8 different slots of a 128-byte one.
+__device__ __forceinline__ void block_load_to_lds(const void* from, unsigned lds_at) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(from), "s"(lds_at) : "m0");
+}
+template <int N_> __device__ __forceinline__ void block_wait_loads() {
+  __builtin_amdgcn_s_waitcnt((N_ & 15) | (7 << 4) | (15 << 8) | ((N_ >> 4) << 14));
+}
+
+template <int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
+    const __bf16* __restrict__ x, const __bf16* __restrict__ w, const float* __restrict__ bias,
+    void* __restrict__ y, int M, int N, int K, int out_f32, int KS) {
+  constexpr int WAVES = WM * WN, BM = 64 * WM, BN = 64 * WN, STAGES = 3;
+  constexpr int ROWS = BM + BN;                      // rows of a stage: x, then W; 128 bytes each
+  constexpr int STAGE_BYTES = ROWS * 128;
+  constexpr int LOADS = ROWS / 8 / WAVES;            // wavefront-wide loads (8 rows) a wavefront makes per chunk
+  static_assert(LOADS * 8 * WAVES == ROWS, "the rows of a stage must divide evenly over the wavefronts");
+  __shared__ __attribute__((aligned(1024))) char ring[STAGES * STAGE_BYTES];
+  const int t = threadIdx.x, lane = t & 63, i = lane & 15, gq = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int chunks = K / 64;
+  const int cbeg = (int)((long long)chunks * blockIdx.z / KS);
+  const int cend = (int)((long long)chunks * (blockIdx.z + 1) / KS);
+
+  // what this lane fetches of every chunk: unit `cu ^ f(row)` of row 8 q + lane / 8 of the stage
+  const __bf16* src[LOADS];
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) {
+    const int row = 8 * (wave + WAVES * j) + (lane >> 3);
+    const int c = (lane & 7) ^ (((row >> 1) & 7) ^ (4 * (row & 1)));
+    if (row < BM) {
+      const int m = m0 + row < M ? m0 + row : M - 1;           // rows past the end: the last row again, never stored
+      src[j] = x + (size_t)m * K + 8 * c;
+    } else {
+      const int n = n0 + row - BM < N ? n0 + row - BM : N - 1;
+      src[j] = w + (size_t)n * K + 8 * c;
+    }
+  }
+  const unsigned ring_at = (unsigned)(size_t)(__attribute__((address_space(3))) char*)ring;
+  auto fetch = [&](int c, int stage) {
+    const unsigned at = ring_at + STAGE_BYTES * stage + 1024 * wave;
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) block_load_to_lds(src[j] + 64 * (size_t)c, at + 1024 * WAVES * j);
+  };
+  // where this lane reads its operands: row R0 + i (R0 a multiple of 16), unit 4 kk + gq
+  int at_kk[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) at_kk[kk] = 128 * i + 16 * ((4 * kk + gq) ^ (((i >> 1) & 7) ^ (4 * (i & 1))));
+
+  f32x4 acc[4][4];                                   // [tile of W rows][tile of x rows]
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (cbeg < cend) {
+    fetch(cbeg, 0);
+    if (cbeg + 1 < cend) {
+      fetch(cbeg + 1, 1);
+      block_wait_loads<LOADS>();
+    } else {
+      block_wait_loads<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" : : : "memory");
+  }
+  int stage = 0;
+  for (int c = cbeg; c < cend; ++c) {
+    const bool more = c + 2 < cend;
+    if (more) fetch(c + 2, stage >= 1 ? stage - 1 : 2);        // the stage the last chunk was read from
+    const char* st = ring + STAGE_BYTES * stage;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      bf16x8 a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = *(const bf16x8*)(st + 128 * (BM + 64 * wn + 16 * u) + at_kk[kk]);
+        b[u] = *(const bf16x8*)(st + 128 * (64 * wm + 16 * u) + at_kk[kk]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          acc[u][v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[v], acc[u][v], 0, 0, 0);
+    }
+    if (more) block_wait_loads<LOADS>();                       // all but the chunk just asked for
+    else block_wait_loads<0>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" : : : "memory");
+    stage = stage == 2 ? 0 : stage + 1;
+  }
+
+  // lane: row m of x (16 v + i), four consecutive rows n of W (16 u + 4 gq ..)
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const int m = m0 + 64 * wm + 16 * v + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int n = n0 + 64 * wn + 16 * u + 4 * gq;
+      if (n >= N) continue;
+      const bool whole = n + 3 < N && N % 4 == 0;
+      f32x4 r = acc[u][v];
+      if (KS > 1) {
+        float* o = (float*)y + ((size_t)blockIdx.z * M + m) * N + n;
+        if (whole) {
+          *(f32x4*)o = r;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) o[e] = r[e];
+        }
+        continue;
+      }
+      if (bias != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) r[e] += bias[n + e];
+      }
+      if (whole && out_f32) {
+        *(f32x4*)((float*)y + (size_t)m * N + n) = r;
+      } else if (whole) {
+        bf16x4 h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = (__bf16)r[e];
+        *(bf16x4*)((__bf16*)y + (size_t)m * N + n) = h;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (n + e >= N) continue;
+          if (out_f32) ((float*)y)[(size_t)m * N + n + e] = r[e];
+          else ((__bf16*)y)[(size_t)m * N + n + e] = (__bf16)r[e];
+        }
+      }
+    }
+  }
+}
+
+// x and W row-major.  ks > 1: `part` holds ks * M * N floats; with y == nullptr they are left
+// there for the reader to add (and the bias with them), else splitk_reduce adds them into y.
+extern "C" const char* sl_gemm_block(const void* x, const void* w, const float* bias, void* y,
+                                     int M, int N, int K, int out_f32, int ks, float* part,
+                                     hipStream_t stream) {
+  SL_CHECK(M > 0 && N > 0 && K > 0, "gemm_block: sizes must be positive");
+  SL_CHECK(K % 64 == 0, "gemm_block: K must be a multiple of 64");
+  SL_CHECK(ks >= 1 && ks <= 64 && ks <= K / 64, "gemm_block: ks must be in 1..64 and <= K / 64");
+  SL_CHECK(ks == 1 || part != nullptr, "gemm_block: a split of K needs the partial buffer");
+  SL_CHECK(y != nullptr || ks > 1, "gemm_block: no output");
+  SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_block: x and W must be 16-byte aligned");
+  void* dst = ks > 1 ? (void*)part : y;
+  const __bf16* xx = (const __bf16*)x;
+  const __bf16* ww = (const __bf16*)w;
+  // (Tiles of 64 x 256 and 128 x 256 for fewer rows of x were built and measured: alone they beat the
+  // LDS-staged kernel above, in a decode step of 24 to 128 requests they lost 2-5 % tokens/s to it,
+  // so that kernel keeps those rows and this one starts where it ends.)
+  const dim3 grid((N + 127) / 128, (M + 255) / 256, ks);
+  SL_CHECK(grid.y <= 65535, "gemm_block: too many rows");
+  gemm_block_kernel<4, 2><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, ks);
+  const char* e = sl_launch_status();
+  if (e || ks == 1 || y == nullptr) return e;
+  const size_t total = (size_t)M * N;
+  splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(part, bias, y, M, N, ks, out_f32);
+  return sl_launch_status();
+}
 #endif

@@ -170,6 +170,7 @@ class HipOps:
                      for stem in build.DEFAULT_STEMS}
         self._fn = {}
         self.use_mfma_attention = True
+        self.use_block_products = act_dtype == torch.bfloat16  # products in tiles over the row-major copy (gemm_block)
         self._num_cus = max(1, torch.cuda.get_device_properties(self.device).multi_processor_count)
         self._resident_k = {}
         self.fuse_norms = act_dtype == torch.bfloat16
@@ -459,6 +460,11 @@ class HipOps:
                 return self.linear_f32_mfma(x, weight.w, bias)
             return self.linear_tiled(x, weight.w, bias, out_f32)
         limit = self._few_rows_limit(weight)
+        shares = self._block_shares(M, N, K, weight)
+        if shares:
+            # (deferred: the norm adds the partial sums)
+            return self.linear_block(x, weight, bias, out_f32, shares,
+                                     partial=defer and self.fuse_norms and not out_f32)
         if (defer and self.fuse_norms and not out_f32 and self.WIDE_MIN_M <= M <= limit
                 and K % 32 == 0 and N % 4 == 0 and self._takes_mid(M, N, K)):
             return self.linear_mid(x, weight, bias, partial=True,     # the norm adds the partial sums
@@ -529,6 +535,49 @@ class HipOps:
         y = self._new((M, N // 2 if gated else N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_mid", _p(x), _p(weight.tiled), _p(bias), _p(y), M, N, K,
                    int(out_f32), int(gated), int(ks), self.MID_WIDE_WORKGROUPS, self._num_cus, _p(part))
+        return y
+
+    def _block_shares(self, M, N, K, weight) -> int:
+        """Over how many workgroups the block kernel splits K for a product of
+        M rows, or 0 when the product is not one of its own: bfloat16, a
+        row-major copy of the weight, K in chunks of 64, a matrix of few rows
+        (its tiles alone would leave most CUs idle, which is what the split
+        repairs) but of MID_MIN_ELEMENTS_MANY elements at least (smaller ones
+        stay with the kernels they were measured on), and BLOCK_MIN_M to
+        BLOCK_MAX_M rows of x.  As many shares as give every CU a workgroup,
+        16 at most, of at least 3 chunks each (7B shape, down projection at 256
+        rows: 70 / 44 / 41 us with 4 / 8 / 9 shares; q/k/v: 21 / 17 / 26 us
+        with 4 / 7 / 8, the last being more workgroups than CUs)."""
+        w = weight.w if isinstance(weight, LinearWeight) else weight
+        if (self.act_dtype != torch.bfloat16 or not self.use_block_products or w is None
+                or K % 64 or N % 4 or N > self.BLOCK_MAX_N or N * K < self.MID_MIN_ELEMENTS_MANY
+                or not self.BLOCK_MIN_M <= M <= self.BLOCK_MAX_M):
+            return 0
+        tiles = -(-N // 128) * -(-M // 256)
+        return max(1, min(16, K // 64 // 3, self._num_cus // tiles))
+
+    def linear_block(self, x, weight, bias, out_f32=False, ks=1, partial=False):
+        """A few hundred rows over the row-major copy of the weight: workgroups
+        own a tile of 256 rows of x by 128 rows of W over one of ``ks`` shares
+        of K.  ``partial``: the product comes back as ``PartialSums`` for its
+        reader to add up."""
+        M, K = x.shape
+        N = weight.shape[0]
+        w = weight.w if isinstance(weight, LinearWeight) else weight
+        if w is None:
+            raise KernelError("linear_block needs the row-major copy of the weight")
+        self._check(x, self.act_dtype, (M, K), "x")
+        self._check(w, self.act_dtype, (N, K), "weight")
+        part = self._new((ks, M, N), torch.float32) if ks > 1 or partial else None
+        if partial:
+            if ks > 1:
+                self._call("gemm", "sl_gemm_block", _p(x), _p(w), None, None, M, N, K, 0, int(ks), _p(part))
+            else:
+                self._call("gemm", "sl_gemm_block", _p(x), _p(w), None, _p(part), M, N, K, 1, 1, None)
+            return PartialSums(part, bias)
+        y = self._new((M, N), torch.float32 if out_f32 else None)
+        self._call("gemm", "sl_gemm_block", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32),
+                   int(ks), _p(part))
         return y
 
     def linear_skinny(self, x, weight, bias, out_f32=False):
@@ -792,6 +841,15 @@ class HipOps:
         fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
                  and weight.tiled is not None and weight.shape == (N, K))
         if not fused:
+            shares = 0 if isinstance(x, ScaledRows) else self._block_shares(M, N, K, weight)
+            if shares:
+                # K split over workgroups of the block kernel; the rotation kernel adds the partial sums up
+                self._check(x, self.act_dtype, (M, K), "x")
+                product = self.linear_block(x, weight, bias, ks=shares, partial=True)
+                qkv = self._new((M, N))
+                self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                                True, split=product, rot_dim=rot, q_scale=q_scale)
+                return qkv
             if (self.WIDE_MIN_M <= M <= self._few_rows_limit(weight) and K % 32 == 0
                     and not isinstance(x, ScaledRows)):
                 # K split over workgroups; the rotation kernel adds the partial sums up

@@ -45,6 +45,19 @@ class Tuning:
     # ... and of this many at 33..128 rows, where re-reading x costs more
     mid_min_elements_many: int = 8 << 20
 
+    # ---- products over the row-major copy in tiles of 256 rows of x by 128 rows of W (gemm_block)
+    # matrices of at most block_max_n rows (q/k/v, o, down: K is split over workgroups until every CU has
+    # one; gate/up and the head have tiles enough for the library) take it from block_min_m rows of x
+    # on, where the LDS-staged kernel ends, up to block_max_m (7B shape, against the library's tuned
+    # kernels at 160 / 256 / 512 rows: down 44 / 46 / 83 us against 62 / 65 / 109, o 15 / 17 / 23 against 34 /
+    # 32 / 31, q/k/v 20 / 22 / 35 against 31 / 38 / 37; a third tile of 256 rows makes it read W a third time
+    # and the library wins: 544 rows down 124 against 114 us).  Below block_min_m it was measured too:
+    # alone faster than the LDS-staged kernel (down at 64 / 128 rows 27 / 33 against 38 / 62 us), inside a
+    # decode step of 24 to 128 requests 2-5 % slower, so those rows stay where they were.
+    block_max_n: int = 8192
+    block_min_m: int = 129
+    block_max_m: int = 512
+
     # ---- few-rows consumer products on workgroups that stay
     # tiles per CU from which walking the tiles beats a workgroup per tile (gate/up: 9, head: 37;
     # q/k/v with one or two tiles a CU has nothing to walk)

@@ -204,7 +204,9 @@ def test_tiled_only_weight_layout_runs_the_whole_model(tmp_path, monkeypatch):
     one: prompts go through the row-major scratch, decode straight to the matrix
     cores; logits equal those with both copies.  (No further copies in lower
     tiles here, which only the model with two copies would make: they group
-    the sums of squares of the stream differently.)"""
+    the sums of squares of the stream differently; the products in tiles
+    over the row-major copy, which a model without that copy cannot take, are
+    for larger matrices than this model has.)"""
     from servelab_amd.kernels import HipOps, Tuning
     folder = make_folder(tmp_path, "B", seed=27)
     toks = list(range(100, 180))

@@ -203,9 +203,12 @@ def test_linear_mid(M, N, K):
 def test_tiled_only_weights(M, N, K):
     """Only the tiled copy kept: few rows go straight to the matrix cores, many
     rows through the row-major scratch and the library; same results as with
-    both copies."""
+    both copies (whose products in tiles over the row-major copy are switched
+    off here: without that copy they are not taken; with them the results agree
+    to rounding)."""
     from servelab_amd.kernels import HipOps
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    ops.use_block_products = False
     w = randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5)
     b = randn(N, seed=6)
     both_copies = ops.prepare_weight(w)
@@ -216,6 +219,9 @@ def test_tiled_only_weights(M, N, K):
     for rows in (M, 100):
         x = randn(rows, K, dtype=torch.bfloat16, seed=rows)
         assert torch.equal(ops.linear(x, tiled_only, b), ops.linear(x, both_copies, b))
+        ops.use_block_products = True
+        assert rel_err(ops.linear(x, both_copies, b), emu.linear(x, w, b)) < 2 ** -7
+        ops.use_block_products = False
     kept = ops.prepare_weight(w, keep_rows=True)
     assert kept.w is w and kept.tiled is not None
     ops.weight_layout = "rows"
@@ -341,9 +347,11 @@ def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs, th):
     picked = ops.rows_add_rmsnorm(resid, ops.linear(x, w1, None, defer=True), rows, gain, eps, fuse=True)
     assert isinstance(picked, ScaledRows) and picked.shape == (rows.shape[0], H)
     assert rel_err(ops.linear(picked, w2, None, out_f32=True), normed[rows.long()] @ w2.w.float().T) < 2 ** -7
-    # more rows than the fused kernels take: the product is simply done
+    # more rows than the fused kernels take: the product is done (whole, or as partial sums for the norm)
     big = randn(17, K1, dtype=torch.bfloat16, seed=7)
-    assert torch.is_tensor(ops.linear(big, w1, None, defer=True))
+    done = ops.linear(big, w1, None, defer=True)
+    assert not isinstance(done, Deferred)
+    assert rel_err(ops.materialize(done), big.float() @ w1.w.float().T) < 2 ** -7
 
 
 def test_lower_tiles_for_the_products_that_add_to_the_stream():
@@ -1175,6 +1183,56 @@ def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
     many = randn(300, K, dtype=torch.bfloat16, seed=4)
     got = ops.linear(many, weight, b, out_f32=True)
     assert got.shape == (300, N) and rel_err(got, emu.linear(many, w, b, True)) < 2e-5
+
+
+def test_products_of_129_to_512_rows_of_matrices_of_few_rows_run_in_tiles():
+    """Where the LDS-staged kernel ends, matrices of at most 8,192 rows take the kernel in tiles
+    over the row-major copy, K split until every CU has a workgroup (plain, deferred as partial
+    sums for the norm, q/k/v with the rotation kernel adding the sums); larger matrices, more rows,
+    a model without the row-major copy and small matrices go to the library as before."""
+    from servelab_amd.kernels import HipOps
+    from servelab_amd.kernels.ops import PartialSums
+    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    K, N = 1024, 8192
+    w = randn(N, K, dtype=torch.bfloat16, scale=0.05, seed=2)
+    weight, b = ops.prepare_weight(w), randn(N, seed=3)
+    for M in (129, 300, 512):
+        x = randn(M, K, dtype=torch.bfloat16, seed=M)
+        shares = ops._block_shares(M, N, K, weight)
+        assert shares == max(1, min(K // 64 // 3, ops._num_cus // (N // 128 * -(-M // 256))))
+        assert torch.equal(ops.linear(x, weight, b), ops.linear_block(x, weight, b, ks=shares))
+        assert rel_err(ops.linear(x, weight, b), emu.linear(x, w, b)) < 2 ** -7
+        delta = ops.linear(x, weight, b, defer=True)
+        assert isinstance(delta, PartialSums) and delta.parts.shape == (shares, M, N)
+        assert rel_err(ops.materialize(delta), emu.linear(x, w, b)) < 2 ** -7
+    assert not ops._block_shares(128, N, K, weight) and not ops._block_shares(513, N, K, weight)
+    assert not ops._block_shares(300, 8208, K, ops.prepare_weight(randn(8208, K, dtype=torch.bfloat16)))
+    assert not ops._block_shares(300, 256, K, ops.prepare_weight(w[:256].contiguous()))
+    ops.weight_layout = "tiled"
+    assert not ops._block_shares(300, N, K, ops.prepare_weight(w.clone()))
+    ops.use_block_products = False
+    assert not ops._block_shares(300, N, K, weight)
+
+
+@pytest.mark.parametrize("M,N,K,ks", [(17, 3584, 3584, 16), (64, 3584, 18944, 12), (65, 4608, 3584, 7), (128, 520, 640, 3),
+                                      (129, 136, 64, 1), (160, 4608, 3584, 1), (300, 3584, 3584, 4), (512, 1000, 640, 2),
+                                      (513, 1000, 640, 3), (700, 260, 128, 1)])
+def test_products_in_tiles_over_the_row_major_copy(M, N, K, ks):
+    """The kernel alone at each of its tile shapes (up to 64 rows of x, up to 128, more), ragged in
+    rows and columns, with and without a split of K, a bias, float32 output and partial sums."""
+    from servelab_amd.kernels import HipOps
+    ops = HipOps(torch.bfloat16, "cuda:0")
+    x = randn(M, K, dtype=torch.bfloat16, seed=1)
+    w = randn(N, K, dtype=torch.bfloat16, scale=0.05, seed=2)
+    b = randn(N, seed=3)
+    ref = x.float() @ w.float().T
+    assert rel_err(ops.linear_block(x, w, b, out_f32=True, ks=ks), ref + b) < 2e-5
+    assert rel_err(ops.linear_block(x, w, None, ks=ks), ref) < 2 ** -7
+    assert rel_err(ops.linear_block(x, w, b, ks=1), ref + b) < 2 ** -7
+    parts = ops.linear_block(x, w, b, ks=ks, partial=True)
+    assert parts.parts.shape == (ks, M, N) and parts.bias is b
+    assert rel_err(parts.parts.sum(0) + b, ref + b) < 2e-5
+    assert rel_err(ops.materialize(parts), ref + b) < 2 ** -7
 
 
 @pytest.mark.parametrize("M,N,K", [(2, 130, 48), (8, 3584, 3584), (33, 200, 64), (64, 100, 96), (65, 100, 96),
