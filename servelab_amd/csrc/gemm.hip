@@ -72,8 +72,71 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(
   }
 }
 
+// The same product with the rows of x staged through LDS: the eight wavefronts of a workgroup own
+// four columns each and share every chunk of x, so x leaves the cache hierarchy once per 32 columns
+// of W instead of once per 4 (with 8 rows of x that was twice the bytes of W itself, and what the
+// float32 decode step spent most of its time pulling).  A lane keeps its own running sums over its
+// share of K, as above.
+template <int MB>
+__global__ __launch_bounds__(512) void gemm_rows_shared_kernel(
+    const act_t* __restrict__ x, const act_t* __restrict__ w, const float* __restrict__ bias,
+    void* __restrict__ y, int M, int N, int K, int out_f32) {
+  constexpr int NC = 4, KC = 256 * SL_VEC;           // values of k in a chunk: four steps of a wavefront
+  __shared__ vec_t xs[MB][KC / SL_VEC];
+  const int lane = threadIdx.x % SL_WAVE, wave = threadIdx.x / SL_WAVE;
+  const int n0 = (blockIdx.x * (blockDim.x / SL_WAVE) + wave) * NC;
+  const act_t* wr[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) wr[c] = w + (size_t)(n0 + c < N ? n0 + c : N - 1) * K;
+  float acc[MB][NC];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc[i][c] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += KC) {
+    const int kv = (K - k0 < KC ? K - k0 : KC) / SL_VEC;       // vectors of this chunk in a row
+    __syncthreads();                                           // the last chunk has been read
+    for (int idx = threadIdx.x; idx < MB * kv; idx += blockDim.x) {
+      const int m = idx / kv, v = idx % kv;
+      xs[m][v] = *(const vec_t*)(x + (size_t)(m < M ? m : M - 1) * K + k0 + v * SL_VEC);
+    }
+    __syncthreads();
+    for (int v = lane; v < kv; v += SL_WAVE) {
+      float wf[NC][SL_VEC];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const vec_t wv = *(const vec_t*)(wr[c] + k0 + v * SL_VEC);
+#pragma unroll
+        for (int j = 0; j < SL_VEC; ++j) wf[c][j] = to_f(wv.v[j]);
+      }
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const vec_t xv = xs[i][v];
+#pragma unroll
+        for (int j = 0; j < SL_VEC; ++j) {
+          const float xf = to_f(xv.v[j]);
+#pragma unroll
+          for (int c = 0; c < NC; ++c) acc[i][c] += wf[c][j] * xf;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const float s = wave_sum(acc[i][c]);
+      if (lane == 0 && i < M && n0 + c < N) {
+        const float r = s + (bias != nullptr ? bias[n0 + c] : 0.f);
+        if (out_f32) ((float*)y)[(size_t)i * N + n0 + c] = r;
+        else ((act_t*)y)[(size_t)i * N + n0 + c] = from_f<act_t>(r);
+      }
+    }
+}
+
+// `shared`: 4 to 16 rows of x (to 8 of bfloat16) go through LDS once per 32 columns (gemm_rows_shared_kernel).
 extern "C" const char* sl_gemm_rows(const void* x, const void* w, const float* bias, void* y,
-                                    int M, int N, int K, int out_f32, hipStream_t stream) {
+                                    int M, int N, int K, int out_f32, int shared, hipStream_t stream) {
   SL_CHECK(M >= 0 && N > 0 && K > 0, "gemm_rows: sizes must be positive");
   SL_CHECK(K % SL_VEC == 0, "gemm_rows: K must be a multiple of the 16-byte vector");
   SL_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
@@ -82,6 +145,20 @@ extern "C" const char* sl_gemm_rows(const void* x, const void* w, const float* b
   const int waves = 4;
   const act_t* xx = (const act_t*)x;
   const act_t* ww = (const act_t*)w;
+  // (measured, float32, 7B shape: from 4 rows on the staged form wins, 8 rows 139 -> 113 us for gate/up and
+  // 176 -> 114 us for down, 16 rows 281 -> 172 and 494 -> 174 us; with 1 to 3 rows it loses up to 18 us of 44)
+  constexpr int SHARED_MAX_M = sizeof(act_t) == 4 ? 16 : 8;   // (16 rows of bfloat16 spill registers)
+  if (shared && M >= 4 && M <= SHARED_MAX_M) {
+    // (eight wavefronts a workgroup also for matrices of few rows: four, for twice the workgroups, measured
+    // slower: down of the 7B shape at 8 / 16 rows 125 / 214 us against 114 / 174)
+    const int threads = 512;
+    const int cols = 4 * threads / SL_WAVE;
+    const dim3 grid((N + cols - 1) / cols);
+    if (M <= 4) gemm_rows_shared_kernel<4><<<grid, threads, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+    else if (M <= 8) gemm_rows_shared_kernel<8><<<grid, threads, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+    else if constexpr (SHARED_MAX_M == 16) gemm_rows_shared_kernel<16><<<grid, threads, 0, stream>>>(xx, ww, bias, y, M, N, K, out_f32);
+    return sl_launch_status();
+  }
   // one row of x: a column per wavefront keeps the most wavefronts in flight;
   // more rows: 4 columns per wavefront share each load of x
   if (M == 1) {

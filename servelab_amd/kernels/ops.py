@@ -676,7 +676,8 @@ class HipOps:
         M, K = x.shape
         N = w.shape[0]
         y = self._new((M, N), torch.float32 if out_f32 else None)
-        self._call("gemm", "sl_gemm_rows", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32))
+        self._call("gemm", "sl_gemm_rows", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32),
+                   int(self.ROWS_THROUGH_LDS))
         return y
 
     def linear_tiled(self, x, w, bias, out_f32=False):

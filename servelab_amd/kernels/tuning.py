@@ -45,6 +45,10 @@ class Tuning:
     # ... and of this many at 33..128 rows, where re-reading x costs more
     mid_min_elements_many: int = 8 << 20
 
+    # ---- the wavefront-per-column products (float32 table, bfloat16 fallbacks)
+    # up to 16 rows of x go through LDS once per 32 columns of W instead of through L1 once per 4
+    rows_through_lds: bool = True
+
     # ---- products over the row-major copy in tiles of 256 rows of x by 128 rows of W (gemm_block)
     # matrices of at most block_max_n rows (q/k/v, o, down: K is split over workgroups until every CU has
     # one; gate/up and the head have tiles enough for the library) take it from block_min_m rows of x
