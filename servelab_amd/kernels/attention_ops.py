@@ -1,0 +1,369 @@
+"""Position encodings of a mixer (tables, rotation and cache write, the q/k/v product that carries
+them) and attention over the paged cache (matrix-core kernels per head size, the general kernel
+for everything they refuse)."""
+import ctypes
+
+import torch
+
+from . import build
+from .values import (KernelError, LinearWeight, PartialSums, RotationPlan, ScaledRows, TiledRows,
+                     _RopeStore, _c_float, _p, _ptr)
+
+
+class AttentionOps:
+    # ----------------------------------------------------------------- rope
+    def rope_tables(self, positions, inv_freq):
+        T, half = positions.shape[0], inv_freq.shape[0]
+        self._check(positions, torch.int32, (T,), "positions")
+        self._check(inv_freq, torch.float32, (half,), "inv_freq")
+        cos = self._new((T, half), torch.float32)
+        sin = self._new((T, half), torch.float32)
+        self._call("elementwise", "sl_rope_tables", _p(positions), _p(inv_freq), _p(cos), _p(sin),
+                   T, half)
+        return cos, sin
+
+    def _check_pages(self, k_cache, v_cache, nkv, D, page_size):
+        pages = k_cache.shape[0]
+        self._check(k_cache, self.act_dtype, (pages, nkv, page_size, D), "K pages")
+        self._check(v_cache, self.act_dtype, (pages, nkv, D, page_size), "V pages")
+        return pages
+
+    def rope_store(self, qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                   pairs8=False, split=None, rot_dim=None, q_scale=1.0):
+        """Rotate q and k of ``qkv`` in place (``cos`` None: no rotation) and write
+        k and v to their cache rows (``k_cache`` None: no write).  The first
+        ``rot_dim`` channels of a head are rotated (default: all), pair j being
+        (j, j + rot_dim / 2); ``pairs8``: they come in blocks of 8 channels and
+        their 8 partners (the order ``qkv_rope_store`` uses) instead.
+        ``split``: the product arrives as ``PartialSums``; ``qkv`` is then only
+        written (its q columns).  ``q_scale`` multiplies the q heads after the
+        rotation, before their rounding."""
+        T = qkv.shape[0]
+        rot = D if rot_dim is None else int(rot_dim)
+        if rot % 2 or not 0 <= rot <= D or (pairs8 and rot % 16) or (cos is not None and rot == 0):
+            raise KernelError(f"rope_store: cannot rotate {rot} of {D} channels"
+                              + (" in blocks of 8 pairs" if pairs8 else ""))
+        self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
+        parts = bias = None
+        if split is not None:
+            parts, bias = split.parts, split.bias
+            self._check(parts, torch.float32, (parts.shape[0], T, (nh + 2 * nkv) * D), "partial sums")
+            if bias is not None:
+                self._check(bias, torch.float32, ((nh + 2 * nkv) * D,), "bias")
+        if cos is not None:
+            self._check(cos, torch.float32, (T, rot // 2), "cos")
+            self._check(sin, torch.float32, (T, rot // 2), "sin")
+        if k_cache is not None:
+            self._check_pages(k_cache, v_cache, nkv, D, page_size)
+            self._check(slots, torch.int32, (T,), "slots")
+        self._call("elementwise", "sl_rope_store", _p(qkv), _p(cos), _p(sin), _p(slots),
+                   _p(k_cache), _p(v_cache), T, nh, nkv, D, rot, page_size, int(pairs8),
+                   _p(parts), parts.shape[0] if parts is not None else 0, _p(bias), _c_float(q_scale))
+
+    def qkv_rope_store(self, x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
+                       page_size, rot_dim=None, q_scale=1.0):
+        """q/k/v product, rotation and cache write.  The rows of ``weight`` (and
+        ``bias``) hold every q and k head in the blocked pair order (``pairs8``
+        above).  Returns the [T, (nh + 2 nkv) D] buffer whose q columns the
+        attention reads.  For at most 16 rows and a tiled weight all of it is
+        one kernel; k and v columns of the buffer are then not written."""
+        if not isinstance(weight, LinearWeight):
+            weight = LinearWeight(weight)
+        M, K = x.shape
+        N = weight.shape[0]
+        rot = D if rot_dim is None else int(rot_dim)
+        if N != (nh + 2 * nkv) * D or D % 16 or rot % 16 or not 0 <= rot <= D:
+            raise KernelError("qkv_rope_store: weight rows must be (nh + 2 nkv) * D with D % 16 == 0, "
+                              "the rotated width a multiple of 16")
+        fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
+                 and weight.tiled is not None and weight.shape == (N, K))
+        if not fused:
+            shares = 0 if isinstance(x, ScaledRows) else self._block_shares(M, N, K, weight)
+            if shares:
+                # K split over workgroups of the block kernel; the rotation kernel adds the partial sums up
+                self._check(x, self.act_dtype, (M, K), "x")
+                product = self.linear_block(x, weight, bias, ks=shares, partial=True)
+                qkv = self._new((M, N))
+                self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                                True, split=product, rot_dim=rot, q_scale=q_scale)
+                return qkv
+            if (self.WIDE_MIN_M <= M <= self._few_rows_limit(weight) and K % 32 == 0
+                    and not isinstance(x, ScaledRows)):
+                # K split over workgroups; the rotation kernel adds the partial sums up
+                product = self.linear_mid(x, weight, bias, partial=True)
+                if isinstance(product, PartialSums):
+                    qkv = self._new((M, N))
+                    self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                                    True, split=product, rot_dim=rot, q_scale=q_scale)
+                    return qkv
+                qkv = product
+            elif (self.act_dtype == torch.bfloat16 and not isinstance(x, ScaledRows)
+                    and M > self._few_rows_limit(weight)):
+                # many rows: the library keeps the float32 sums, and the rotation kernel adds the
+                # float32 bias, rotates and rounds once, exactly as the fused few-rows kernel does
+                self._check(x, self.act_dtype, (M, K), "x")
+                sums = self.library_sums(x, self.rows_of(weight), torch.float32)
+                qkv = self._new((M, N))
+                self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                                True, split=PartialSums(sums.unsqueeze(0), bias), rot_dim=rot,
+                                q_scale=q_scale)
+                return qkv
+            else:
+                qkv = self.linear(x, weight, bias)
+            self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size, True,
+                            rot_dim=rot, q_scale=q_scale)
+            return qkv
+        scaled = x if isinstance(x, ScaledRows) else None
+        if scaled is None:
+            self._check(x, self.act_dtype, None, "x")
+        if bias is not None:
+            self._check(bias, torch.float32, (N,), "bias")
+        if cos is not None:
+            self._check(cos, torch.float32, (M, rot // 2), "cos")
+            self._check(sin, torch.float32, (M, rot // 2), "sin")
+        if k_cache is not None:
+            self._check_pages(k_cache, v_cache, nkv, D, page_size)
+            self._check(slots, torch.int32, (M,), "slots")
+        rope = _RopeStore(_ptr(cos), _ptr(sin), _ptr(slots if k_cache is not None else None),
+                          _ptr(k_cache), _ptr(v_cache), nh, nkv, D, page_size, rot, q_scale)
+        qkv = self._new((M, N))
+        self._skinny(scaled.x if scaled is not None else x, weight, bias, qkv, M, N, K,
+                     scaled=scaled, rope=rope)
+        return qkv
+
+    # --------------------------------------------- position encodings of a mixer
+    def plan_rotation(self, head_dim, layout) -> RotationPlan:
+        """The channel order of q and k heads for a position encoding whose
+        ``layout`` is None (nothing is rotated) or says ``rot_dim`` (the leading
+        channels that are rotated) and ``pairing``: "half" pairs channel j with
+        j + rot_dim / 2, "interleaved" 2j with 2j + 1.  Scores do not depend on
+        the order of the channels as long as q and the cached k agree, so an
+        interleaved pairing is turned into halves by the order alone, and the
+        rotated channels are laid out in blocks of 8 and their 8 partners where
+        the fused q/k/v kernel can take them (head size and rotated width
+        multiples of 16)."""
+        D = int(head_dim)
+        rot = 0 if layout is None else int(layout.rot_dim)
+        pairing = "half" if layout is None else layout.pairing
+        if rot % 2 or not 0 <= rot <= D:
+            raise KernelError(f"a rotation of {rot} of {D} channels has no kernel: the width must be even")
+        if pairing not in ("half", "interleaved"):
+            raise KernelError(f"pairing '{pairing}' has no kernel (half or interleaved)")
+        order = list(range(D))
+        if pairing == "interleaved":
+            order[:rot] = list(range(0, rot, 2)) + list(range(1, rot, 2))
+        blocked = D % 16 == 0 and rot % 16 == 0
+        if blocked and rot:
+            halves = order[:rot]
+            order[:rot] = [halves[(i % 16 >= 8) * (rot // 2) + 8 * (i // 16) + i % 8] for i in range(rot)]
+        plain = order == list(range(D))
+        return RotationPlan(None if plain else torch.tensor(order, dtype=torch.long), rot, blocked)
+
+    LOG2E = 1.4426950408889634
+
+    def split_attention_scale(self, scale: float):
+        """(factor for q at its producer, scale left for ``paged_attention``).
+        The matrix-core attention kernels want their scores in units of log 2:
+        q then leaves ``project_qkv`` multiplied by scale * log2(e) (before its
+        one rounding) and the attention call gets ln 2, whose product with
+        log2(e) is 1, so no multiply-add per score is left.  The float32 table
+        keeps the scale where the reference has it."""
+        if self.act_dtype != torch.bfloat16 or not self.use_mfma_attention:
+            return 1.0, float(scale)
+        return float(scale) * self.LOG2E, 1.0 / self.LOG2E
+
+    def project_qkv(self, x, weight, bias, nh, nkv, D, plan, tables, slots, k_cache, v_cache,
+                    page_size, q_scale=1.0):
+        """What a mixer calls: the q/k/v product of ``x`` (rows of ``weight`` in
+        the order of ``plan``), the position encoding's work on q and k for this
+        step's ``tables`` (whatever the encoding's ``tables()`` returned: None,
+        or an object with ``cos`` and ``sin`` [T, rot_dim / 2]) and the write of
+        k and v into the cache.  Returns [T, (nh + 2 nkv) D] whose q columns the
+        attention reads, multiplied by ``q_scale`` (see ``split_attention_scale``)."""
+        cos = sin = None
+        if tables is not None:
+            cos, sin = getattr(tables, "cos", None), getattr(tables, "sin", None)
+            if cos is None or sin is None:
+                raise KernelError(f"position tables of type {type(tables).__name__} have no kernel: "
+                                  "this table rotates channel pairs by cos and sin and nothing else")
+            if plan.rot_dim == 0:
+                raise KernelError("the position encoding gives tables but its layout rotates nothing")
+        if plan.blocked:
+            return self.qkv_rope_store(x, weight, bias, nh, nkv, D, cos, sin, slots, k_cache, v_cache,
+                                       page_size, rot_dim=plan.rot_dim, q_scale=q_scale)
+        qkv = self.linear(x, weight, bias)
+        self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
+                        rot_dim=plan.rot_dim, q_scale=q_scale)
+        return qkv
+
+    # ------------------------------------------------------------ attention
+    def attend_and_project(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                           batch, scale, window, w_out, bias=None, defer=False):
+        """``paged_attention`` followed by ``linear`` with the output projection.  For a step of a few
+        single tokens the kernel table keeps what lies between them laid out by k-step, as
+        ``gated_mlp`` does (at 16 rows the projection reads as many bytes of x as of W)."""
+        if not isinstance(w_out, LinearWeight):
+            w_out = LinearWeight(w_out)
+        T = qkv.shape[0]
+        tiled = (self.tile_few_rows and 1 < T <= self.FUSED_NORM_MAX_M and batch.max_q_len == 1
+                 and batch.num_prefill_seqs == 0 and batch.num_seqs == T and w_out.tiled is not None
+                 and w_out.shape[1] == nh * D
+                 and self._mfma_attention_fits(D, nh // nkv, block_tables.shape[1], page_size, batch))
+        attn = self.paged_attention(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                                    batch, scale, window, _tiled_out=tiled)
+        return self.linear(attn, w_out, bias, defer=defer)
+
+    def paged_attention(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                        batch, scale, window, _tiled_out=False):
+        T = qkv.shape[0]
+        S, max_pages = block_tables.shape
+        self._check(qkv, self.act_dtype, (T, (nh + 2 * nkv) * D), "qkv")
+        self._check_pages(k_cache, v_cache, nkv, D, page_size)
+        self._check(block_tables, torch.int32, None, "block tables")
+        self._check(batch.tok_seq, torch.int32, (T,), "tok_seq")
+        self._check(batch.positions, torch.int32, (T,), "positions")
+        if S != batch.num_seqs:
+            raise KernelError(f"block tables hold {S} sequences, the batch {batch.num_seqs}")
+        if batch.max_ctx_len > max_pages * page_size:
+            raise KernelError("block table is shorter than the context")
+        out = self._new((T, nh * D))
+        if self._mfma_attention_fits(D, nh // nkv, max_pages, page_size, batch):
+            self._attention_mfma(qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables,
+                                 batch, scale, window, out, out_rows=T if _tiled_out else 0)
+            return TiledRows(out, (T, nh * D)) if _tiled_out else out
+        stride = (nh + 2 * nkv) * D
+        first = 0                         # tokens before this one are done
+        n_pre, n_pre_tok = batch.num_prefill_seqs, batch.num_prefill_tokens
+        if n_pre and D % 16 == 0 and batch.max_q_len > 1:
+            # prompt portions (they come first in the batch): workgroups that stage each block of keys
+            # once for 16 columns, instead of a wavefront per (token, head) that reads its own
+            self._check(batch.cu_q, torch.int32, (batch.num_seqs + 1,), "cu_q")
+            self._call("attention", "sl_attention_general_tiles", _p(qkv), stride, _p(k_cache),
+                       _p(v_cache), _p(block_tables), max_pages, _p(batch.cu_q), _p(batch.positions),
+                       n_pre, batch.max_q_len, nh, nkv, D, page_size, _c_float(scale),
+                       int(window or 0), _p(out))
+            first = n_pre_tok
+        rest = T - first
+        if rest == 0:
+            return out
+        # few tokens (a decode step): the keys of every (token, head) are shared out over several
+        # wavefronts; the count depends on the number of tokens only, so that a captured step and an
+        # eager one add up in the same order
+        single = first > 0 or batch.max_q_len == 1
+        group = nh // nkv                 # a wavefront takes up to 8 heads of a group together
+        per_token = nkv * -(-group // 8) if group > 1 else nh
+        nsplit = max(1, min(64, self.GENERAL_ATTENTION_WAVES // (rest * per_token))) if single else 1
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = self._new((rest, nh, nsplit, D), torch.float32)
+            part_ml = self._new((rest, nh, nsplit, 2), torch.float32)
+        self._call("attention", "sl_attention_general", _p(qkv[first:]), stride, _p(k_cache),
+                   _p(v_cache), _p(block_tables), max_pages, _p(batch.tok_seq[first:]),
+                   _p(batch.positions[first:]), rest, nh, nkv, D, page_size, _c_float(scale),
+                   int(window or 0), _p(out[first:]), nsplit, _p(part_o), _p(part_ml))
+        return out
+
+    def _mfma_attention_fits(self, D, group, max_pages, page_size, batch):
+        """The matrix-core kernels take bfloat16, head sizes that are multiples
+        of 32, and block tables that cover the context rounded up to a whole
+        32-key block; everything else goes to the general kernel."""
+        if self.act_dtype != torch.bfloat16 or not self.use_mfma_attention:
+            return False
+        if D % 32 or D > 256 or group > 64:
+            return False
+        return max_pages * page_size >= -(-batch.max_ctx_len // 32) * 32
+
+    def _attention_lib(self, D):
+        key = ("attention_mfma", D)
+        lib = self._lib.get(key)
+        if lib is None:
+            lib = build.load(build.unit("attention_mfma", "bfloat16", SL_HEAD_DIM=D))
+            self._lib[key] = lib
+        return key
+
+    def _decode_shares(self, units, most) -> int:
+        """Into how many shares the keys of each of ``units`` (request, kv head) pairs are cut, ``most`` at
+        most.  A share is a wavefront, and a wavefront streams its keys at the pace of its round trips to
+        memory, so the launch takes what its busiest CU holds: TARGET_WAVES wavefronts (two a CU) are best,
+        and a launch slightly above a whole number of wavefronts per CU is the worst (7B shape, contexts of
+        4,096: 14 requests in 10 shares, 560 wavefronts: 30.6 us a layer; in 9, 504 wavefronts: about 22 us;
+        24 requests 576 against 480 wavefronts: 4.73 against 4.40 ms a step; 48 requests 384 / 576 / 768
+        wavefronts: 5.62 / 5.77 / 5.49 ms).  Taken: the count whose wavefronts fill their rounds over the CUs
+        best, less a fifth of its relative distance from the target; no more than half again the target."""
+        cus, target = self._num_cus, self.TARGET_WAVES
+        best, best_score = 1, None
+        for shares in range(1, max(1, min(most, (3 * target // 2) // units)) + 1):
+            waves = units * shares
+            score = waves / (-(-waves // cus) * cus) - 0.2 * abs(waves - target) / target
+            if best_score is None or score > best_score + 1e-9:
+                best, best_score = shares, score
+        return best
+
+    def _pair_prompt_tiles(self, tiles, prompts_and_heads) -> bool:
+        """Whether the workgroups of a whole prompt's attention take a late tile of the causal triangle and
+        its early mirror (equal work for all, half as many workgroups) or a tile each, long ones first.
+        Equal workgroups fill the chip in rounds of two per CU, and the last round may be nearly empty;
+        tiles of their own leave the balance to the order in which workgroups start, at the price of
+        twice the prologues.  7B shape, one prompt, pairs against a tile each: 4,096 tokens (448 pairs, one
+        round) 175 against 223 us, 5,120 (560) 335 against 270, 7,168 (784) 546 against 461, 8,192 (896) 615
+        against 572, 10,240 (1,120) 972 against 880, 14,336 (1,568) 1,842 against 1,618, 16,384 (1,792: three
+        and a half rounds) 2,040 either way."""
+        if not self.PAIR_PROMPT_TILES:
+            return False
+        pairs = -(-tiles // 2) * prompts_and_heads
+        slots = 2 * self._num_cus
+        rounds = -(-pairs // slots)
+        return rounds == 1 or pairs >= self.UNPAIRED_BELOW_FILL * rounds * slots
+
+    def _attention_mfma(self, qkv, nh, nkv, D, k_cache, v_cache, page_size, block_tables, batch,
+                        scale, window, out, out_rows=0):
+        lib = self._attention_lib(D)
+        self._check(batch.cu_q, torch.int32, (batch.num_seqs + 1,), "cu_q")
+        max_pages = block_tables.shape[1]
+        n_pre, n_pre_tok = batch.num_prefill_seqs, batch.num_prefill_tokens
+        n_dec = batch.num_seqs - n_pre
+        if n_dec and n_pre_tok + n_dec != batch.num_tokens:
+            raise KernelError("single-token sequences must come last in the batch")
+        common = (_p(qkv), (nh + 2 * nkv) * D, _p(k_cache), _p(v_cache), _p(block_tables),
+                  max_pages, _p(batch.cu_q), _p(batch.positions))
+        tail = (nh, nkv, D, page_size, _c_float(scale), int(window or 0))
+        name = f"sl_attention_mfma@{D}"
+        if name not in self._fn:
+            fn = self._lib[lib].sl_attention_mfma
+            fn.restype = ctypes.c_char_p
+            self._fn[name] = fn
+        if n_pre:
+            waves = -(-batch.max_q_len * (nh // nkv) // 32) * nkv * n_pre
+            shared = (waves >= self.SHARED_ATTENTION_MIN_WAVES and
+                      batch.max_ctx_len >= self.SHARED_ATTENTION_MIN_CONTEXT and
+                      bool(self._lib[lib].sl_attention_mfma_shares_keys()))
+            # tiles of a causal triangle differ in length and are paired; those of a portion
+            # that starts deeper in its context than it is long do not
+            triangle = batch.max_ctx_len < 2 * batch.max_q_len
+            pair = triangle and self._pair_prompt_tiles(-(-batch.max_q_len * (nh // nkv) // 128), nkv * n_pre)
+            # few unpaired tiles over a long context: each is cut into shares of its keys
+            nsplit, part_o, part_ml = 1, None, None
+            if shared and not triangle:
+                nsplit = max(1, min(self.PROMPT_SPLIT_MAX, batch.max_ctx_len // 32 // self.PROMPT_SPLIT_MIN_BLOCKS,
+                                    -(-self.PROMPT_SPLIT_WORKGROUPS // -(-waves // 4)),
+                                    self.PROMPT_SPLIT_BYTES // (n_pre_tok * nh * D * 4)))
+            if nsplit > 1:
+                part_o = self._new((n_pre_tok, nh, nsplit, D), torch.float32)
+                part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
+            self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
+                       0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
+                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS, 0)
+        if n_dec:
+            blocks = -(-batch.max_ctx_len // 32)
+            if window:
+                blocks = min(blocks, -(-int(window) // 32) + 1)
+            # (a few requests with long contexts: up to 256 shares, so that the launch still has TARGET_WAVES
+            # wavefronts; 7B shape, one request at 32,000 tokens: 64 shares leave one wavefront per CU)
+            most = int(self._lib[lib].sl_attention_mfma_max_splits())
+            nsplit = self._decode_shares(n_dec * nkv, min(most, blocks // 2))
+            part_o = part_ml = None
+            if nsplit > 1:
+                part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
+                part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
+            self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, 0, _p(out),
+                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0, 0, int(out_rows))

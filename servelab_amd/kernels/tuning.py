@@ -1,7 +1,7 @@
 """The numbers that choose between kernels, in one place.
 
 Kernel *limits* (how many rows a kernel can take, which head sizes) stay with
-the kernels' wrappers in ``ops.py``: they are facts of the code.  What is here
+the kernels' wrappers in the kernel table (``*_ops.py``): they are facts of the code.  What is here
 are *choices* that were measured on one MI355X with the projection sizes of the
 Qwen2.5 7B, 32B and 72B shapes; another GPU or another architecture's sizes may
 want others.  ``HipOps(dtype, device, tuning=Tuning(target_waves=...))`` takes a
