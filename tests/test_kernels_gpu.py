@@ -1216,7 +1216,7 @@ def test_products_of_129_to_512_rows_of_matrices_of_few_rows_run_in_tiles():
 
 @pytest.mark.parametrize("M,N,K,ks", [(17, 3584, 3584, 16), (64, 3584, 18944, 12), (65, 4608, 3584, 7), (128, 520, 640, 3),
                                       (129, 136, 64, 1), (160, 4608, 3584, 1), (300, 3584, 3584, 4), (512, 1000, 640, 2),
-                                      (513, 1000, 640, 3), (700, 260, 128, 1)])
+                                      (513, 1000, 640, 3), (700, 260, 128, 1), (200, 1001, 192, 2), (256, 130, 64, 1)])
 def test_products_in_tiles_over_the_row_major_copy(M, N, K, ks):
     """The kernel alone at each of its tile shapes (up to 64 rows of x, up to 128, more), ragged in
     rows and columns, with and without a split of K, a bias, float32 output and partial sums."""

@@ -136,6 +136,22 @@ def test_float32_error_at_depth():
         got = torch.cat(rows).double()
         report[layers] = ((got - exact).abs().max().item(), (plain32 - exact).abs().max().item(),
                           exact.abs().max().item())
+        if layers == 28:
+            # at the full depth also in portions and mixed: a second request whose portions (down to two
+            # tokens) run beside the first one's, which is cut at other places than above
+            other = [rng.randrange(4099) for _ in range(41)]
+            exact_other = plain.forward(raw, weights, other, dtype=torch.float64)
+            runner.close("a")
+            cuts_a, cuts_b = [0, 30, 31, 33, 50, 64], [0, 5, 25, 27, 28, 41]
+            mixed = 0.0
+            for i in range(5):
+                ta, tb = toks[cuts_a[i]:cuts_a[i + 1]], other[cuts_b[i]:cuts_b[i + 1]]
+                out = runner.step([StepEntry("a", ta, list(range(len(ta)))),
+                                   StepEntry("b", tb, list(range(len(tb))))]).double()
+                mixed = max(mixed, (out[:len(ta)] - exact[cuts_a[i]:cuts_a[i + 1]]).abs().max().item(),
+                            (out[len(ta):] - exact_other[cuts_b[i]:cuts_b[i + 1]]).abs().max().item())
+            print(f"float32 at 28 layers, two requests in portions side by side: {mixed:.2e}")
+            assert mixed <= 1e-4, mixed
         del model, runner, weights
         torch.cuda.empty_cache()
     for layers, (engine, arithmetic, top) in report.items():
