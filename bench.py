@@ -224,7 +224,7 @@ def main():
             "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "page_size": page, "prefill_tokens": args.prefill_tokens,
             "decode_mean_context": round(mean_ctx, 1), "sampling": "greedy",
-            "weight_layout": model.rt.ops.weight_layout,
+            "weight_layout": model.rt.ops.layout_summary(),
             "library_tuning": "off" if args.no_tune or args.no_prefill else "tunableop",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,

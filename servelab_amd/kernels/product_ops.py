@@ -56,9 +56,21 @@ class ProductOps:
         if self.act_dtype == torch.bfloat16:
             total = torch.cuda.get_device_properties(self.device).total_memory
             self.weight_layout = "dual" if 2 * total_bytes <= self.DUAL_MEMORY_SHARE * total else "tiled"
+            # "tiled": as many matrices as fit below ROWS_COPIES_MEMORY_SHARE keep their row-major copy as
+            # well, in the order in which they are loaded; the products of many rows of the others go
+            # through the scratch buffer
+            self._rows_budget = 0 if self.weight_layout == "dual" else \
+                max(0, int(self.ROWS_COPIES_MEMORY_SHARE * total) - total_bytes)
             # a third copy of the matrices that add to the stream (about a third of all), in lower tiles
             self.lower_tiles = self.weight_layout == "dual" and 2.35 * total_bytes <= self.LOWER_TILES_MEMORY_SHARE * total
         return self.weight_layout
+
+    def layout_summary(self) -> str:
+        """The layout in words, for records: "dual", "rows", or "tiled" with how many of the
+        matrices kept a row-major copy as well."""
+        if self.weight_layout != "tiled" or not self._matrices_with_rows:
+            return self.weight_layout
+        return f"tiled, {self._matrices_with_rows} of {self._matrices} matrices also row-major"
 
     def producer_tile_height(self, N, rows=8):
         """(rows per tile, rows of x from which it pays) for the few-rows product of a matrix of N rows that
@@ -106,9 +118,13 @@ class ProductOps:
             return LinearWeight(w)
         tiled = torch.empty(-(-N // 16) * 16 * K, dtype=torch.bfloat16, device=self.device)
         self._call("gemm", "sl_tile_weight", _p(w), _p(tiled), N, K, 16)
-        if self.weight_layout == "tiled" and not keep_rows:
+        self._matrices += 1
+        if self.weight_layout == "tiled" and not keep_rows and 2 * N * K > self._rows_budget:
             weight = LinearWeight(None, tiled, (N, K))
         else:
+            if self.weight_layout == "tiled" and not keep_rows:
+                self._rows_budget -= 2 * N * K
+            self._matrices_with_rows += 1
             weight = LinearWeight(w, tiled)
         if residual_delta and self.fuse_norms and self.lower_tiles:
             th, lower_from = (_th, 1) if _th is not None else self.producer_tile_height(N)

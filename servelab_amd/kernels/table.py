@@ -58,6 +58,8 @@ class KernelTable:
         self.weight_layout = "dual" if act_dtype == torch.bfloat16 else "rows"
         self.lower_tiles = act_dtype == torch.bfloat16        # see plan_weights
         self._untiled = None          # scratch for "tiled": the row-major form of one matrix
+        self._rows_budget = 0         # bytes of row-major copies a "tiled" model may still keep (plan_weights)
+        self._matrices = self._matrices_with_rows = 0
         # Up to this many rows no product of a prepared weight goes to the library
         # (whose kernels may record memsets, which HIP graphs replay wrongly here):
         # decode steps of at most this many requests can be captured.

@@ -17,6 +17,12 @@ class Tuning:
     # both copies of a matrix (row-major for the library, tiled for the few-rows kernels) are kept
     # while they stay below this share of the device's memory; beyond it only the tiled copy
     dual_memory_share: float = 0.45
+    # a model beyond that keeps the tiled copy of every matrix and, while all copies stay below this
+    # share of the device's memory, the row-major copy of as many matrices as fit as well, in the order
+    # they are loaded: their products of many rows go straight to the library (72B shape, 145 GB of
+    # weights: 77 GB of row-major copies, 44 of 80 layers; writing a matrix row-major into the scratch
+    # buffer before each of its products was a fifth of a 2,048-token prefill)
+    rows_copies_memory_share: float = 0.72
     # the matrices whose few-rows products add to the residual stream get a further copy in tiles of fewer
     # than 16 rows where those go round the CUs more evenly (HipOps.producer_tile_height), while all copies
     # stay below this share of the device's memory and the busiest CU pulls at least min_gain less (32B shape,

@@ -212,14 +212,30 @@ def test_tiled_only_weight_layout_runs_the_whole_model(tmp_path, monkeypatch):
     toks = list(range(100, 180))
     rows = {}
     for share in (0.45, 0.0):
-        ops = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(dual_memory_share=share, lower_tiles_min_gain=1.0))
+        ops = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(dual_memory_share=share, lower_tiles_min_gain=1.0,
+                                                             rows_copies_memory_share=0.0))
         _, model = load_model_on_device(folder, "bfloat16", ops=ops)
-        assert model.rt.ops.weight_layout == ("dual" if share else "tiled")
+        assert model.rt.ops.layout_summary() == ("dual" if share else "tiled")
         runner = ModelRunner(model, 16, 16)
         out = [runner.step([StepEntry("a", toks[:70], [0, 69])])]
         out += [runner.step([StepEntry("a", [t], [0])]).clone() for t in toks[70:]]
         rows[share] = torch.cat(out)
     assert torch.equal(rows[0.45], rows[0.0])
+    # with room for some row-major copies beside the tiled ones, the first matrices loaded keep theirs
+    # (here: room for four of the model's matrices) and their many-row products skip the scratch buffer
+    total = torch.cuda.get_device_properties(0).total_memory
+    cfg = load_config(folder)
+    sizes = [s.shape[0] * s.shape[1] * 2 for s in model.spec.param_specs().values() if len(s.shape) == 2]
+    room = (sum(sizes) + 2.5 * max(sizes)) / total
+    ops = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(dual_memory_share=0.0, lower_tiles_min_gain=1.0,
+                                                         rows_copies_memory_share=room))
+    _, some = load_model_on_device(folder, "bfloat16", ops=ops, config=cfg)
+    assert ops.weight_layout == "tiled" and 0 < ops._matrices_with_rows < ops._matrices
+    assert "also row-major" in ops.layout_summary()
+    runner = ModelRunner(some, 16, 16)
+    out = [runner.step([StepEntry("a", toks[:70], [0, 69])])]
+    out += [runner.step([StepEntry("a", [t], [0])]).clone() for t in toks[70:]]
+    assert torch.equal(torch.cat(out), rows[0.0])
 
 
 def test_tuned_library_products_keep_the_logits(tmp_path):
