@@ -99,12 +99,47 @@ struct AttnParams {
   int pair;                      // prompt workgroups take a late tile and its early mirror
   int out_rows;                  // 0: out is [T, nh * D]; else its rows are laid out by k-step for the few-rows
                                  // product that reads them: element (t, c) at (c / 32) * (out_rows * 32) + t * 32 + c % 32
+  int by_chiplet;                // a one-dimensional grid laid out by Place below (else x: workgroup of a pair, y: kv head, z: sequence)
+  int grid_x, num_seqs;          // ... its extent per (sequence, kv head) pair, and the sequences
 };
 
 // where element (row, col) of the result goes (col = head * D + channel; runs of four channels stay together)
 __device__ __forceinline__ size_t out_index(int out_rows, int nh, size_t row, int col) {
   return out_rows ? (size_t)(col / 32) * (out_rows * 32) + row * 32 + col % 32 : row * (size_t)(nh * D) + col;
 }
+
+// Workgroups go to the eight chiplets in turn (workgroup i to chiplet i % 8), and each chiplet has an L2 of
+// its own.  The workgroups of one kv head read the same keys and values, so a launch laid out head by head
+// spreads every head's keys over all eight L2s: eight times the footprint, and beyond a few thousand tokens
+// the keys come from memory again and again (7B shape, 8,192 tokens: 644 us; laid out as below: 533 us).
+// Laid out by chiplet, a kv head's workgroups all run on the 8 / nkv chiplets it has to itself (or, with
+// 8, 16, .. kv heads, on the one chiplet it shares with nkv / 8 - 1 others); the workgroups of a head are
+// dealt to its chiplets in turn, first workgroup of every sequence first, so each chiplet gets the same mix
+// of long and short tiles.
+struct Place {
+  int x, kvh, seq;
+  bool valid;
+  __device__ __forceinline__ Place(const AttnParams& P) {
+    if (!P.by_chiplet) {
+      x = blockIdx.x, kvh = blockIdx.y, seq = P.seq_begin + blockIdx.z, valid = true;
+      return;
+    }
+    const int chiplet = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    if (P.nkv < 8) {
+      const int each = 8 / P.nkv;                  // chiplets a head: each takes every each-th workgroup of every sequence
+      const int per_seq = (P.grid_x + each - 1) / each;
+      kvh = chiplet % P.nkv;
+      x = idx % per_seq * each + chiplet / P.nkv;
+      seq = P.seq_begin + idx / per_seq;
+    } else {
+      const int share = P.nkv / 8;                 // heads a chiplet
+      kvh = chiplet + 8 * (idx % share);
+      x = idx / share % P.grid_x;
+      seq = P.seq_begin + idx / share / P.grid_x;
+    }
+    valid = x < P.grid_x;
+  }
+};
 
 // The columns of one wavefront: queries, reference points and sums, outputs.
 //
@@ -510,7 +545,9 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   // (wave as a scalar: the products below sit under conditions that depend on it, and matrix
   // instructions ignore the execution mask)
   const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63, n = lane & 15, gq = lane >> 4;
-  const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
+  const Place at(P);
+  if (!at.valid) return;                             // (the whole workgroup)
+  const int seq = at.seq, kvh = at.kvh;
   const int g = P.nh / P.nkv;
   const int q0 = P.cu_q[seq];
   const int qlen = P.cu_q[seq + 1] - q0;
@@ -595,8 +632,8 @@ void attention_mfma_shared_kernel(const AttnParams P) {
   // Unpaired tiles of a long context may also be cut into P.nsplit shares of
   // their key blocks, a workgroup each, whose partial results the combine
   // kernel merges: more and shorter workgroups for a launch of few tiles.
-  const int tile_rev = P.pair ? (int)blockIdx.x : (int)blockIdx.x / P.nsplit;
-  const int split = P.pair ? 0 : (int)blockIdx.x % P.nsplit;
+  const int tile_rev = P.pair ? at.x : at.x / P.nsplit;
+  const int split = P.pair ? 0 : at.x % P.nsplit;
   for (int half = 0; half < 2; ++half) {
   if (P.pair ? 2 * tile_rev + half > ntiles - 1 : half > 0 || tile_rev >= ntiles)
     break;                                                  // no such tile; the whole workgroup leaves together
@@ -745,6 +782,8 @@ extern "C" int sl_attention_mfma_max_splits() { return 64 * COMBINE_PER_LANE; }
 extern "C" int sl_attention_mfma_head_dim() { return D; }
 // whether this head size has the prompt kernel that shares keys through LDS (its buffers fit)
 extern "C" int sl_attention_mfma_shares_keys() { return SHARED_FITS ? 1 : 0; }
+// whether the workgroups that share keys through LDS are laid out by chiplet for this many kv heads (see Place)
+extern "C" int sl_attention_mfma_by_chiplet(int nkv) { return nkv > 0 && (nkv < 8 ? 8 % nkv == 0 : nkv % 8 == 0) ? 1 : 0; }
 
 // One launch over sequences [seq_begin, seq_begin + num_seqs), all with at
 // most max_q_len tokens.  nsplit > 1 needs part_o / part_ml for the rows
@@ -752,8 +791,7 @@ extern "C" int sl_attention_mfma_shares_keys() { return SHARED_FITS ? 1 : 0; }
 // Prompt portions go to the workgroups that share keys through LDS once the
 // launch would have shared_min_waves wavefronts of 32 columns or more;
 // pair_tiles: see the kernel; narrow_below: with fewer workgroups of 128
-// columns than this (but a third of it at least: smaller launches are all
-// latency either way), workgroups of 64 columns are launched instead.
+// columns than this, workgroups of 64 columns are launched instead.
 extern "C" const char* sl_attention_mfma(
     const void* qkv, int row_stride, const void* kc, const void* vc, const int* block_tables,
     int max_pages, const int* cu_q, const int* positions, int seq_begin, int num_seqs,
@@ -772,7 +810,7 @@ extern "C" const char* sl_attention_mfma(
   const int g = nh / nkv;
   AttnParams P{(const __bf16*)qkv, row_stride, (const __bf16*)kc, (const __bf16*)vc, block_tables,
                max_pages, cu_q, positions, seq_begin, nh, nkv, page, scale, window, nsplit,
-               (__bf16*)out, part_o, part_ml, part_row0, pair_tiles, out_rows};
+               (__bf16*)out, part_o, part_ml, part_row0, pair_tiles, out_rows, 0, 0, 0};
   SL_CHECK(out_rows >= 0 && (out_rows == 0 || (max_q_len == 1 && seq_begin == 0 && out_rows == num_seqs)),
            "attention_mfma: a result laid out by k-step is that of a step of single tokens, all of its rows");
   const long long cols = (long long)max_q_len * g;
@@ -799,22 +837,22 @@ extern "C" const char* sl_attention_mfma(
                                                                   part_row0, (__bf16*)out, out_rows);
     return sl_launch_status();
   }
-  // Prompt portions.  One wavefront per 32 columns, each reading its keys
-  // straight from the pages, has the most wavefronts in flight and wins while
-  // the chip is not full; with more of them than about two per SIMD the
-  // delivery of operands from L2 limits it and the workgroups that share a
-  // block through LDS win (MI355X, 7B shape, one prompt: 2,048 tokens 97 us
-  // against 108 us, 8,192 tokens 1,050 us against 854 us); the caller sets
-  // the crossover.
+  // Prompt portions.  The workgroups that share a block through LDS, or one
+  // wavefront per 32 columns, each reading its keys straight from the pages;
+  // the caller sets the crossover.  (MI355X, 7B shape: with the launch laid out
+  // by chiplet and a workgroup per tile the LDS form is as fast or faster at
+  // every size measured: one prompt of 128 / 512 / 1,024 / 2,048 tokens 11.8 /
+  // 19.1 / 31.8 / 57.5 us against 14.9 / 20.2 / 42.0 / 97 us; eight prompts of
+  // 512: 46 against 99 us; 512 tokens after 7,680: 108 against 278 us.)
   const long long tiles = (cols + 31) / 32;
   SL_CHECK(tiles <= 1 << 30, "attention_mfma: too many column tiles");
-  const bool shared = cols > 16 && SHARED_FITS && tiles * nkv * num_seqs >= shared_min_waves;
+  const bool shared = SHARED_FITS && tiles * nkv * num_seqs >= shared_min_waves;
   if (nsplit > 1) {
     SL_CHECK(shared && !pair_tiles, "attention_mfma: prompt portions are split only as unpaired tiles through LDS");
     SL_CHECK(nsplit <= 64 * COMBINE_PER_LANE && part_o != nullptr && part_ml != nullptr && part_rows > 0,
              "attention_mfma: a split launch needs partial buffers for its rows and not too many splits");
   }
-  if (cols <= 16) {
+  if (!shared && cols <= 16) {
     if (fold) attention_mfma_kernel<1, false, true><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);
     else attention_mfma_kernel<1, false, false><<<dim3(1, nkv, num_seqs), 64, 0, stream>>>(P);
   } else if (!shared) {
@@ -825,9 +863,18 @@ extern "C" const char* sl_attention_mfma(
     // workgroups of 128 columns, or of 64 when those would leave SIMDs with one wavefront
     long long wg = (cols + 32 * SHARED_WAVES - 1) / (32 * SHARED_WAVES);
     const long long wide = (pair_tiles ? (wg + 1) / 2 : wg) * nkv * num_seqs;
-    const bool narrow = nsplit == 1 && wide < narrow_below && wide >= narrow_below / 3;
+    const bool narrow = nsplit == 1 && wide < narrow_below;
     if (narrow) wg = (cols + 16 * SHARED_WAVES - 1) / (16 * SHARED_WAVES);
-    const dim3 grid((unsigned)(pair_tiles ? (wg + 1) / 2 : wg * nsplit), nkv, num_seqs);
+    dim3 grid((unsigned)(pair_tiles ? (wg + 1) / 2 : wg * nsplit), nkv, num_seqs);
+    if (sl_attention_mfma_by_chiplet(nkv)) {                     // (else the grid stays laid out pair by pair)
+      P.by_chiplet = 1;
+      P.grid_x = (int)grid.x;
+      P.num_seqs = num_seqs;
+      const long long each = nkv < 8 ? (long long)((grid.x + 8 / nkv - 1) / (8 / nkv)) * num_seqs
+                                     : (long long)grid.x * num_seqs * (nkv / 8);
+      SL_CHECK(8 * each < (1ll << 31), "attention_mfma: grid too large");
+      grid = dim3((unsigned)(8 * each), 1, 1);
+    }
     if (narrow) {
       if (fold) attention_mfma_shared_kernel<true, 1><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);
       else attention_mfma_shared_kernel<false, 1><<<grid, 64 * SHARED_WAVES, 0, stream>>>(P);

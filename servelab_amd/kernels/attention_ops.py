@@ -301,7 +301,8 @@ class AttentionOps:
 
     def _pair_prompt_tiles(self, tiles, prompts_and_heads) -> bool:
         """Whether the workgroups of a whole prompt's attention take a late tile of the causal triangle and
-        its early mirror (equal work for all, half as many workgroups) or a tile each, long ones first.
+        its early mirror (equal work for all, half as many workgroups) or a tile each, long ones first;
+        asked only for launches that are not laid out by chiplet, which always take a tile each.
         Equal workgroups fill the chip in rounds of two per CU, and the last round may be nearly empty;
         tiles of their own leave the balance to the order in which workgroups start, at the price of
         twice the prologues.  7B shape, one prompt, pairs against a tile each: 4,096 tokens (448 pairs, one
@@ -337,22 +338,29 @@ class AttentionOps:
             shared = (waves >= self.SHARED_ATTENTION_MIN_WAVES and
                       batch.max_ctx_len >= self.SHARED_ATTENTION_MIN_CONTEXT and
                       bool(self._lib[lib].sl_attention_mfma_shares_keys()))
-            # tiles of a causal triangle differ in length and are paired; those of a portion
-            # that starts deeper in its context than it is long do not
+            tiles = -(-batch.max_q_len * (nh // nkv) // 128) * nkv * n_pre      # workgroups of 128 columns
+            # tiles of a causal triangle differ in length; those of a portion that starts deeper in
+            # its context than it is long do not
             triangle = batch.max_ctx_len < 2 * batch.max_q_len
-            pair = triangle and self._pair_prompt_tiles(-(-batch.max_q_len * (nh // nkv) // 128), nkv * n_pre)
-            # few unpaired tiles over a long context: each is cut into shares of its keys
+            by_chiplet = bool(self._lib[lib].sl_attention_mfma_by_chiplet(nkv))
+            pair = (triangle and not by_chiplet and
+                    self._pair_prompt_tiles(-(-batch.max_q_len * (nh // nkv) // 128), nkv * n_pre))
+            # few tiles over a long context: each is cut into shares of its keys
             nsplit, part_o, part_ml = 1, None, None
             if shared and not triangle:
-                nsplit = max(1, min(self.PROMPT_SPLIT_MAX, batch.max_ctx_len // 32 // self.PROMPT_SPLIT_MIN_BLOCKS,
-                                    -(-self.PROMPT_SPLIT_WORKGROUPS // -(-waves // 4)),
+                blocks = batch.max_ctx_len // 32
+                nsplit = self.PROMPT_SPLIT_WORKGROUPS // tiles
+                if blocks >= self.PROMPT_SPLIT_DEEP_BLOCKS:
+                    nsplit = max(nsplit, self.PROMPT_SPLIT_DEEP)
+                nsplit = max(1, min(nsplit, self.PROMPT_SPLIT_MAX, blocks // self.PROMPT_SPLIT_MIN_BLOCKS,
+                                    int(self._lib[lib].sl_attention_mfma_max_splits()),
                                     self.PROMPT_SPLIT_BYTES // (n_pre_tok * nh * D * 4)))
             if nsplit > 1:
                 part_o = self._new((n_pre_tok, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
                        0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
-                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS, 0)
+                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS if triangle else 0, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:

@@ -85,24 +85,35 @@ class Tuning:
     # the same for the matrix-core kernel (384, 768 and 1,024 measured within noise or slower)
     target_waves: int = 512
     # prompt launches share keys through LDS from this many 32-column wavefronts and this context
-    # on (7B shape, one prompt: 1,024 tokens 46 us either way, 2,048: 80 against 95 us, 8,192: 737
-    # against 1,125 us; eight prompts of 256: 23.5 against 21.6 us)
-    shared_attention_min_waves: int = 1024
-    shared_attention_min_context: int = 1024
-    # such a launch with fewer workgroups than this and unpaired tiles (a portion deep in a long
-    # context) has every tile cut into shares of at least min_blocks key blocks, at most max, and
-    # no more than keep the partial outputs below split_bytes
-    prompt_split_workgroups: int = 4096
-    prompt_split_min_blocks: int = 64
-    prompt_split_max: int = 8
+    # on (7B shape, laid out by chiplet, a workgroup per tile: as fast or faster than a wavefront
+    # per 32 columns straight from the pages at every size measured, from 8 tokens to 32 k)
+    shared_attention_min_waves: int = 0
+    shared_attention_min_context: int = 0
+    # a launch of unpaired tiles that does not start at the beginning of its contexts (a portion
+    # deep in a prompt) has every tile cut into shares of its keys, a workgroup each: as many as
+    # bring the launch to split_workgroups workgroups (7B shape: 512 tokens after 7,680, 112 tiles:
+    # 223 / 135 / 108 / 116 us in 1 / 2 / 4 / 8 shares; 32 tokens after 4,064, 8 tiles: 118 us in one,
+    # 23.5 in 16), from deep_blocks key blocks on at least split_deep (2,048 tokens after 30,720: 1,106
+    # / 1,023 / 1,065 us in 1 / 4 / 8), at most split_max, none of fewer than min_blocks key blocks
+    # (16 tokens after 2,032, 16 requests: 34 us with shares of 8 blocks, 46 us of 4), and no more
+    # than keep the partial outputs below split_bytes
+    prompt_split_workgroups: int = 512
+    prompt_split_min_blocks: int = 8
+    prompt_split_max: int = 32
+    prompt_split_deep_blocks: int = 384
+    prompt_split_deep: int = 4
     prompt_split_bytes: int = 512 << 20
-    # a launch of fewer workgroups of 128 columns than this (and a third of it at least) takes
-    # workgroups of 64 columns: a wavefront then holds 16 columns and three fit a SIMD
-    # (2,048 tokens of the 7B shape: 77 against 88 us)
-    narrow_attention_workgroups: int = 400
-    # a workgroup of a whole prompt's launch takes a late tile of the causal triangle and its early mirror,
-    # unless the pairs would fill the chip (two workgroups a CU) in several rounds, the last of them
-    # mostly empty: below this share of the slots of all rounds, every tile gets a workgroup of its own
+    # a launch of whole prompts with fewer workgroups of 128 columns than this takes workgroups of 64
+    # columns: a wavefront then holds 16 columns and three fit a SIMD (7B shape, one prompt, a workgroup
+    # per tile: 2,048 tokens 57.5 against 71.4 us, 2,560: 78 against 86, 3,072: 113 against 102; portions
+    # deep in a context keep 128 columns: 2,048 tokens after 6,144: 290 against 332 us)
+    narrow_attention_workgroups: int = 600
+    # where the launch is not laid out by chiplet (3, 5, 6, 7, 9.. kv heads), a workgroup of a whole
+    # prompt takes a late tile of the causal triangle and its early mirror, unless the pairs would
+    # fill the chip (two workgroups a CU) in several rounds, the last of them mostly empty: below
+    # this share of the slots of all rounds, every tile gets a workgroup of its own.  Laid out by
+    # chiplet, a workgroup per tile, long tiles first, is as fast or faster everywhere (7B shape:
+    # 1,536 tokens 44 against 57 us, 2,048: 57.5 against 70, 4,096: 168 against 178, 8,192: 537 against 613)
     pair_prompt_tiles: bool = True
     unpaired_below_fill: float = 0.9
 

@@ -782,6 +782,7 @@ def test_paged_attention(both, nh, nkv, D, page, window, units):
 
 @pytest.mark.parametrize("nh,nkv,D,page", [(8, 1, 32, 16), (28, 4, 128, 16), (6, 2, 192, 64),
                                            (40, 2, 64, 32), (3, 3, 96, 16), (66, 1, 32, 16),
+                                           (16, 8, 64, 16), (32, 16, 32, 32),     # 1, 2, 4, 8, 16 kv heads: laid out by chiplet
                                            (4, 2, 256, 16)])     # 256: no LDS form; the same calls take the other kernel
 @pytest.mark.parametrize("window", [None, 16, 50])
 @pytest.mark.parametrize("form", ["paired", "a tile each", "unpaired", "shares"])
