@@ -1682,10 +1682,21 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
   const int t = threadIdx.x, lane = t & 63, i = lane & 15, gq = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = wave / WN, wn = wave % WN;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  // Workgroups go to the eight chiplets in turn, each with an L2 of its own, and the workgroups of
+  // one share of K read the same columns of x: the grid is one-dimensional and chiplet c takes a
+  // contiguous eighth of the (share, column tile, row tile) triples, so that a share's slice of x
+  // lies in one or two L2s instead of eight and the rows of W that two row tiles share come from
+  // memory once.
+  const int gx = (N + BN - 1) / BN, gy = (M + BM - 1) / BM, total = gx * gy * KS;
+  const int per = (total + 7) / 8;
+  const int triple = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= per || triple >= total) return;       // (the whole workgroup)
+  // (row tiles fastest: the workgroups that read the same rows of W run side by side on one chiplet)
+  const int share = triple / (gx * gy);
+  const int m0 = triple % gy * BM, n0 = triple / gy % gx * BN;
   const int chunks = K / 64;
-  const int cbeg = (int)((long long)chunks * blockIdx.z / KS);
-  const int cend = (int)((long long)chunks * (blockIdx.z + 1) / KS);
+  const int cbeg = (int)((long long)chunks * share / KS);
+  const int cend = (int)((long long)chunks * (share + 1) / KS);
 
   // what this lane fetches of every chunk: unit `cu ^ f(row)` of row 8 q + lane / 8 of the stage
   const __bf16* src[LOADS];
@@ -1767,7 +1778,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
       const bool whole = n + 3 < N && N % 4 == 0;
       f32x4 r = acc[u][v];
       if (KS > 1) {
-        float* o = (float*)y + ((size_t)blockIdx.z * M + m) * N + n;
+        float* o = (float*)y + ((size_t)share * M + m) * N + n;
         if (whole) {
           *(f32x4*)o = r;
         } else {
@@ -1818,8 +1829,9 @@ extern "C" const char* sl_gemm_block(const void* x, const void* w, const float* 
   // (Tiles of 64 x 256 and 128 x 256 for fewer rows of x were built and measured: alone they beat the
   // LDS-staged kernel above, in a decode step of 24 to 128 requests they lost 2-5 % tokens/s to it,
   // so that kernel keeps those rows and this one starts where it ends.)
-  const dim3 grid((N + 127) / 128, (M + 255) / 256, ks);
-  SL_CHECK(grid.y <= 65535, "gemm_block: too many rows");
+  const long long triples = (long long)((N + 127) / 128) * ((M + 255) / 256) * ks;
+  SL_CHECK(triples < (1ll << 28), "gemm_block: too many tiles");
+  const dim3 grid((unsigned)(8 * ((triples + 7) / 8)));              // laid out by chiplet (see the kernel)
   gemm_block_kernel<4, 2><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, ks);
   const char* e = sl_launch_status();
   if (e || ks == 1 || y == nullptr) return e;
