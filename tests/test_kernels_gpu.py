@@ -815,6 +815,37 @@ def test_prompt_attention_through_lds(nh, nkv, D, page, window, form, units):
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+def test_portions_deep_in_a_context_take_shares_of_their_keys_by_default():
+    """The launches the table chooses by itself (no threshold moved): whole prompts, short or long,
+    take the kernel that shares keys through LDS with a workgroup for every tile; a portion that
+    starts deep in its context, down to two tokens, has its tiles cut into shares of their keys
+    (no share of fewer than 8 key blocks, none for a context of fewer than 16).  Results against
+    the plain computation."""
+    from servelab_amd.kernels import HipOps
+    dt = torch.bfloat16
+    nh, nkv, D, page = 8, 2, 64, 16
+    for seqs, shares in (([(40, 40), (300, 300), (7, 7)], 1), ([(2000, 40), (700, 3), (333, 2)], 7),
+                         ([(4100, 2)], 16), ([(300, 5)], 1), ([(520, 9), (514, 2)], 2)):
+        ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+        seen = []
+        call = ops._call
+
+        def spy(stem, name, *args):
+            if name.startswith("sl_attention_mfma@"):
+                seen.append((args[17], args[18], args[19]))          # shares, wavefronts for the LDS form, pairs
+            return call(stem, name, *args)
+        ops._call = spy
+        qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=11)
+        qkv, scale = in_units(UNITS[1], qkv, nh, D, 1.0 / math.sqrt(D))
+        got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, None)
+        assert seen == [(shares, 0, 0)], (seqs, seen)
+        ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                                  types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                           for k, v in vars(batch).items()}),
+                                  scale, None)
+        assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+
+
 def test_decode_shares_fill_whole_rounds_over_the_cus():
     """The number of shares of a request's keys at the batch sizes it was measured at (4 kv heads, 256 CUs,
     contexts of 4,096: 64 shares at most): never slightly more wavefronts than a whole number per CU."""
