@@ -197,12 +197,14 @@ __global__ void rope_store_kernel(act_t* __restrict__ qkv, const SplitProduct sp
   }
 }
 
-// The same work in two vectorised kernels, for head sizes that are multiples
-// of 16 (many-token steps: the per-pair kernel above needs one block of 64
-// threads per token and head and moves 2 bytes per access).  With few tokens
-// the second launch costs more than the wider accesses save (64 tokens of the
-// 7B shape: 10.9 us in two kernels against 5.2 us in one).
-constexpr int VECTOR_MIN_TOKENS = 256;
+// The same work with 16-byte accesses, for head sizes that are multiples of 16
+// (many-token steps: the per-pair kernel above needs one block of 64 threads
+// per token and head and moves 2 bytes per access).  With few tokens, or with
+// several partial sums to add, the per-pair kernel's many threads win (7B
+// shape, graph-timed: 64 tokens 5.2 against 3.3 us, 256: 5.7 against 5.2, 512:
+// 6.5 against 7.9, 2,048: 13.0 against 22.8; 512 tokens in 4 partial sums: 16.3
+// against 12.8).
+constexpr int VECTOR_MIN_TOKENS = 384;
 struct __attribute__((aligned(16))) Act8 { act_t v[8]; };
 struct __attribute__((aligned(16))) F4 { float v[4]; };
 
@@ -210,13 +212,13 @@ struct __attribute__((aligned(16))) F4 { float v[4]; };
 // one token and writes them back, k also to its cache row.  From partial sums
 // (sp.parts): the 16 inputs are bias + the sums, q is written to qkv and k only
 // to its cache row, as in the kernel above.
-__global__ __launch_bounds__(256) void rope_store_qk_kernel(
-    act_t* __restrict__ qkv, const SplitProduct sp, const float* __restrict__ cosv,
+__device__ __forceinline__ void rope_store_qk_block(
+    int t, int by, int gy, act_t* __restrict__ qkv, const SplitProduct& sp, const float* __restrict__ cosv,
     const float* __restrict__ sinv, const int* __restrict__ slots, act_t* __restrict__ kc, int nh,
     int nkv, int D, int rot, int page, int pairs8, float qscale) {
-  const int t = blockIdx.x, half = rot / 2, chunks = D / 16, rotated = rot / 16;
+  const int half = rot / 2, chunks = D / 16, rotated = rot / 16;
   const int items = (nh + nkv) * chunks;
-  for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < items; w += gridDim.y * blockDim.x) {
+  for (int w = by * blockDim.x + threadIdx.x; w < items; w += gy * blockDim.x) {
     const int hd = w / chunks, c = w % chunks;
     // chunks below `rotated` hold 8 pairs; the others 16 channels that pass unrotated
     const bool turn = c < rotated;
@@ -283,12 +285,11 @@ __global__ __launch_bounds__(256) void rope_store_qk_kernel(
 // v heads: a block takes 16 consecutive tokens of one kv head through LDS, so
 // that neighbouring lanes write neighbouring slots of a channel's row (tokens
 // of one request usually sit in consecutive slots of a page).
-__global__ __launch_bounds__(256) void store_v_kernel(
-    const act_t* __restrict__ qkv, const SplitProduct sp, const int* __restrict__ slots,
+__device__ __forceinline__ void store_v_block(
+    int t0, int kvh, const act_t* __restrict__ qkv, const SplitProduct& sp, const int* __restrict__ slots,
     act_t* __restrict__ vc, int T, int nh, int nkv, int D, int page) {
   __shared__ act_t tile[16][256 + 2];
   __shared__ int slot_of[16];
-  const int t0 = blockIdx.x * 16, kvh = blockIdx.y;
   const int nt = T - t0 < 16 ? T - t0 : 16;
   if (threadIdx.x < 16) slot_of[threadIdx.x] = threadIdx.x < nt ? slots[t0 + threadIdx.x] : 0;
   for (int idx = threadIdx.x; idx < nt * D; idx += blockDim.x) {
@@ -309,6 +310,25 @@ __global__ __launch_bounds__(256) void store_v_kernel(
       const int slot = slot_of[i];
       vc[(((size_t)(slot / page) * nkv + kvh) * D + d) * page + slot % page] = tile[i][d];
     }
+  }
+}
+
+// One launch for both: the first v_blocks workgroups take the v heads (16 tokens of one kv head
+// each), the others the q and k heads (gy workgroups a token).  The two halves read and write
+// different heads, so they run side by side instead of one launch after the other (2,048 tokens
+// of the 7B shape: 14 + 7 us in two launches).
+__global__ __launch_bounds__(256) void rope_store_vec_kernel(
+    act_t* __restrict__ qkv, const SplitProduct sp, const float* __restrict__ cosv,
+    const float* __restrict__ sinv, const int* __restrict__ slots, act_t* __restrict__ kc,
+    act_t* __restrict__ vc, int T, int nh, int nkv, int D, int rot, int page, int pairs8, float qscale,
+    int v_blocks, int gy) {
+  const int b = blockIdx.x;
+  if (b < v_blocks) {                                // (the same for the whole workgroup)
+    const int groups = (T + 15) / 16;
+    store_v_block(b % groups * 16, b / groups, qkv, sp, slots, vc, T, nh, nkv, D, page);
+  } else {
+    rope_store_qk_block((b - v_blocks) / gy, (b - v_blocks) % gy, gy, qkv, sp, cosv, sinv, slots, kc, nh, nkv, D, rot,
+                        page, pairs8, qscale);
   }
 }
 
@@ -339,15 +359,15 @@ extern "C" const char* sl_rope_store(void* qkv, const float* cosv, const float* 
                        ((uintptr_t)cosv % 16) == 0 && ((uintptr_t)sinv % 16) == 0;
   const bool sums_aligned = parts == nullptr || (((uintptr_t)parts % 16) == 0 && ((uintptr_t)bias % 16) == 0 &&
                                                   ((size_t)T * (nh + 2 * nkv) * D) % 4 == 0);
-  if (T >= VECTOR_MIN_TOKENS && D % 16 == 0 && rot % 16 == 0 && D <= 256 && aligned && sums_aligned &&
-      nkv <= 65535) {
+  if (T >= VECTOR_MIN_TOKENS && nparts <= 1 && D % 16 == 0 && rot % 16 == 0 && D <= 256 && aligned &&
+      sums_aligned) {
     const int items = (nh + nkv) * (D / 16);
-    rope_store_qk_kernel<<<dim3(T, (items + 255) / 256 < 64 ? (items + 255) / 256 : 64), 256, 0, stream>>>(
-        (act_t*)qkv, sp, cosv, sinv, slots, (act_t*)kc, nh, nkv, D, rot, page, pairs8, qscale);
-    const char* e = sl_launch_status();
-    if (e || vc == nullptr) return e;
-    store_v_kernel<<<dim3((T + 15) / 16, nkv), 256, 0, stream>>>((const act_t*)qkv, sp, slots, (act_t*)vc, T,
-                                                                 nh, nkv, D, page);
+    const int gy = (items + 255) / 256 < 64 ? (items + 255) / 256 : 64;
+    const long long v_blocks = vc != nullptr ? (long long)((T + 15) / 16) * nkv : 0;
+    SL_CHECK(v_blocks + (long long)T * gy < (1ll << 31), "rope_store: too many tokens");
+    rope_store_vec_kernel<<<(unsigned)(v_blocks + (long long)T * gy), 256, 0, stream>>>(
+        (act_t*)qkv, sp, cosv, sinv, slots, (act_t*)kc, (act_t*)vc, T, nh, nkv, D, rot, page, pairs8, qscale,
+        (int)v_blocks, gy);
     return sl_launch_status();
   }
   rope_store_kernel<<<dim3(T, heads), 64, 0, stream>>>((act_t*)qkv, sp, cosv, sinv, slots, (act_t*)kc,

@@ -493,7 +493,7 @@ def test_rope_tables(both):
 
 
 @pytest.mark.parametrize("pairs8", [False, True])
-@pytest.mark.parametrize("T", [5, 37, 300])        # per-pair kernel for few tokens, vectorised kernels for many
+@pytest.mark.parametrize("T", [5, 37, 400])        # per-pair kernel for few tokens, the vectorised kernel for many
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (6, 1, 48, 32), (7, 7, 128, 64), (3, 1, 24, 16)])
 def test_rope_store(both, nh, nkv, D, page, pairs8, T):
     ops, emu, dt = both
@@ -522,7 +522,7 @@ def test_rope_store(both, nh, nkv, D, page, pairs8, T):
     assert torch.equal(kc[0], k_before)
 
 
-@pytest.mark.parametrize("T", [9, 300])
+@pytest.mark.parametrize("T", [9, 400])
 @pytest.mark.parametrize("nh,nkv,D,rot,page,pairs8", [(4, 2, 32, 16, 16, True), (4, 2, 32, 16, 16, False),
                                                       (6, 1, 48, 32, 32, True), (3, 3, 24, 10, 16, False),
                                                       (2, 1, 128, 64, 64, True), (5, 1, 64, 0, 16, True)])
@@ -588,16 +588,17 @@ def test_rotation_plans():
                         None, None, None, 16)
 
 
-@pytest.mark.parametrize("T", [40, 300])
+@pytest.mark.parametrize("T,nparts", [(40, 3), (400, 3), (400, 1)])
 @pytest.mark.parametrize("nh,nkv,D,page", [(4, 2, 16, 16), (28, 4, 128, 16), (5, 1, 48, 32), (3, 1, 96, 64)])
-def test_rope_store_from_partial_sums(both, nh, nkv, D, page, T):
+def test_rope_store_from_partial_sums(both, nh, nkv, D, page, T, nparts):
     """The q/k/v product arrives as float partial sums of a split K plus a bias:
-    rotation and cache write see their sum; q lands in the buffer.  With few tokens one
-    block per token and head, with many the vectorised pair of kernels."""
+    rotation and cache write see their sum; q lands in the buffer.  With few tokens or
+    several sums one block per token and head, with many tokens and one sum (the library's
+    float32 product) the vectorised kernel."""
     from servelab_amd.kernels.ops import PartialSums
     ops, emu, dt = both
     pages, N = -(-T // page) + 3, (nh + 2 * nkv) * D
-    parts = randn(3, T, N, seed=1)
+    parts = randn(nparts, T, N, seed=1)
     bias = randn(N, seed=2)
     inv = (1.0 / 10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D)).cuda()
     cos, sin = emu.rope_tables(torch.arange(50, 50 + T, dtype=torch.int32).cuda(), inv)
