@@ -1669,11 +1669,12 @@ template <int N_> __device__ __forceinline__ void block_wait_loads() {
   __builtin_amdgcn_s_waitcnt((N_ & 15) | (7 << 4) | (15 << 8) | ((N_ >> 4) << 14));
 }
 
-template <int WM, int WN>
+template <int WM, int WN, int STAGES>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
     const __bf16* __restrict__ x, const __bf16* __restrict__ w, const float* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int out_f32, int KS) {
-  constexpr int WAVES = WM * WN, BM = 64 * WM, BN = 64 * WN, STAGES = 3;
+  constexpr int WAVES = WM * WN, BM = 64 * WM, BN = 64 * WN;
+  static_assert(STAGES == 2 || STAGES == 3, "a ring of two or three stages");
   constexpr int ROWS = BM + BN;                      // rows of a stage: x, then W; 128 bytes each
   constexpr int STAGE_BYTES = ROWS * 128;
   constexpr int LOADS = ROWS / 8 / WAVES;            // wavefront-wide loads (8 rows) a wavefront makes per chunk
@@ -1731,7 +1732,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
 
   if (cbeg < cend) {
     fetch(cbeg, 0);
-    if (cbeg + 1 < cend) {
+    if (STAGES == 3 && cbeg + 1 < cend) {
       fetch(cbeg + 1, 1);
       block_wait_loads<LOADS>();
     } else {
@@ -1742,8 +1743,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
   }
   int stage = 0;
   for (int c = cbeg; c < cend; ++c) {
-    const bool more = c + 2 < cend;
-    if (more) fetch(c + 2, stage >= 1 ? stage - 1 : 2);        // the stage the last chunk was read from
+    const bool more = c + STAGES - 1 < cend;
+    if (more) fetch(c + STAGES - 1, stage >= 1 ? stage - 1 : STAGES - 1);        // the stage the last chunk was read from
     const char* st = ring + STAGE_BYTES * stage;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
@@ -1759,11 +1760,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
         for (int v = 0; v < 4; ++v)
           acc[u][v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[v], acc[u][v], 0, 0, 0);
     }
-    if (more) block_wait_loads<LOADS>();                       // all but the chunk just asked for
+    if (more && STAGES == 3) block_wait_loads<LOADS>();        // all but the chunk just asked for
     else block_wait_loads<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" : : : "memory");
-    stage = stage == 2 ? 0 : stage + 1;
+    stage = stage == STAGES - 1 ? 0 : stage + 1;
   }
 
   // lane: row m of x (16 v + i), four consecutive rows n of W (16 u + 4 gq ..)
@@ -1815,7 +1816,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_block_kernel(
 // x and W row-major.  ks > 1: `part` holds ks * M * N floats; with y == nullptr they are left
 // there for the reader to add (and the bias with them), else splitk_reduce adds them into y.
 extern "C" const char* sl_gemm_block(const void* x, const void* w, const float* bias, void* y,
-                                     int M, int N, int K, int out_f32, int ks, float* part,
+                                     int M, int N, int K, int out_f32, int ks, int square, float* part,
                                      hipStream_t stream) {
   SL_CHECK(M > 0 && N > 0 && K > 0, "gemm_block: sizes must be positive");
   SL_CHECK(K % 64 == 0, "gemm_block: K must be a multiple of 64");
@@ -1829,10 +1830,15 @@ extern "C" const char* sl_gemm_block(const void* x, const void* w, const float* 
   // (Tiles of 64 x 256 and 128 x 256 for fewer rows of x were built and measured: alone they beat the
   // LDS-staged kernel above, in a decode step of 24 to 128 requests they lost 2-5 % tokens/s to it,
   // so that kernel keeps those rows and this one starts where it ends.)
-  const long long triples = (long long)((N + 127) / 128) * ((M + 255) / 256) * ks;
+  // square: tiles of 256 x 256 (sixteen wavefronts, a ring of two stages in 128 KB of LDS) instead of
+  // 256 x 128 (eight wavefronts, three stages): a workgroup pulls 512 rows for 256 x 256 of result
+  // instead of 384 for 256 x 128, which is what the time of these products follows.
+  const int bn = square ? 256 : 128;
+  const long long triples = (long long)((N + bn - 1) / bn) * ((M + 255) / 256) * ks;
   SL_CHECK(triples < (1ll << 28), "gemm_block: too many tiles");
   const dim3 grid((unsigned)(8 * ((triples + 7) / 8)));              // laid out by chiplet (see the kernel)
-  gemm_block_kernel<4, 2><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, ks);
+  if (square) gemm_block_kernel<4, 4, 2><<<grid, 1024, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, ks);
+  else gemm_block_kernel<4, 2, 3><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, ks);
   const char* e = sl_launch_status();
   if (e || ks == 1 || y == nullptr) return e;
   const size_t total = (size_t)M * N;

@@ -78,11 +78,11 @@ class AttentionOps:
         fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
                  and weight.tiled is not None and weight.shape == (N, K))
         if not fused:
-            shares = 0 if isinstance(x, ScaledRows) else self._block_shares(M, N, K, weight)
-            if shares:
+            plan = None if isinstance(x, ScaledRows) else self._block_plan(M, N, K, weight)
+            if plan:
                 # K split over workgroups of the block kernel; the rotation kernel adds the partial sums up
                 self._check(x, self.act_dtype, (M, K), "x")
-                product = self.linear_block(x, weight, bias, ks=shares, partial=True)
+                product = self.linear_block(x, weight, bias, ks=plan[0], partial=True, square=plan[1])
                 qkv = self._new((M, N))
                 self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
                                 True, split=product, rot_dim=rot, q_scale=q_scale)

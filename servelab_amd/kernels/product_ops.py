@@ -192,11 +192,11 @@ class ProductOps:
                 return self.linear_f32_mfma(x, weight.w, bias)
             return self.linear_tiled(x, weight.w, bias, out_f32)
         limit = self._few_rows_limit(weight)
-        shares = self._block_shares(M, N, K, weight)
-        if shares:
+        plan = self._block_plan(M, N, K, weight)
+        if plan:
             # (deferred: the norm adds the partial sums)
-            return self.linear_block(x, weight, bias, out_f32, shares,
-                                     partial=defer and self.fuse_norms and not out_f32)
+            return self.linear_block(x, weight, bias, out_f32, plan[0],
+                                     partial=defer and self.fuse_norms and not out_f32, square=plan[1])
         if (defer and self.fuse_norms and not out_f32 and self.WIDE_MIN_M <= M <= limit
                 and K % 32 == 0 and N % 4 == 0 and self._takes_mid(M, N, K)):
             return self.linear_mid(x, weight, bias, partial=True,     # the norm adds the partial sums
@@ -269,30 +269,38 @@ class ProductOps:
                    int(out_f32), int(gated), int(ks), self.MID_WIDE_WORKGROUPS, self._num_cus, _p(part))
         return y
 
-    def _block_shares(self, M, N, K, weight) -> int:
-        """Over how many workgroups the block kernel splits K for a product of
-        M rows, or 0 when the product is not one of its own: bfloat16, a
-        row-major copy of the weight, K in chunks of 64, a matrix of few rows
-        (its tiles alone would leave most CUs idle, which is what the split
-        repairs) but of MID_MIN_ELEMENTS_MANY elements at least (smaller ones
-        stay with the kernels they were measured on), and BLOCK_MIN_M to
-        BLOCK_MAX_M rows of x.  As many shares as give every CU a workgroup,
-        16 at most, of at least 3 chunks each (7B shape, down projection at 256
-        rows: 70 / 44 / 41 us with 4 / 8 / 9 shares; q/k/v: 21 / 17 / 26 us
-        with 4 / 7 / 8, the last being more workgroups than CUs)."""
+    def _block_plan(self, M, N, K, weight):
+        """How the block kernel takes a product of M rows: (shares of K, square tiles), or None
+        when the product is not one of its own: bfloat16, a row-major copy of the weight, K in
+        chunks of 64, a matrix of few rows (its tiles alone would leave most CUs idle, which is
+        what the split repairs) but of MID_MIN_ELEMENTS_MANY elements at least (smaller ones stay
+        with the kernels they were measured on).  Tiles of 256 x 128 for BLOCK_MIN_M to BLOCK_MAX_M
+        rows of x; tiles of 256 x 256 for matrices with long rows (K of BLOCK_SQUARE_MIN_K and
+        more: the down projection) from 257 to BLOCK_SQUARE_MAX_M rows, if their tiles and shares
+        fill three quarters of the CUs.  As many shares as give every CU a workgroup, 16 at most,
+        of at least 3 chunks each (7B shape, down projection at 256 rows: 70 / 44 / 41 us with 4 / 8
+        / 9 shares; q/k/v: 21 / 17 / 26 us with 4 / 7 / 8, the last being more workgroups than CUs;
+        down at 527 rows: 84 us in square tiles, 101 us in 256 x 128, 130 us in the library's tuned
+        kernel; at 1,024 rows 111 us in 4 shares, 144 us in 6)."""
         w = weight.w if isinstance(weight, LinearWeight) else weight
         if (self.act_dtype != torch.bfloat16 or not self.use_block_products or w is None
-                or K % 64 or N % 4 or N > self.BLOCK_MAX_N or N * K < self.MID_MIN_ELEMENTS_MANY
-                or not self.BLOCK_MIN_M <= M <= self.BLOCK_MAX_M):
-            return 0
+                or K % 64 or N % 4 or N > self.BLOCK_MAX_N or N * K < self.MID_MIN_ELEMENTS_MANY):
+            return None
+        if K >= self.BLOCK_SQUARE_MIN_K and 256 < M <= self.BLOCK_SQUARE_MAX_M:
+            tiles = -(-N // 256) * -(-M // 256)
+            shares = min(16, K // 64 // 3, self._num_cus // tiles)
+            if shares >= 1 and 4 * tiles * shares >= 3 * self._num_cus:
+                return shares, True
+        if not self.BLOCK_MIN_M <= M <= self.BLOCK_MAX_M:
+            return None
         tiles = -(-N // 128) * -(-M // 256)
-        return max(1, min(16, K // 64 // 3, self._num_cus // tiles))
+        return max(1, min(16, K // 64 // 3, self._num_cus // tiles)), False
 
-    def linear_block(self, x, weight, bias, out_f32=False, ks=1, partial=False):
+    def linear_block(self, x, weight, bias, out_f32=False, ks=1, partial=False, square=False):
         """A few hundred rows over the row-major copy of the weight: workgroups
-        own a tile of 256 rows of x by 128 rows of W over one of ``ks`` shares
-        of K.  ``partial``: the product comes back as ``PartialSums`` for its
-        reader to add up."""
+        own a tile of 256 rows of x by 128 rows of W (``square``: by 256) over
+        one of ``ks`` shares of K.  ``partial``: the product comes back as
+        ``PartialSums`` for its reader to add up."""
         M, K = x.shape
         N = weight.shape[0]
         w = weight.w if isinstance(weight, LinearWeight) else weight
@@ -303,13 +311,14 @@ class ProductOps:
         part = self._new((ks, M, N), torch.float32) if ks > 1 or partial else None
         if partial:
             if ks > 1:
-                self._call("gemm", "sl_gemm_block", _p(x), _p(w), None, None, M, N, K, 0, int(ks), _p(part))
+                self._call("gemm", "sl_gemm_block", _p(x), _p(w), None, None, M, N, K, 0, int(ks), int(square),
+                           _p(part))
             else:
-                self._call("gemm", "sl_gemm_block", _p(x), _p(w), None, _p(part), M, N, K, 1, 1, None)
+                self._call("gemm", "sl_gemm_block", _p(x), _p(w), None, _p(part), M, N, K, 1, 1, int(square), None)
             return PartialSums(part, bias)
         y = self._new((M, N), torch.float32 if out_f32 else None)
         self._call("gemm", "sl_gemm_block", _p(x), _p(w), _p(bias), _p(y), M, N, K, int(out_f32),
-                   int(ks), _p(part))
+                   int(ks), int(square), _p(part))
         return y
 
     def linear_skinny(self, x, weight, bias, out_f32=False):

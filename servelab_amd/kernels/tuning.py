@@ -67,6 +67,10 @@ class Tuning:
     block_max_n: int = 8192
     block_min_m: int = 129
     block_max_m: int = 512
+    # matrices with rows of this many values and more (the down projection) take tiles of 256 x 256 from
+    # 257 rows of x up to this many (7B shape, down at 768 / 1,024 / 1,536 rows: 83 / 111 / 168 us)
+    block_square_min_k: int = 8192
+    block_square_max_m: int = 1536
 
     # ---- few-rows consumer products on workgroups that stay
     # tiles per CU from which walking the tiles beats a workgroup per tile (gate/up: 9, head: 37;

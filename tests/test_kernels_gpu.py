@@ -1231,38 +1231,60 @@ def test_products_of_129_to_512_rows_of_matrices_of_few_rows_run_in_tiles():
     weight, b = ops.prepare_weight(w), randn(N, seed=3)
     for M in (129, 300, 512):
         x = randn(M, K, dtype=torch.bfloat16, seed=M)
-        shares = ops._block_shares(M, N, K, weight)
-        assert shares == max(1, min(K // 64 // 3, ops._num_cus // (N // 128 * -(-M // 256))))
+        shares, square = ops._block_plan(M, N, K, weight)
+        assert shares == max(1, min(K // 64 // 3, ops._num_cus // (N // 128 * -(-M // 256)))) and not square
         assert torch.equal(ops.linear(x, weight, b), ops.linear_block(x, weight, b, ks=shares))
         assert rel_err(ops.linear(x, weight, b), emu.linear(x, w, b)) < 2 ** -7
         delta = ops.linear(x, weight, b, defer=True)
         assert isinstance(delta, PartialSums) and delta.parts.shape == (shares, M, N)
         assert rel_err(ops.materialize(delta), emu.linear(x, w, b)) < 2 ** -7
-    assert not ops._block_shares(128, N, K, weight) and not ops._block_shares(513, N, K, weight)
-    assert not ops._block_shares(300, 8208, K, ops.prepare_weight(randn(8208, K, dtype=torch.bfloat16)))
-    assert not ops._block_shares(300, 256, K, ops.prepare_weight(w[:256].contiguous()))
+    assert not ops._block_plan(128, N, K, weight) and not ops._block_plan(513, N, K, weight)
+    assert not ops._block_plan(300, 8208, K, ops.prepare_weight(randn(8208, K, dtype=torch.bfloat16)))
+    assert not ops._block_plan(300, 256, K, ops.prepare_weight(w[:256].contiguous()))
+    # rows of 8,192 values and more (a down projection): tiles of 256 x 256 from 257 rows on, further up
+    # than the others, as long as tiles and shares fill three quarters of the CUs
+    K2, N2 = 8192, 1024
+    w2 = randn(N2, K2, dtype=torch.bfloat16, scale=0.02, seed=5)
+    long_rows, b2 = ops.prepare_weight(w2), randn(N2, seed=6)
+    ops._num_cus = 64
+    assert ops._block_plan(256, N2, K2, long_rows) == (8, False)
+    assert ops._block_plan(257, N2, K2, long_rows) == (8, True) and ops._block_plan(700, N2, K2, long_rows) == (5, True)
+    assert ops._block_plan(1536, N2, K2, long_rows) == (2, True) and not ops._block_plan(1537, N2, K2, long_rows)
+    ops._num_cus = 256
+    assert ops._block_plan(700, N2, K2, long_rows) == (16, True)
+    assert ops._block_plan(700, 512, K2, ops.prepare_weight(w2[:512].contiguous())) is None    # 6 tiles x 16 shares: too few
+    for M in (300, 700):
+        x = randn(M, K2, dtype=torch.bfloat16, seed=M)
+        shares, square = ops._block_plan(M, N2, K2, long_rows)
+        assert torch.equal(ops.linear(x, long_rows, b2), ops.linear_block(x, long_rows, b2, ks=shares, square=square))
+        assert rel_err(ops.linear(x, long_rows, b2), emu.linear(x, w2, b2)) < 2 ** -7
+        delta = ops.linear(x, long_rows, b2, defer=True)
+        assert isinstance(delta, PartialSums) and delta.parts.shape == (shares, M, N2)
+        assert rel_err(ops.materialize(delta), emu.linear(x, w2, b2)) < 2 ** -7
     ops.weight_layout = "tiled"
-    assert not ops._block_shares(300, N, K, ops.prepare_weight(w.clone()))
+    assert not ops._block_plan(300, N, K, ops.prepare_weight(w.clone()))
     ops.use_block_products = False
-    assert not ops._block_shares(300, N, K, weight)
+    assert not ops._block_plan(300, N, K, weight)
 
 
 @pytest.mark.parametrize("M,N,K,ks", [(17, 3584, 3584, 16), (64, 3584, 18944, 12), (65, 4608, 3584, 7), (128, 520, 640, 3),
                                       (129, 136, 64, 1), (160, 4608, 3584, 1), (300, 3584, 3584, 4), (512, 1000, 640, 2),
                                       (513, 1000, 640, 3), (700, 260, 128, 1), (200, 1001, 192, 2), (256, 130, 64, 1)])
-def test_products_in_tiles_over_the_row_major_copy(M, N, K, ks):
-    """The kernel alone at each of its tile shapes (up to 64 rows of x, up to 128, more), ragged in
-    rows and columns, with and without a split of K, a bias, float32 output and partial sums."""
+@pytest.mark.parametrize("square", [False, True])
+def test_products_in_tiles_over_the_row_major_copy(M, N, K, ks, square):
+    """The kernel alone in both of its tile shapes (256 x 128 with eight wavefronts and a ring of
+    three stages, 256 x 256 with sixteen and a ring of two), ragged in rows and columns, with and
+    without a split of K, a bias, float32 output and partial sums."""
     from servelab_amd.kernels import HipOps
     ops = HipOps(torch.bfloat16, "cuda:0")
     x = randn(M, K, dtype=torch.bfloat16, seed=1)
     w = randn(N, K, dtype=torch.bfloat16, scale=0.05, seed=2)
     b = randn(N, seed=3)
     ref = x.float() @ w.float().T
-    assert rel_err(ops.linear_block(x, w, b, out_f32=True, ks=ks), ref + b) < 2e-5
-    assert rel_err(ops.linear_block(x, w, None, ks=ks), ref) < 2 ** -7
-    assert rel_err(ops.linear_block(x, w, b, ks=1), ref + b) < 2 ** -7
-    parts = ops.linear_block(x, w, b, ks=ks, partial=True)
+    assert rel_err(ops.linear_block(x, w, b, out_f32=True, ks=ks, square=square), ref + b) < 2e-5
+    assert rel_err(ops.linear_block(x, w, None, ks=ks, square=square), ref) < 2 ** -7
+    assert rel_err(ops.linear_block(x, w, b, ks=1, square=square), ref + b) < 2 ** -7
+    parts = ops.linear_block(x, w, b, ks=ks, partial=True, square=square)
     assert parts.parts.shape == (ks, M, N) and parts.bias is b
     assert rel_err(parts.parts.sum(0) + b, ref + b) < 2e-5
     assert rel_err(ops.materialize(parts), ref + b) < 2 ** -7
