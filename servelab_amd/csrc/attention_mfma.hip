@@ -376,32 +376,11 @@ struct Columns {
 // One wavefront per workgroup; operands straight from the pages.  Used for
 // decode tokens (SPLIT: the wavefront takes one share of the key blocks) and
 // for prompt portions whose launch does not saturate L2.
-template <int NB, bool SPLIT, bool FOLD, bool PAIRS = false>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 256 ? 2 : 1))) void attention_mfma_kernel(const AttnParams P) {
-  const int lane = threadIdx.x, n = lane & 15, gq = lane >> 4;
-  const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
-  const int g = P.nh / P.nkv;
-  const int q0 = P.cu_q[seq];
-  const int qlen = P.cu_q[seq + 1] - q0;
-  const int ncols = qlen * g;
-  const int ntiles = (ncols + 16 * NB - 1) / (16 * NB);
-  const int tile_rev = blockIdx.x / P.nsplit, split = blockIdx.x % P.nsplit;
-  if (tile_rev >= ntiles) return;
-  const int tile = ntiles - 1 - tile_rev;          // long (late) tiles first
-  const int pos0 = P.positions[q0];
-  const int* table = P.block_tables + (size_t)seq * P.max_pages;
+// The key blocks [kb_begin, kb_end) of one wavefront's columns, operands straight from the pages.
+template <int NB, bool FOLD, bool PAIRS>
+__device__ __forceinline__ void walk_blocks(Columns<NB, FOLD>& C, const AttnParams& P, const int* table, int kvh,
+                                            int n, int gq, int kb_begin, int kb_end) {
   const int page = P.page, page_shift = 31 - __builtin_clz(page);
-
-  Columns<NB, FOLD> C;
-  C.init(P, q0, ncols, tile * 16 * NB, pos0, kvh, g, n, gq);
-  int kb_begin = C.kb_begin, kb_end = C.kb_end;
-  if (SPLIT) {
-    const int nblk = kb_end - kb_begin;
-    const int first = kb_begin + (int)((long long)nblk * split / P.nsplit);
-    kb_end = kb_begin + (int)((long long)nblk * (split + 1) / P.nsplit);
-    kb_begin = first;
-  }
-
   // The two table entries a block of 32 keys can touch are the same for every
   // lane, so they come through the scalar path, one block ahead of the keys.
   auto load_pages = [&](int kb, int (&pg)[2]) {
@@ -433,29 +412,29 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 25
   // have a SIMD to themselves: two blocks are asked for at once and the page
   // ids of the next two before that, so a wavefront makes half as many trips to
   // memory (7B shape, contexts of 4,096: +1.5 % tokens/s at batch 8, +6.5 % at 64).
-  if (kb_begin < kb_end) {
-    if (PAIRS) {
-      int kb = kb_begin;
-      int pga[2], pgb[2], pga_next[2], pgb_next[2];
-      const int last = kb_end - 1;
-      load_pages(kb, pga_next);
-      load_pages(kb < last ? kb + 1 : last, pgb_next);
-      for (; kb + 1 < kb_end; kb += 2) {
-        bf16x8 kfa[2][KK], vfa[DD], kfb[2][KK], vfb[DD];
-        pga[0] = pga_next[0], pga[1] = pga_next[1], pgb[0] = pgb_next[0], pgb[1] = pgb_next[1];
-        load_pages(kb + 2 < last ? kb + 2 : last, pga_next);
-        load_pages(kb + 3 < last ? kb + 3 : last, pgb_next);
-        load_block(kb, pga, kfa, vfa);
-        load_block(kb + 1, pgb, kfb, vfb);
-        C.block(kb, kfa, vfa, gq);
-        C.block(kb + 1, kfb, vfb, gq);
-      }
-      if (kb < kb_end) {
-        bf16x8 kf[2][KK], vf[DD];
-        load_block(kb, pga_next, kf, vf);
-        C.block(kb, kf, vf, gq);
-      }
-    } else {
+  if (kb_begin >= kb_end) return;
+  if (PAIRS) {
+    int kb = kb_begin;
+    int pga[2], pgb[2], pga_next[2], pgb_next[2];
+    const int last = kb_end - 1;
+    load_pages(kb, pga_next);
+    load_pages(kb < last ? kb + 1 : last, pgb_next);
+    for (; kb + 1 < kb_end; kb += 2) {
+      bf16x8 kfa[2][KK], vfa[DD], kfb[2][KK], vfb[DD];
+      pga[0] = pga_next[0], pga[1] = pga_next[1], pgb[0] = pgb_next[0], pgb[1] = pgb_next[1];
+      load_pages(kb + 2 < last ? kb + 2 : last, pga_next);
+      load_pages(kb + 3 < last ? kb + 3 : last, pgb_next);
+      load_block(kb, pga, kfa, vfa);
+      load_block(kb + 1, pgb, kfb, vfb);
+      C.block(kb, kfa, vfa, gq);
+      C.block(kb + 1, kfb, vfb, gq);
+    }
+    if (kb < kb_end) {
+      bf16x8 kf[2][KK], vf[DD];
+      load_block(kb, pga_next, kf, vf);
+      C.block(kb, kf, vf, gq);
+    }
+  } else {
     int pg[2], pg_next[2];
     const int last = kb_end - 1;
     load_pages(kb_begin, pg_next);
@@ -467,9 +446,99 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 25
       load_block(kb, pg, kf, vf);
       C.block(kb, kf, vf, gq);
     }
+  }
+}
+
+// One wavefront per workgroup; operands straight from the pages.  Used for
+// decode tokens (SPLIT: the wavefront takes one share of the key blocks) and
+// for prompt portions whose launch does not saturate L2.
+template <int NB, bool SPLIT, bool FOLD, bool PAIRS = false>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 256 ? 2 : 1))) void attention_mfma_kernel(const AttnParams P) {
+  const int lane = threadIdx.x, n = lane & 15, gq = lane >> 4;
+  const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
+  const int g = P.nh / P.nkv;
+  const int q0 = P.cu_q[seq];
+  const int qlen = P.cu_q[seq + 1] - q0;
+  const int ncols = qlen * g;
+  const int ntiles = (ncols + 16 * NB - 1) / (16 * NB);
+  const int tile_rev = blockIdx.x / P.nsplit, split = blockIdx.x % P.nsplit;
+  if (tile_rev >= ntiles) return;
+  const int tile = ntiles - 1 - tile_rev;          // long (late) tiles first
+  const int pos0 = P.positions[q0];
+  const int* table = P.block_tables + (size_t)seq * P.max_pages;
+
+  Columns<NB, FOLD> C;
+  C.init(P, q0, ncols, tile * 16 * NB, pos0, kvh, g, n, gq);
+  int kb_begin = C.kb_begin, kb_end = C.kb_end;
+  if (SPLIT) {
+    const int nblk = kb_end - kb_begin;
+    const int first = kb_begin + (int)((long long)nblk * split / P.nsplit);
+    kb_end = kb_begin + (int)((long long)nblk * (split + 1) / P.nsplit);
+    kb_begin = first;
+  }
+  walk_blocks<NB, FOLD, PAIRS>(C, P, table, kvh, n, gq, kb_begin, kb_end);
+  C.template store<SPLIT>(P, q0, split, gq);
+}
+
+// Decode tokens, a workgroup of GROUP_WAVES wavefronts per (sequence, kv head): the wavefronts cut the
+// key blocks among themselves, each walks its own as above, and they merge their results in LDS:
+// out = sum_w 2^(m_w - m) o_w / sum_w 2^(m_w - m) l_w, m the largest reference point.  The workgroup
+// writes the rows of the result itself and no second kernel follows (a kernel that only waits for
+// this one's partial results costs 4-5 us a layer whatever it does).  How a request's keys are cut
+// depends on its own context and the workgroup's size only, not on what else is in the batch.
+constexpr int GROUP_WAVES = 8;
+// column tiles whose partial results fit LDS: two (up to 32 query heads a kv head) for head sizes up to 128, else one
+constexpr int GROUP_MAX_NB = GROUP_WAVES * 32 * (D + 4) * 4 <= 150 * 1024 ? 2 : 1;
+template <int NB, bool FOLD>
+__global__ __launch_bounds__(64 * GROUP_WAVES) __attribute__((amdgpu_waves_per_eu(NB * D <= 256 ? 2 : 1)))
+void attention_mfma_group_kernel(const AttnParams P) {
+  constexpr int COLS = 16 * NB, PITCH = D + 4;       // (rows of D + 4 floats: the 16 lanes of a column tile write to different banks)
+  __shared__ __attribute__((aligned(16))) float so[GROUP_WAVES][COLS][PITCH];
+  __shared__ float sm[GROUP_WAVES][COLS], sl[GROUP_WAVES][COLS];
+  const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63, n = lane & 15, gq = lane >> 4;
+  const int seq = P.seq_begin + blockIdx.y, kvh = blockIdx.x;
+  const int g = P.nh / P.nkv;                        // (one token a sequence: its g columns are one tile)
+  const int q0 = P.cu_q[seq];
+  const int pos0 = P.positions[q0];
+  const int* table = P.block_tables + (size_t)seq * P.max_pages;
+
+  Columns<NB, FOLD> C;
+  C.init(P, q0, g, 0, pos0, kvh, g, n, gq);
+  const int nblk = C.kb_end - C.kb_begin;
+  // (two blocks asked for at once where the registers hold them: one column tile)
+  walk_blocks<NB, FOLD, NB == 1>(C, P, table, kvh, n, gq, C.kb_begin + nblk * wave / GROUP_WAVES,
+                              C.kb_begin + nblk * (wave + 1) / GROUP_WAVES);
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if (C.pos_c[b] < 0) continue;                    // padding columns
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd) *(f32x4*)&so[wave][16 * b + n][16 * dd + 4 * gq] = C.o[b][dd];
+    if (gq == 0) {
+      sm[wave][16 * b + n] = C.reference(b);
+      sl[wave][16 * b + n] = C.l_acc[b][0];
     }
   }
-  C.template store<SPLIT>(P, q0, split, gq);
+  __syncthreads();
+  for (int idx = t; idx < g * (D / 4); idx += 64 * GROUP_WAVES) {
+    const int col = idx / (D / 4), d = 4 * (idx % (D / 4));
+    float top = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < GROUP_WAVES; ++w) top = fmaxf(top, sm[w][col]);
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+#pragma unroll
+    for (int w = 0; w < GROUP_WAVES; ++w) {
+      const float m = sm[w][col];
+      const float wt = m == -INFINITY ? 0.f : fast_exp2(m - top);
+      num += wt * *(const f32x4*)&so[w][col][d];                      // (a wavefront without keys wrote zeros)
+      den += wt * sl[w][col];
+    }
+    const float inv = 1.f / den;
+    bf16x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = (__bf16)(num[j] * inv);
+    *(bf16x4*)(P.out + out_index(P.out_rows, P.nh, (size_t)q0, (kvh * g + col) * D + d)) = r;
+  }
 }
 
 // Prompt portions: four wavefronts, one per SIMD, take 32 columns each and
@@ -782,12 +851,15 @@ extern "C" int sl_attention_mfma_max_splits() { return 64 * COMBINE_PER_LANE; }
 extern "C" int sl_attention_mfma_head_dim() { return D; }
 // whether this head size has the prompt kernel that shares keys through LDS (its buffers fit)
 extern "C" int sl_attention_mfma_shares_keys() { return SHARED_FITS ? 1 : 0; }
+// the most query heads per kv head that the single-token workgroups which merge in LDS take
+extern "C" int sl_attention_mfma_group_heads() { return 16 * GROUP_MAX_NB; }
 // whether the workgroups that share keys through LDS are laid out by chiplet for this many kv heads (see Place)
 extern "C" int sl_attention_mfma_by_chiplet(int nkv) { return nkv > 0 && (nkv < 8 ? 8 % nkv == 0 : nkv % 8 == 0) ? 1 : 0; }
 
 // One launch over sequences [seq_begin, seq_begin + num_seqs), all with at
 // most max_q_len tokens.  nsplit > 1 needs part_o / part_ml for the rows
 // [part_row0, part_row0 + part_rows) these sequences own (one token each).
+// group (single tokens, nsplit 1): the workgroups of eight wavefronts that merge in LDS.
 // Prompt portions go to the workgroups that share keys through LDS once the
 // launch would have shared_min_waves wavefronts of 32 columns or more;
 // pair_tiles: see the kernel; narrow_below: with fewer workgroups of 128
@@ -797,7 +869,7 @@ extern "C" const char* sl_attention_mfma(
     int max_pages, const int* cu_q, const int* positions, int seq_begin, int num_seqs,
     int max_q_len, int nh, int nkv, int head_dim, int page, float scale, int window, int nsplit,
     int shared_min_waves, int pair_tiles, void* out, float* part_o, float* part_ml, int part_row0, int part_rows,
-    int narrow_below, int out_rows, hipStream_t stream) {
+    int narrow_below, int out_rows, int group, hipStream_t stream) {
   SL_CHECK(head_dim == D, "attention_mfma: built for another head size");
   SL_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: heads must be a multiple of kv heads");
   SL_CHECK(page == 16 || page == 32 || page == 64, "attention_mfma: page size must be 16, 32 or 64");
@@ -816,6 +888,20 @@ extern "C" const char* sl_attention_mfma(
   const long long cols = (long long)max_q_len * g;
   // scale * log2(e) == 1: the caller's q is already in units of log 2 (see Columns)
   const bool fold = fabsf(scale * 1.4426950408889634f - 1.f) < 1e-6f;
+  if (group) {
+    // single tokens, a workgroup per (sequence, kv head) whose wavefronts merge in LDS
+    SL_CHECK(max_q_len == 1 && nsplit == 1, "attention_mfma: the workgroups that merge in LDS take single tokens, unsplit");
+    SL_CHECK(g <= 16 * GROUP_MAX_NB, "attention_mfma: too many query heads per kv head for the workgroups that merge in LDS");
+    const dim3 grid(nkv, num_seqs);
+    if (g <= 16) {
+      if (fold) attention_mfma_group_kernel<1, true><<<grid, 64 * GROUP_WAVES, 0, stream>>>(P);
+      else attention_mfma_group_kernel<1, false><<<grid, 64 * GROUP_WAVES, 0, stream>>>(P);
+    } else {
+      if (fold) attention_mfma_group_kernel<GROUP_MAX_NB, true><<<grid, 64 * GROUP_WAVES, 0, stream>>>(P);
+      else attention_mfma_group_kernel<GROUP_MAX_NB, false><<<grid, 64 * GROUP_WAVES, 0, stream>>>(P);
+    }
+    return sl_launch_status();
+  }
   if (nsplit > 1 && max_q_len == 1) {
     SL_CHECK(part_o != nullptr && part_ml != nullptr && part_rows == num_seqs,
              "attention_mfma: a split launch needs partial buffers for its rows");
@@ -846,7 +932,8 @@ extern "C" const char* sl_attention_mfma(
   // 512: 46 against 99 us; 512 tokens after 7,680: 108 against 278 us.)
   const long long tiles = (cols + 31) / 32;
   SL_CHECK(tiles <= 1 << 30, "attention_mfma: too many column tiles");
-  const bool shared = SHARED_FITS && tiles * nkv * num_seqs >= shared_min_waves;
+  // (single tokens of at most 16 heads a kv head, unsplit: one wavefront each, as before)
+  const bool shared = SHARED_FITS && (max_q_len > 1 || cols > 16) && tiles * nkv * num_seqs >= shared_min_waves;
   if (nsplit > 1) {
     SL_CHECK(shared && !pair_tiles, "attention_mfma: prompt portions are split only as unpaired tiles through LDS");
     SL_CHECK(nsplit <= 64 * COMBINE_PER_LANE && part_o != nullptr && part_ml != nullptr && part_rows > 0,

@@ -360,18 +360,31 @@ class AttentionOps:
                 part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
                        0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
-                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS if triangle else 0, 0)
+                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS if triangle else 0, 0, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
                 blocks = min(blocks, -(-int(window) // 32) + 1)
-            # (a few requests with long contexts: up to 256 shares, so that the launch still has TARGET_WAVES
-            # wavefronts; 7B shape, one request at 32,000 tokens: 64 shares leave one wavefront per CU)
             most = int(self._lib[lib].sl_attention_mfma_max_splits())
-            nsplit = self._decode_shares(n_dec * nkv, min(most, blocks // 2))
+            # With a (request, kv head) pair or more for every CU, a workgroup of eight wavefronts takes a pair:
+            # its wavefronts cut the keys among themselves and merge in LDS, no partial results in memory and
+            # no second kernel.  With fewer pairs that would leave a pair's keys to the one CU that runs its
+            # workgroup, and a CU pulls 50 GB/s whatever is in flight (7B shape, contexts of 4,096, 8 requests:
+            # 61 us against 16 us): then a wavefront of a workgroup of its own takes a share, shares enough for
+            # TARGET_WAVES wavefronts spread over all CUs, and the combine kernel merges them (a few requests
+            # with long contexts: up to 256 shares; one request at 32,000 tokens: 64 shares leave one wavefront
+            # per CU).  Short contexts merge in the workgroup from half as many pairs on.
+            # Workgroups of one pair each go round the CUs in whole rounds, so the pairs must fill their last
+            # round too (96 requests of 4 kv heads on 256 CUs, one round and a half: 8.45 ms a step against 8.09).
+            pairs, cus = n_dec * nkv, self._num_cus
+            even = pairs <= cus or pairs >= self.GROUP_ATTENTION_ROUNDS_FILL * -(-pairs // cus) * cus
+            need = self.GROUP_ATTENTION_FILL * cus
+            group = (nh // nkv <= int(self._lib[lib].sl_attention_mfma_group_heads()) and even
+                     and (pairs >= need or (2 * pairs >= need and blocks <= self.GROUP_ATTENTION_SHORT_BLOCKS)))
+            nsplit = 1 if group else self._decode_shares(n_dec * nkv, min(most, blocks // 2))
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, 0, _p(out),
-                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0, 0, int(out_rows))
+                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0, 0, int(out_rows), int(group))

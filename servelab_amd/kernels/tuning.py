@@ -88,6 +88,15 @@ class Tuning:
     general_attention_waves: int = 4096
     # the same for the matrix-core kernel (384, 768 and 1,024 measured within noise or slower)
     target_waves: int = 512
+    # single tokens: with this many (request, kv head) pairs per CU and more, a workgroup of eight wavefronts
+    # takes a pair's keys and merges in LDS; below, a wavefront takes a share and a second kernel merges
+    # (7B shape, a layer: contexts of 4,096, 64 / 128 requests: 89.7 / 177 against 91.1 / 209 us, 32 requests
+    # 76 against 50; contexts of 640, 32 / 64 / 128 requests: 13.8 / 16.9 / 32.2 against 15.1 / 20.0 / 35.8 us,
+    # 16 requests 12.7 against 9.8); contexts of at most short_blocks key blocks from half as many pairs on
+    group_attention_fill: float = 1.0
+    group_attention_short_blocks: int = 32
+    # ... and only if the pairs fill this share of the slots of their rounds over the CUs
+    group_attention_rounds_fill: float = 0.9
     # prompt launches share keys through LDS from this many 32-column wavefronts and this context
     # on (7B shape, laid out by chiplet, a workgroup per tile: as fast or faster than a wavefront
     # per 32 columns straight from the pages at every size measured, from 8 tokens to 32 k)

@@ -920,6 +920,50 @@ def test_decode_attention_shares_out_the_keys(both, nh, nkv, D, page, window, un
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+@pytest.mark.parametrize("nh,nkv,D,page", [(28, 4, 128, 16), (8, 8, 32, 32), (40, 2, 64, 16), (32, 1, 96, 64), (6, 2, 256, 16)])
+@pytest.mark.parametrize("window", [None, 50])
+@pytest.mark.parametrize("units", UNITS)
+def test_decode_attention_merged_inside_the_workgroup(nh, nkv, D, page, window, units):
+    """Single-token rows with a workgroup of eight wavefronts per (request, kv head) that cut the keys
+    among themselves and merge in LDS (forced here at a batch far smaller than the one that takes it
+    by itself): contexts of 1 token (seven wavefronts without a key), of fewer blocks than wavefronts,
+    of hundreds and of thousands of keys; 1, 7, 20 and 32 query heads a kv head (one and two column
+    tiles); and that the table takes this form by itself once the batch fills the chip with it."""
+    from servelab_amd.kernels import HipOps, Tuning
+    dt = torch.bfloat16
+    ops, emu = HipOps(dt, "cuda:0", tuning=Tuning(group_attention_fill=0.0)), EmulatedOps(dt)
+    seen = []
+    call = ops._call
+
+    def spy(stem, name, *args):
+        if name.startswith("sl_attention_mfma@"):
+            seen.append((args[17], args[-1]))                    # shares, merged inside the workgroup
+        return call(stem, name, *args)
+    ops._call = spy
+    seqs = [(1, 1), (5, 1), (64, 1), (65, 1), (333, 1), (700, 1), (129, 1), (4100, 1)]
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=9)
+    qkv, scale = in_units(units, qkv, nh, D, 1.0 / math.sqrt(D))
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
+    assert len(seen) == 1 and seen[0] == (1, 1)
+    ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                              types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                       for k, v in vars(batch).items()}),
+                              scale, window)
+    assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+    # by itself: with a pair for every CU (here: a table told that it has 24 CUs), or half as many of short contexts
+    plain = HipOps(dt, "cuda:0")
+    plain._num_cus = 24
+    for n_seqs, ctx, merged in ((-(-24 // nkv), 4000, True), (max(1, 23 // nkv), 4000, False), (-(-12 // nkv), 900, True),
+                                (-(-12 // nkv), 1100, False)) if window is None else ():      # (a window makes every context short)
+        seen.clear()
+        plain._call = lambda stem, name, *args: (seen.append((args[17], args[-1])) if name.startswith("sl_attention_mfma@") else None,
+                                                 HipOps._call(plain, stem, name, *args))[1]
+        case = make_attention_case(dt, nh, nkv, D, page, [(ctx - 3 * i, 1) for i in range(n_seqs)], seed=3)
+        q2, s2 = in_units(units, case[0], nh, D, 1.0 / math.sqrt(D))
+        plain.paged_attention(q2, nh, nkv, D, case[1], case[2], page, case[3], case[4], s2, window)
+        assert len(seen) == 1 and bool(seen[0][1]) == bool(merged) and (seen[0][0] == 1 or not merged), (n_seqs, ctx, seen)
+
+
 @pytest.mark.parametrize("nh,nkv,D,page", [(28, 4, 128, 16), (8, 1, 64, 32)])
 @pytest.mark.parametrize("contexts", [(9000,), (9000, 5000)])
 def test_decode_attention_with_more_shares_than_lanes(nh, nkv, D, page, contexts):
