@@ -25,16 +25,21 @@
 // K pages are key-major ([page, nkv, page_size, D]): its A operand is one
 // 16-byte load as well.
 //
-// Three launches share that inner block (struct Columns):
-//   - decode (one token per sequence, g columns): the context is split over
-//     several wavefronts; each writes an unnormalised partial (o, reference,
-//     sum) and attention_combine_kernel merges them;
+// Four launches share that inner block (struct Columns):
+//   - decode (one token per sequence, g columns), few sequences: the context
+//     is split over several wavefronts, each a workgroup of its own; each
+//     writes an unnormalised partial (o, reference, sum) and
+//     attention_combine_kernel merges them;
+//   - decode, a (sequence, kv head) pair or more for every CU: a workgroup of
+//     eight wavefronts per pair that split the context and merge in LDS
+//     (attention_mfma_group_kernel);
+//   - prompt portions, four wavefronts per workgroup that share each block of
+//     keys and values through LDS (attention_mfma_shared_kernel), the launch
+//     laid out by chiplet; tiles of a portion deep in its context cut into
+//     shares of their keys, merged by attention_combine_kernel;
 //   - prompt portions, one wavefront per 32 columns, operands straight from
 //     the pages, two wavefronts per SIMD so that one computes while the other
-//     waits for its loads;
-//   - prompt portions, four wavefronts per workgroup that share each block of
-//     keys and values through LDS (attention_mfma_shared_kernel), for launches
-//     large enough that L2 traffic, not latency, is the limit.
+//     waits for its loads: for head sizes whose blocks do not fit the LDS ring.
 // The softmax keeps a reference point per column instead of the exact running
 // maximum (see LAZY) and folds the scale into the exponent's multiply-add.
 #include "common.h"
@@ -373,9 +378,6 @@ struct Columns {
   }
 };
 
-// One wavefront per workgroup; operands straight from the pages.  Used for
-// decode tokens (SPLIT: the wavefront takes one share of the key blocks) and
-// for prompt portions whose launch does not saturate L2.
 // The key blocks [kb_begin, kb_end) of one wavefront's columns, operands straight from the pages.
 template <int NB, bool FOLD, bool PAIRS>
 __device__ __forceinline__ void walk_blocks(Columns<NB, FOLD>& C, const AttnParams& P, const int* table, int kvh,
