@@ -847,6 +847,39 @@ def test_portions_deep_in_a_context_take_shares_of_their_keys_by_default():
         assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_attention_over_random_batches(seed):
+    """Seeded random batches through the launches the table chooses by itself: whole prompts, portions
+    deep in their contexts (two tokens to hundreds), single tokens after them; 1 to 16 kv heads (laid
+    out by chiplet or not), with and without a window; on a table that believes in 8 CUs, so that a few
+    single tokens already merge inside their workgroups.  Against the plain computation."""
+    import random
+    from servelab_amd.kernels import HipOps
+    rnd = random.Random(seed)
+    dt = torch.bfloat16
+    nkv = rnd.choice([1, 2, 3, 4, 8, 16])
+    g = rnd.choice([1, 2, 7, 8, 20])
+    D, page = rnd.choice([(32, 16), (64, 32), (128, 16), (96, 64)])
+    nh = nkv * g
+    window = rnd.choice([None, None, 40, 300])
+    prompts = []
+    for _ in range(rnd.randint(0, 4)):
+        q = rnd.choice([2, 3, 17, 64, 130, 300])
+        prompts.append((q + rnd.choice([0, 0, 5, 200, 900]), q))
+    singles = [(rnd.randint(1, 1500), 1) for _ in range(rnd.choice([0, 1, 3, 9]))]
+    seqs = prompts + singles or [(77, 77)]
+    ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+    ops._num_cus = 8
+    qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=seed)
+    qkv, scale = in_units(UNITS[seed % 2], qkv, nh, D, 1.0 / math.sqrt(D))
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
+    ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                              types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                       for k, v in vars(batch).items()}),
+                              scale, window)
+    assert rel_err(got.cpu(), ref) < ATTN_TOL[dt], (nh, nkv, D, page, window, seqs)
+
+
 def test_decode_shares_fill_whole_rounds_over_the_cus():
     """The number of shares of a request's keys at the batch sizes it was measured at (4 kv heads, 256 CUs,
     contexts of 4,096: 64 shares at most): never slightly more wavefronts than a whole number per CU."""
