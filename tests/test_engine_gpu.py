@@ -98,6 +98,40 @@ def test_long_decoding_across_graph_captures(tmp_path, which, page, dtype, monke
     assert worst < bar, f"max abs err {worst} at {where}, bar {bar}"
 
 
+@pytest.mark.parametrize("page,other", [(32, {}), (16, dict(head_dim=64, num_key_value_heads=2, use_sliding_window=False))])
+def test_long_decoding_with_the_keys_merged_inside_the_workgroup(tmp_path, page, other, monkeypatch):
+    """The decode attention that a large batch takes by itself (a workgroup of eight wavefronts per
+    request and kv head, merged in LDS), asked for at four requests: a prompt each, then 150 tokens
+    one by one through the captured graphs, contexts from 3 to 190 keys (fewer key blocks than
+    wavefronts for most of the run); the configuration whose head size the matrix-core kernels take, with
+    its window in one layer, and the same with two kv heads of 64 and no window."""
+    from servelab_amd.kernels import HipOps, Tuning
+    monkeypatch.setattr(ModelRunner, "GRAPH_MIN_CONTEXT", 64)
+    folder = make_folder(tmp_path, "B", seed=29, **other)
+    vocab = TINY["B"]["vocab_size"]
+    rng = random.Random(5)
+    starts = {"p": 40, "q": 3, "r": 17, "s": 33}
+    requests = {r: [rng.randrange(vocab) for _ in range(n + 150)] for r, n in starts.items()}
+    reference = plain_logits(folder, requests)
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": requests[r][:n], "want": [n - 1]} for r, n in starts.items()],
+              "end": []}]
+    for i in range(150):
+        steps.append({"step": i + 1, "entries": [{"id": r, "tokens": [requests[r][n + i]], "want": [0]}
+                                                 for r, n in starts.items()],
+                      "end": list(starts) if i == 149 else []})
+    ops = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(group_attention_fill=0.0))
+    merged = []
+    call = ops._call
+    ops._call = lambda stem, name, *args: (merged.append(args[-1]) if name.startswith("sl_attention_mfma@") and args[10] == 1
+                                           else None, call(stem, name, *args))[1]
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, "bfloat16", rs.max_tokens_needed(steps), block_size=page, ops=ops)
+    assert merged and all(merged)                    # (every launch over single tokens took that form)
+    worst, where = compare(out, steps, reference, vocab)
+    bar = bfloat16_bar(folder, requests, reference, vocab, ("merged", page))
+    assert worst < bar, f"max abs err {worst} at {where}, bar {bar}"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replay_equals_eager(tmp_path, dtype):
     """The same decode steps with and without graphs; the graph is replayed
