@@ -42,8 +42,18 @@ QWEN25_32B = dict(QWEN25_7B, num_hidden_layers=64, hidden_size=5120, num_attenti
                   num_key_value_heads=8, intermediate_size=27648)
 QWEN25_72B = dict(QWEN25_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
                   num_key_value_heads=8, intermediate_size=29568)
+QWEN25_05B = dict(QWEN25_7B, num_hidden_layers=24, hidden_size=896, num_attention_heads=14, num_key_value_heads=2,
+                  head_dim=64, intermediate_size=4864, vocab_size=151936, tie_word_embeddings=True)
+QWEN25_15B = dict(QWEN25_7B, num_hidden_layers=28, hidden_size=1536, num_attention_heads=12, num_key_value_heads=2,
+                  intermediate_size=8960, vocab_size=151936, tie_word_embeddings=True)
+QWEN25_3B = dict(QWEN25_7B, num_hidden_layers=36, hidden_size=2048, num_attention_heads=16, num_key_value_heads=2,
+                 intermediate_size=11008, vocab_size=151936, tie_word_embeddings=True)
+QWEN25_14B = dict(QWEN25_7B, num_hidden_layers=48, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                  intermediate_size=13824)
 SHAPES = {"7b": ("Qwen2.5-7B shape", QWEN25_7B), "32b": ("Qwen2.5-32B shape", QWEN25_32B),
-          "72b": ("Qwen2.5-72B shape", QWEN25_72B)}
+          "72b": ("Qwen2.5-72B shape", QWEN25_72B), "0.5b": ("Qwen2.5-0.5B shape", QWEN25_05B),
+          "1.5b": ("Qwen2.5-1.5B shape", QWEN25_15B), "3b": ("Qwen2.5-3B shape", QWEN25_3B),
+          "14b": ("Qwen2.5-14B shape", QWEN25_14B)}
 
 
 def build(args):

@@ -299,6 +299,29 @@ class AttentionOps:
                 best, best_score = shares, score
         return best
 
+    def _decode_many(self, pairs, blocks, D, merged_fits, most):
+        """(merged in the workgroup, shares) for single-token rows of more (request, kv head) pairs than
+        CUs, by the estimate of the launch's time that ``Tuning.many_*`` describes.  Wavefronts of a share
+        each all have to be on the chip at once (eight a CU), or the launch runs in two waves of them."""
+        cus = self._num_cus
+        stream = pairs * blocks * 32 * D * 4 / (self.MANY_STREAM_GBS_PER_CU * 1e3 * cus)      # us for K and V
+
+        def rounds(units):                           # as if every CU had as many units as the fullest
+            return -(-units // cus) * cus / units
+
+        def fullest(waves):
+            return rounds(waves) if waves <= self.MANY_CROWDED_WAVES * cus else 1 + self.MANY_CROWDED * (rounds(waves) - 1)
+
+        forms = []                                   # (estimate, merged, shares), fewest shares first
+        if merged_fits:
+            forms.append((stream * (1 + self.MANY_MERGED_ROUNDS * (rounds(pairs) - 1)) * self.MANY_MERGED_BASE, True, 1))
+        for k in range(1, max(1, min(most, 8 * cus // pairs)) + 1):
+            t = max(-(-blocks // (2 * k)) * self.MANY_TRIP_US, stream * fullest(pairs * k)) + self.MANY_SHARE_US * k
+            forms.append((t + (self.MANY_COMBINE_US if k > 1 else 0.0), False, k))
+        lowest = min(t for t, _, _ in forms)
+        _, merged, shares = next(f for f in forms if f[0] <= self.MANY_FEWER_WITHIN * lowest)
+        return merged, shares
+
     def _pair_prompt_tiles(self, tiles, prompts_and_heads) -> bool:
         """Whether the workgroups of a whole prompt's attention take a late tile of the causal triangle and
         its early mirror (equal work for all, half as many workgroups) or a tile each, long ones first;
@@ -366,22 +389,23 @@ class AttentionOps:
             if window:
                 blocks = min(blocks, -(-int(window) // 32) + 1)
             most = int(self._lib[lib].sl_attention_mfma_max_splits())
-            # With a (request, kv head) pair or more for every CU, a workgroup of eight wavefronts takes a pair:
-            # its wavefronts cut the keys among themselves and merge in LDS, no partial results in memory and
+            # With a (request, kv head) pair for every CU, a workgroup of eight wavefronts takes a pair: its
+            # wavefronts cut the keys among themselves and merge in LDS, no partial results in memory and
             # no second kernel.  With fewer pairs that would leave a pair's keys to the one CU that runs its
             # workgroup, and a CU pulls 50 GB/s whatever is in flight (7B shape, contexts of 4,096, 8 requests:
             # 61 us against 16 us): then a wavefront of a workgroup of its own takes a share, shares enough for
             # TARGET_WAVES wavefronts spread over all CUs, and the combine kernel merges them (a few requests
             # with long contexts: up to 256 shares; one request at 32,000 tokens: 64 shares leave one wavefront
-            # per CU).  Short contexts merge in the workgroup from half as many pairs on.
-            # Workgroups of one pair each go round the CUs in whole rounds, so the pairs must fill their last
-            # round too (96 requests of 4 kv heads on 256 CUs, one round and a half: 8.45 ms a step against 8.09).
+            # per CU).  Short contexts merge in the workgroup from half as many pairs on.  More pairs than
+            # CUs: see _decode_many.
             pairs, cus = n_dec * nkv, self._num_cus
-            even = pairs <= cus or pairs >= self.GROUP_ATTENTION_ROUNDS_FILL * -(-pairs // cus) * cus
-            need = self.GROUP_ATTENTION_FILL * cus
-            group = (nh // nkv <= int(self._lib[lib].sl_attention_mfma_group_heads()) and even
-                     and (pairs >= need or (2 * pairs >= need and blocks <= self.GROUP_ATTENTION_SHORT_BLOCKS)))
-            nsplit = 1 if group else self._decode_shares(n_dec * nkv, min(most, blocks // 2))
+            fits = nh // nkv <= int(self._lib[lib].sl_attention_mfma_group_heads())
+            if pairs <= cus:
+                need = self.GROUP_ATTENTION_FILL * cus
+                group = fits and (pairs >= need or (2 * pairs >= need and blocks <= self.GROUP_ATTENTION_SHORT_BLOCKS))
+                nsplit = 1 if group else self._decode_shares(pairs, min(most, blocks // 2))
+            else:
+                group, nsplit = self._decode_many(pairs, blocks, D, fits, min(most, blocks // 2))
             part_o = part_ml = None
             if nsplit > 1:
                 part_o = self._new((n_dec, nh, nsplit, D), torch.float32)

@@ -88,15 +88,36 @@ class Tuning:
     general_attention_waves: int = 4096
     # the same for the matrix-core kernel (384, 768 and 1,024 measured within noise or slower)
     target_waves: int = 512
-    # single tokens: with this many (request, kv head) pairs per CU and more, a workgroup of eight wavefronts
-    # takes a pair's keys and merges in LDS; below, a wavefront takes a share and a second kernel merges
+    # single tokens, no more (request, kv head) pairs than CUs: with this many pairs per CU, a workgroup of eight
+    # wavefronts takes a pair's keys and merges in LDS; below, a wavefront takes a share and a second kernel merges
     # (7B shape, a layer: contexts of 4,096, 64 / 128 requests: 89.7 / 177 against 91.1 / 209 us, 32 requests
     # 76 against 50; contexts of 640, 32 / 64 / 128 requests: 13.8 / 16.9 / 32.2 against 15.1 / 20.0 / 35.8 us,
     # 16 requests 12.7 against 9.8); contexts of at most short_blocks key blocks from half as many pairs on
     group_attention_fill: float = 1.0
     group_attention_short_blocks: int = 32
-    # ... and only if the pairs fill this share of the slots of their rounds over the CUs
-    group_attention_rounds_fill: float = 0.9
+    # With more pairs than CUs the form is taken by an estimate of the launch's time, whose constants
+    # are fitted to 63 launches of 288 to 1,024 pairs over contexts of 640 to 4,096 (3.5 % rms; the form
+    # taken is 0.8 % slower than the best measured one on average, 6 % at worst).  The keys and values
+    # stream at many_stream_gbs_per_cu GB/s times the CUs (6.3 TB/s on 256).  Wavefronts that take a
+    # share each are spread over the CUs, and the launch takes as long as if every CU had as many as
+    # the fullest (a factor of ceil(w / CUs) CUs / w; with more than many_crowded_waves a CU only
+    # many_crowded of what it exceeds 1 by), no less than a wavefront's trips to memory, many_trip_us
+    # for two key blocks, plus many_share_us per share and many_combine_us for the second kernel.
+    # The workgroups that merge in LDS pay many_merged_rounds of that factor (those of the last round
+    # have the chip to themselves) and many_merged_base overall.  Of estimates within many_fewer_within
+    # of the lowest, the form with the fewest shares is taken.  Contexts of 4,096, us a layer for 72 / 104
+    # / 112 / 144 / 160 requests of 4 kv heads: 110 / 153 / 160 / 207 / 228 (in 4 / 3 / 4 / 3 / 2 shares),
+    # against 126 / 206 / 208 / 256 / 264 when more pairs than CUs meant two shares up to 384 pairs,
+    # then one, or merged where the rounds were nearly full.
+    many_stream_gbs_per_cu: float = 24.6
+    many_trip_us: float = 2.95
+    many_share_us: float = 0.84
+    many_combine_us: float = 2.05
+    many_crowded_waves: int = 3
+    many_crowded: float = 0.46
+    many_merged_rounds: float = 0.57
+    many_merged_base: float = 1.048
+    many_fewer_within: float = 1.02
     # prompt launches share keys through LDS from this many 32-column wavefronts and this context
     # on (7B shape, laid out by chiplet, a workgroup per tile: as fast or faster than a wavefront
     # per 32 columns straight from the pages at every size measured, from 8 tokens to 32 k)

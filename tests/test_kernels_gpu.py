@@ -997,6 +997,44 @@ def test_decode_attention_merged_inside_the_workgroup(nh, nkv, D, page, window, 
         assert len(seen) == 1 and bool(seen[0][1]) == bool(merged) and (seen[0][0] == 1 or not merged), (n_seqs, ctx, seen)
 
 
+def test_single_tokens_of_more_pairs_than_cus():
+    """More (request, kv head) pairs than CUs: the form is taken by the estimate of the launch's time
+    (on a table told that it has 256 CUs: shares that fill whole rounds of the CUs between one pair a
+    CU and two, merged in the workgroup where two rounds are nearly full and the context is short, one
+    share once there are four wavefronts for every CU), and every form gives the plain result
+    (a table told that it has 8 CUs; 4, 5 and 40 requests of 4 kv heads: merged, two shares, one)."""
+    from servelab_amd.kernels import HipOps
+    dt = torch.bfloat16
+    ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+    ops._num_cus = 256
+    plan = lambda pairs, blocks, fits=True: ops._decode_many(pairs, blocks, 128, fits, min(256, blocks // 2))
+    assert [plan(p, 128) for p in (288, 384, 416, 576, 640, 1024, 4096)] == \
+        [(False, 4), (False, 2), (False, 3), (False, 3), (False, 2), (False, 1), (False, 1)]
+    assert plan(448, 32) == (True, 1) and plan(448, 32, fits=False) == (False, 2)
+    assert plan(300, 2) == (True, 1) and plan(300, 2, fits=False) == (False, 1)      # (no block to share out)
+    nh, nkv, D, page = 28, 4, 128, 16
+    ops._num_cus = 8
+    seen = []
+    call = ops._call
+    ops._call = lambda stem, name, *args: (seen.append((args[17], args[-1])) if name.startswith("sl_attention_mfma@") else None,
+                                           call(stem, name, *args))[1]
+    for n_seqs, ctx, form in ((4, 700, (1, 1)), (5, 3000, (2, 0)), (40, 700, (1, 0))):
+        seqs = [(ctx - 13 * i, 1) for i in range(n_seqs)]
+        qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=ctx)
+        qkv, scale = in_units(UNITS[1], qkv, nh, D, 1.0 / math.sqrt(D))
+        for shares in (None, 3):                     # the form it takes by itself, and three shares
+            if shares:
+                ops._decode_many = lambda *a: (False, shares)
+            seen.clear()
+            got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, None)
+            assert seen == [form if shares is None else (3, 0)], (n_seqs, ctx, seen)
+            ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
+                                      types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
+                                                               for k, v in vars(batch).items()}), scale, None)
+            assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
+        del ops._decode_many
+
+
 @pytest.mark.parametrize("nh,nkv,D,page", [(28, 4, 128, 16), (8, 1, 64, 32)])
 @pytest.mark.parametrize("contexts", [(9000,), (9000, 5000)])
 def test_decode_attention_with_more_shares_than_lanes(nh, nkv, D, page, contexts):
