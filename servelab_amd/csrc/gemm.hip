@@ -1563,15 +1563,29 @@ extern "C" const char* sl_gemm_mid(const void* x, const void* wt, const float* b
   if (ks == 1 && wide && num_cus > 0 && 2 * groups > num_cus)
     groups = num_cus * ((groups + num_cus - 1) / num_cus);
   const dim3 grid(groups, ks);
+  // blocks of 16 rows of x a wavefront multiplies each tile of W with: as many as the rows need (80
+  // rows in five, not in eight: the products of 65 and more rows are no longer bound by memory
+  // alone); the workgroups of eight wavefronts share out a chunk of x evenly for even counts only
+  const int mb = (M + 15) / 16;
+#define SL_MID(MB_, WAVES_) gemm_mid_kernel<MB_, 2, 4, WAVES_><<<grid, 64 * WAVES_, 0, stream>>>( \
+    xx, ww, bias, dst, M, N, K, out_f32, gated, ks)
   if (wide) {
-    if (M <= 32) gemm_mid_kernel<2, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
-    else if (M <= 64) gemm_mid_kernel<4, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
-    else gemm_mid_kernel<8, 2, 4, 8><<<grid, 512, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    if (mb <= 2) SL_MID(2, 8);
+    else if (mb <= 4) SL_MID(4, 8);
+    else if (mb <= 6) SL_MID(6, 8);
+    else SL_MID(8, 8);
   } else {
-    if (M <= 32) gemm_mid_kernel<2, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
-    else if (M <= 64) gemm_mid_kernel<4, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
-    else gemm_mid_kernel<8, 2, 4, 4><<<grid, 256, 0, stream>>>(xx, ww, bias, dst, M, N, K, out_f32, gated, ks);
+    switch (mb) {
+      case 1: case 2: SL_MID(2, 4); break;
+      case 3: SL_MID(3, 4); break;
+      case 4: SL_MID(4, 4); break;
+      case 5: SL_MID(5, 4); break;
+      case 6: SL_MID(6, 4); break;
+      case 7: SL_MID(7, 4); break;
+      default: SL_MID(8, 4); break;
+    }
   }
+#undef SL_MID
   const char* e = sl_launch_status();
   if (e || ks == 1 || y == nullptr) return e;
   const size_t total = (size_t)M * N;

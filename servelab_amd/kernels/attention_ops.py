@@ -319,8 +319,45 @@ class AttentionOps:
             t = max(-(-blocks // (2 * k)) * self.MANY_TRIP_US, stream * fullest(pairs * k)) + self.MANY_SHARE_US * k
             forms.append((t + (self.MANY_COMBINE_US if k > 1 else 0.0), False, k))
         lowest = min(t for t, _, _ in forms)
-        _, merged, shares = next(f for f in forms if f[0] <= self.MANY_FEWER_WITHIN * lowest)
-        return merged, shares
+        estimate, merged, shares = next(f for f in forms if f[0] <= self.MANY_FEWER_WITHIN * lowest)
+        return merged, shares, estimate
+
+    def _decode_launches(self, n_dec, nkv, blocks, D, merged_fits, most):
+        """The launches over the single-token rows of a step: (first sequence, sequences, merged in
+        the workgroup, shares) each.  With a (request, kv head) pair for every CU, a workgroup of
+        eight wavefronts takes a pair: its wavefronts cut the keys among themselves and merge in LDS,
+        no partial results in memory and no second kernel.  With fewer pairs that would leave a
+        pair's keys to the one CU that runs its workgroup, and a CU pulls 50 GB/s whatever is in
+        flight (7B shape, contexts of 4,096, 8 requests: 61 us against 16 us): then a wavefront of a
+        workgroup of its own takes a share, shares enough for TARGET_WAVES wavefronts spread over all
+        CUs, and the combine kernel merges them (a few requests with long contexts: up to 256 shares;
+        one request at 32,000 tokens: 64 shares leave one wavefront per CU).  Short contexts merge in
+        the workgroup from half as many pairs on.  More pairs than CUs: one launch in the form
+        ``_decode_many`` estimates to be the fastest, or two, the sequences that fill whole rounds of
+        the CUs merged in the workgroup and the others as a launch of few pairs, if the estimates say
+        that is faster (the first launch then runs at the rate of a stream, whatever the number of
+        sequences)."""
+        pairs, cus = n_dec * nkv, self._num_cus
+
+        def few(n):
+            need = self.GROUP_ATTENTION_FILL * cus
+            merged = merged_fits and (n * nkv >= need or (2 * n * nkv >= need and blocks <= self.GROUP_ATTENTION_SHORT_BLOCKS))
+            return merged, 1 if merged else self._decode_shares(n * nkv, min(most, blocks // 2))
+
+        if pairs <= cus:
+            return [(0, n_dec) + few(n_dec)]
+        merged, shares, estimate = self._decode_many(pairs, blocks, D, merged_fits, min(most, blocks // 2))
+        per_round = cus // nkv
+        rest = n_dec % per_round if cus % nkv == 0 else 0
+        if merged_fits and rest and self.MANY_SECOND_LAUNCH_US >= 0:
+            stream = lambda n: n * nkv * blocks * 32 * D * 4 / (self.MANY_STREAM_GBS_PER_CU * 1e3 * cus)
+            m2, k2 = few(rest)
+            each = 8 if m2 else k2                    # wavefronts a pair
+            waves = rest * nkv * each
+            second = max(-(-blocks // (2 * each)) * self.MANY_TRIP_US, stream(rest) * (-(-waves // cus) * cus / waves))
+            if stream(n_dec - rest) + second + self.MANY_SECOND_LAUNCH_US < estimate:
+                return [(0, n_dec - rest, True, 1), (n_dec - rest, rest, m2, k2)]
+        return [(0, n_dec, merged, shares)]
 
     def _pair_prompt_tiles(self, tiles, prompts_and_heads) -> bool:
         """Whether the workgroups of a whole prompt's attention take a late tile of the causal triangle and
@@ -389,26 +426,12 @@ class AttentionOps:
             if window:
                 blocks = min(blocks, -(-int(window) // 32) + 1)
             most = int(self._lib[lib].sl_attention_mfma_max_splits())
-            # With a (request, kv head) pair for every CU, a workgroup of eight wavefronts takes a pair: its
-            # wavefronts cut the keys among themselves and merge in LDS, no partial results in memory and
-            # no second kernel.  With fewer pairs that would leave a pair's keys to the one CU that runs its
-            # workgroup, and a CU pulls 50 GB/s whatever is in flight (7B shape, contexts of 4,096, 8 requests:
-            # 61 us against 16 us): then a wavefront of a workgroup of its own takes a share, shares enough for
-            # TARGET_WAVES wavefronts spread over all CUs, and the combine kernel merges them (a few requests
-            # with long contexts: up to 256 shares; one request at 32,000 tokens: 64 shares leave one wavefront
-            # per CU).  Short contexts merge in the workgroup from half as many pairs on.  More pairs than
-            # CUs: see _decode_many.
-            pairs, cus = n_dec * nkv, self._num_cus
             fits = nh // nkv <= int(self._lib[lib].sl_attention_mfma_group_heads())
-            if pairs <= cus:
-                need = self.GROUP_ATTENTION_FILL * cus
-                group = fits and (pairs >= need or (2 * pairs >= need and blocks <= self.GROUP_ATTENTION_SHORT_BLOCKS))
-                nsplit = 1 if group else self._decode_shares(pairs, min(most, blocks // 2))
-            else:
-                group, nsplit = self._decode_many(pairs, blocks, D, fits, min(most, blocks // 2))
-            part_o = part_ml = None
-            if nsplit > 1:
-                part_o = self._new((n_dec, nh, nsplit, D), torch.float32)
-                part_ml = self._new((n_dec, nh, nsplit, 2), torch.float32)
-            self._call(lib, name, *common, n_pre, n_dec, 1, *tail, nsplit, 0, 0, _p(out),
-                       _p(part_o), _p(part_ml), n_pre_tok, n_dec if nsplit > 1 else 0, 0, int(out_rows), int(group))
+            for first, count, group, nsplit in self._decode_launches(n_dec, nkv, blocks, D, fits, most):
+                part_o = part_ml = None
+                if nsplit > 1:
+                    part_o = self._new((count, nh, nsplit, D), torch.float32)
+                    part_ml = self._new((count, nh, nsplit, 2), torch.float32)
+                self._call(lib, name, *common, n_pre + first, count, 1, *tail, nsplit, 0, 0, _p(out),
+                           _p(part_o), _p(part_ml), n_pre_tok + first, count if nsplit > 1 else 0, 0,
+                           int(out_rows), int(group))

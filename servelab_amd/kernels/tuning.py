@@ -118,6 +118,14 @@ class Tuning:
     many_merged_rounds: float = 0.57
     many_merged_base: float = 1.048
     many_fewer_within: float = 1.02
+    # Two launches instead: the sequences that fill whole rounds of the CUs merged in the workgroup,
+    # which then runs at the rate of the stream, and the others as a launch of few pairs, which costs
+    # its own stream or its wavefronts' trips and many_second_launch_us on top (launch, combine
+    # kernel; fitted to launches of 65 to 200 requests); negative: never.  Taken when the estimates
+    # say so, which is when few sequences are left over (contexts of 4,096, 65 / 72 / 130 / 200 requests
+    # of 4 kv heads: 96 / 107 / 188 / 283 us against 108 / 115 / 199 / 298 in one launch; 80 and 144: as
+    # fast either way, one launch).
+    many_second_launch_us: float = 9.0
     # prompt launches share keys through LDS from this many 32-column wavefronts and this context
     # on (7B shape, laid out by chiplet, a workgroup per tile: as fast or faster than a wavefront
     # per 32 columns straight from the pages at every size measured, from 8 tokens to 32 k)

@@ -1002,12 +1002,13 @@ def test_single_tokens_of_more_pairs_than_cus():
     (on a table told that it has 256 CUs: shares that fill whole rounds of the CUs between one pair a
     CU and two, merged in the workgroup where two rounds are nearly full and the context is short, one
     share once there are four wavefronts for every CU), and every form gives the plain result
-    (a table told that it has 8 CUs; 4, 5 and 40 requests of 4 kv heads: merged, two shares, one)."""
+    (a table told that it has 8 CUs; 4, 5, 40 and 9 requests of 4 kv heads: merged, two shares, one share,
+    and two launches: eight requests, which fill whole rounds, merged and the ninth in 46 shares)."""
     from servelab_amd.kernels import HipOps
     dt = torch.bfloat16
     ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
     ops._num_cus = 256
-    plan = lambda pairs, blocks, fits=True: ops._decode_many(pairs, blocks, 128, fits, min(256, blocks // 2))
+    plan = lambda pairs, blocks, fits=True: ops._decode_many(pairs, blocks, 128, fits, min(256, blocks // 2))[:2]
     assert [plan(p, 128) for p in (288, 384, 416, 576, 640, 1024, 4096)] == \
         [(False, 4), (False, 2), (False, 3), (False, 3), (False, 2), (False, 1), (False, 1)]
     assert plan(448, 32) == (True, 1) and plan(448, 32, fits=False) == (False, 2)
@@ -1018,16 +1019,16 @@ def test_single_tokens_of_more_pairs_than_cus():
     call = ops._call
     ops._call = lambda stem, name, *args: (seen.append((args[17], args[-1])) if name.startswith("sl_attention_mfma@") else None,
                                            call(stem, name, *args))[1]
-    for n_seqs, ctx, form in ((4, 700, (1, 1)), (5, 3000, (2, 0)), (40, 700, (1, 0))):
+    for n_seqs, ctx, form in ((4, 700, [(1, 1)]), (5, 3000, [(2, 0)]), (40, 700, [(1, 0)]), (9, 3000, [(1, 1), (46, 0)])):
         seqs = [(ctx - 13 * i, 1) for i in range(n_seqs)]
         qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=ctx)
         qkv, scale = in_units(UNITS[1], qkv, nh, D, 1.0 / math.sqrt(D))
         for shares in (None, 3):                     # the form it takes by itself, and three shares
             if shares:
-                ops._decode_many = lambda *a: (False, shares)
+                ops._decode_many = lambda *a: (False, shares, 0.0)
             seen.clear()
             got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, None)
-            assert seen == [form if shares is None else (3, 0)], (n_seqs, ctx, seen)
+            assert seen == (form if shares is None else [(3, 0)]), (n_seqs, ctx, seen)
             ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
                                       types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
                                                                for k, v in vars(batch).items()}), scale, None)
