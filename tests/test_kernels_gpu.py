@@ -178,7 +178,9 @@ def test_linear_skinny(M, N, K, pairs):
 
 @pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048),
                                    (65, 144, 352), (100, 1000, 3584), (128, 4608, 1024), (127, 70, 2048),
-                                   (64, 37888, 64), (20, 40016, 96)])   # so many tiles that they are spread over a whole multiple of the CUs
+                                   (48, 1000, 352), (80, 3000, 96), (96, 130, 352), (112, 700, 128),    # three, five, six, seven blocks of 16 rows
+                                   (64, 37888, 64), (20, 40016, 96),    # so many tiles that they are spread over a whole multiple of the CUs
+                                   (90, 37888, 64)])                    # ... in workgroups of eight wavefronts with six blocks of rows
 def test_linear_mid(M, N, K):
     """The LDS-staged 17..128-row kernel alone: whole K and K split over up to
     16 workgroups with the separate reduction, plain and gated."""
