@@ -3,7 +3,9 @@ groups of 7, head size 128, intermediate 18944, vocabulary 152064) with two
 layers and random weights: float32 logits equal the plain implementation's to
 1e-4 for a whole prompt, token by token and in portions; bfloat16 stays within
 its bar.  Reductions of 3584 and 18944 terms and a group size that is no power
-of two show what the tiny models cannot."""
+of two show what the tiny models cannot.  The widths of the smallest and of a
+large model of the family (a width that is no multiple of 256, head size 64 and
+a tied head; 8 kv heads of 5 query heads) run the same kind of schedule."""
 import random
 
 import pytest
@@ -159,3 +161,56 @@ def test_float32_error_at_depth():
               f"{arithmetic:.2e} off the float64 logits (largest {top:.2f})")
     assert all(engine <= 1e-4 for engine, _, _ in report.values()), report
     assert all(engine <= arithmetic for engine, arithmetic, _ in report.values()), report
+
+
+OTHER_WIDTHS = {
+    # hidden 896 is no multiple of 256 (no resident form of the consumer products), head size 64, tied head
+    "0.5b": dict(hidden_size=896, num_attention_heads=14, num_key_value_heads=2, head_dim=64, intermediate_size=4864,
+                 tie_word_embeddings=True),
+    # 8 kv heads of 5 query heads, tiles of 10 rows for the producers of a width of 5,120
+    "32b": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, head_dim=128, intermediate_size=27648),
+}
+
+
+@pytest.mark.parametrize("which", sorted(OTHER_WIDTHS))
+def test_other_widths_of_the_family(tmp_path, which):
+    """Two layers of the widths of the smallest and of a large model of the family (vocabulary cut to
+    5,003 rows): a prompt of 300 tokens, then newcomers beside decoded tokens and decode steps of 1, 8,
+    16 and 40 requests, in float32 and in bfloat16 against the plain implementation."""
+    raw = dict(WIDE, vocab_size=5003, eos_token_id=5002, **OTHER_WIDTHS[which])
+    folder = str(tmp_path / "model")
+    write_random_model(Qwen2Config.from_hf(raw), folder, seed=6)
+    rng = random.Random(3)
+    decoded = {"L": 7}
+    decoded.update({f"s{i}": 6 if i < 7 else 4 if i < 15 else 2 for i in range(39)})
+    requests = {"L": [rng.randrange(5003) for _ in range(300 + decoded["L"])]}
+    for i in range(39):
+        requests[f"s{i}"] = [rng.randrange(5003) for _ in range(4 + i % 5 + decoded[f"s{i}"])]
+    reference = plain_logits(folder, requests)
+    fed = {r: 0 for r in requests}
+    steps = []
+
+    def take(r, n):
+        toks = requests[r][fed[r]:fed[r] + n]
+        fed[r] += n
+        return {"id": r, "tokens": toks, "want": [n - 1]}
+
+    live = ["L"]
+    steps.append({"step": 0, "entries": [take("L", 300)], "end": []})
+    for newcomers in ([], [f"s{i}" for i in range(7)], [f"s{i}" for i in range(7, 15)], [f"s{i}" for i in range(15, 39)]):
+        if newcomers:
+            steps.append({"step": len(steps), "end": [],
+                          "entries": [take(r, len(requests[r]) - decoded[r]) for r in newcomers] + [take(r, 1) for r in live]})
+            live += newcomers
+        steps.append({"step": len(steps), "entries": [take(r, 1) for r in live], "end": []})
+    while any(fed[r] < len(requests[r]) for r in requests):
+        steps.append({"step": len(steps), "entries": [take(r, 1) for r in live if fed[r] < len(requests[r])], "end": []})
+    steps[-1]["end"] = list(requests)
+    for dtype in ("float32", "bfloat16"):
+        out = str(tmp_path / ("out_" + dtype))
+        replay_in_process(folder, steps, out, dtype, rs.max_tokens_needed(steps), max_live=40)
+        worst, where = compare(out, steps, reference, 5003)
+        bar = tolerance(dtype, reference) if dtype == "float32" else \
+            bfloat16_bar(folder, requests, reference, 5003, ("other widths", which))
+        print(f"{which} widths, {dtype}: max abs err {worst:.3e} at {where}, bar {bar:.3e}")
+        assert worst < bar, f"{dtype}: max abs err {worst} at {where}, bar {bar}"
