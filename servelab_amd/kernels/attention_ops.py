@@ -75,7 +75,7 @@ class AttentionOps:
         if N != (nh + 2 * nkv) * D or D % 16 or rot % 16 or not 0 <= rot <= D:
             raise KernelError("qkv_rope_store: weight rows must be (nh + 2 nkv) * D with D % 16 == 0, "
                               "the rotated width a multiple of 16")
-        fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= 16
+        fused = (self.act_dtype == torch.bfloat16 and self.fuse_rope and 0 < M <= self._fused_rows(K)
                  and weight.tiled is not None and weight.shape == (N, K))
         if not fused:
             plan = None if isinstance(x, ScaledRows) else self._block_plan(M, N, K, weight)
@@ -87,7 +87,7 @@ class AttentionOps:
                 self.rope_store(qkv, nh, nkv, D, cos, sin, slots, k_cache, v_cache, page_size,
                                 True, split=product, rot_dim=rot, q_scale=q_scale)
                 return qkv
-            if (self.WIDE_MIN_M <= M <= self._few_rows_limit(weight) and K % 32 == 0
+            if (self._wide_from(K) <= M <= self._few_rows_limit(weight) and K % 32 == 0
                     and not isinstance(x, ScaledRows)):
                 # K split over workgroups; the rotation kernel adds the partial sums up
                 product = self.linear_mid(x, weight, bias, partial=True)
@@ -205,7 +205,7 @@ class AttentionOps:
         if not isinstance(w_out, LinearWeight):
             w_out = LinearWeight(w_out)
         T = qkv.shape[0]
-        tiled = (self.tile_few_rows and 1 < T <= self.FUSED_NORM_MAX_M and batch.max_q_len == 1
+        tiled = (self.tile_few_rows and 1 < T <= self._fused_rows(w_out.shape[0]) and batch.max_q_len == 1
                  and batch.num_prefill_seqs == 0 and batch.num_seqs == T and w_out.tiled is not None
                  and w_out.shape[1] == nh * D
                  and self._mfma_attention_fits(D, nh // nkv, block_tables.shape[1], page_size, batch))

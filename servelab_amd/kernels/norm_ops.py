@@ -54,7 +54,7 @@ class NormOps:
         self._check(weight, torch.float32, (H,), "norm weight")
         self._check(rows, torch.int32, (R,), "rows")
         if isinstance(delta, Deferred):
-            if fuse and R <= 16:
+            if fuse and R <= self._fused_rows(H):
                 scaled = self._produce_scaled_rows(resid, delta, weight, eps)
                 scaled.rows = rows
                 return scaled

@@ -148,7 +148,6 @@ class ProductOps:
         self._call("gemm", "sl_untile_weight", _p(weight.tiled), _p(out), N, K, 16)
         return out
 
-    FUSED_NORM_MAX_M = 16         # the fused add + norm lives in the kernel for up to 16 rows
 
     def linear(self, x, weight, bias, out_f32=False, defer=False):
         """y = x W^T (+ bias); ``weight`` is a LinearWeight or a plain [N, K] tensor.
@@ -175,7 +174,7 @@ class ProductOps:
             y = self._new((M, N), torch.float32 if out_f32 else None)
             self._skinny(x, weight, bias, y, M, N, K, out_f32)
             return y
-        if (defer and self.fuse_norms and not out_f32 and 0 < M <= self.FUSED_NORM_MAX_M
+        if (defer and self.fuse_norms and not out_f32 and 0 < M <= self._fused_rows(N)
                 and weight.tiled is not None and weight.shape == (N, K) and N <= 8192):
             return Deferred(x, weight, bias)
         self._check(x, self.act_dtype, None, "x")
@@ -197,7 +196,7 @@ class ProductOps:
             # (deferred: the norm adds the partial sums)
             return self.linear_block(x, weight, bias, out_f32, plan[0],
                                      partial=defer and self.fuse_norms and not out_f32, square=plan[1])
-        if (defer and self.fuse_norms and not out_f32 and self.WIDE_MIN_M <= M <= limit
+        if (defer and self.fuse_norms and not out_f32 and self._wide_from(N) <= M <= limit
                 and K % 32 == 0 and N % 4 == 0 and self._takes_mid(M, N, K)):
             return self.linear_mid(x, weight, bias, partial=True,     # the norm adds the partial sums
                                    target=self.MID_DEFERRED_WORKGROUPS)
@@ -326,7 +325,7 @@ class ProductOps:
         N = weight.shape[0]
         if weight.tiled is None:
             raise KernelError("linear_skinny needs the tiled copy of the weight")
-        if M >= self.WIDE_MIN_M:
+        if M >= self._wide_from(min(N, K)):       # (the stream is what a projection reads or what it writes)
             if self._takes_mid(M, N, K):
                 return self.linear_mid(x, weight, bias, out_f32)
             return self.linear_wide(x, weight, bias, out_f32)
@@ -379,7 +378,7 @@ class ProductOps:
             return self._linear_scaled(x, weight, None, False, True, y_tiled=_tiled_out)
         M, K = x.shape
         N = weight.shape[0]
-        if (_tiled_out and M < self.WIDE_MIN_M and M <= self._few_rows_limit(weight)
+        if (_tiled_out and M < self._wide_from(K) and M <= self._few_rows_limit(weight)
                 and block == self.GATE_BLOCK and N % 16 == 0):
             self._check(x, self.act_dtype, None, "x")
             y = self._new((M, N // 2))
@@ -387,7 +386,7 @@ class ProductOps:
             return TiledRows(y, (M, N // 2))
         if M <= self._few_rows_limit(weight) and block == self.GATE_BLOCK and N % 16 == 0:
             self._check(x, self.act_dtype, None, "x")
-            if M >= self.WIDE_MIN_M:
+            if M >= self._wide_from(K):
                 if self._takes_mid(M, N, K):
                     return self.linear_mid(x, weight, None, gated=True)
                 return self.linear_wide(x, weight, None, gated=True)
@@ -407,7 +406,7 @@ class ProductOps:
             w_down = LinearWeight(w_down)
         M = x.shape[0]
         inner = w_gate_up.shape[0] // 2
-        tiled = (self.act_dtype == torch.bfloat16 and self.tile_few_rows and 1 < M <= self.FUSED_NORM_MAX_M
+        tiled = (self.act_dtype == torch.bfloat16 and self.tile_few_rows and 1 < M <= self._fused_rows(w_down.shape[0])
                  and block == self.GATE_BLOCK and inner % 32 == 0 and w_gate_up.tiled is not None
                  and w_down.tiled is not None and w_down.shape[1] == inner and w_gate_up.shape[0] % 16 == 0)
         h = self.gated_linear(x, w_gate_up, block, _tiled_out=tiled)

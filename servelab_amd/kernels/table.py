@@ -66,6 +66,19 @@ class KernelTable:
         self.graph_rows_limit = self.MID_MAX_M if act_dtype == torch.bfloat16 else self.SKINNY_MAX_M
 
     # ------------------------------------------------------------ plumbing
+    def _fused_rows(self, width) -> int:
+        """Up to how many rows a step over a residual stream of ``width`` values takes the fused
+        few-rows kernels (``Tuning.fused_rows_by_width``)."""
+        for upto, rows in self.FUSED_ROWS_BY_WIDTH:
+            if width <= upto:
+                return min(int(rows), self.FUSED_NORM_MAX_M)
+        return 0
+
+    def _wide_from(self, width) -> int:
+        """From how many rows on the products of a step over a stream of ``width`` values take
+        the kernels in which tiles of W share their reads of x."""
+        return min(self.WIDE_MIN_M, self._fused_rows(width) + 1)
+
     def _call(self, stem, name, *args):
         fn = self._fn.get(name)
         if fn is None:

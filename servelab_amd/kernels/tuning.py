@@ -33,6 +33,17 @@ class Tuning:
 
     # few-rows products of at most 8 rows load x for two k-steps at once (gemm.hip, stream_k2)
     pair_x_loads: bool = True
+    # Up to how many rows a step takes the few-rows kernels with the residual add, the norm and the
+    # rotation fused in (16 at most: the rows of one matrix instruction), by the width of the residual
+    # stream: (width up to which, rows) pairs.  Those kernels read all rows of x again for every tile of 16
+    # rows of W, the LDS-staged ones once for 128 or 256, at the price of three more kernels a layer; the
+    # wider the stream, the fewer rows the fused ones are ahead for (ms a decode step, contexts of 4,096,
+    # fused up to 16 / 8 / 0 rows: 7B shape, width 3,584, 8 requests 3.14 / 3.14 / 3.59, 16 requests 3.64 / 3.97
+    # / 3.99; 32B shape, 5,120: 8 requests 12.6 / 12.5 / 13.2, 16 requests 14.9 / 14.8 / 14.7; 72B shape, 8,192,
+    # whose gate/up has no form that keeps x in registers: 1 request 25.2 / 25.2 / 24.2, 8 requests 26.3 / 26.3 /
+    # 25.6, 16 requests 31.1 / 27.3 / 27.3)
+    fused_norm_max_m: int = 16
+    fused_rows_by_width: tuple = ((4096, 16), (6144, 8), (1 << 30, 0))
 
     # ---- products of 17 and more rows over the tiled copy
     # from this many rows on two tiles of W share one read of x (gemm_wide / gemm_mid)

@@ -307,9 +307,10 @@ def test_fused_add_norm_around_few_rows_products(M, H, N2, pairs, th):
     same results as product, add, norm and product one after the other; with
     one tile of W per workgroup and with two; with the first matrix in tiles
     of 16 rows and in a further copy of lower tiles (the last tile partly empty)."""
-    from servelab_amd.kernels import HipOps
+    from servelab_amd.kernels import HipOps, Tuning
     from servelab_amd.kernels.ops import Deferred, ScaledRows
-    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    # (the fused kernels at every width, also those whose steps take the LDS-staged ones by themselves)
+    ops, emu = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(fused_rows_by_width=((1 << 30, 16),))), EmulatedOps(torch.bfloat16)
     if pairs:
         ops._pair_tiles = lambda M, N, K, th=16: True
     K1 = 128 if H != 3584 else 4160       # (the long one: 224 tiles, sixteen wavefronts a workgroup)

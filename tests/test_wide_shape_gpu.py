@@ -3,9 +3,11 @@ groups of 7, head size 128, intermediate 18944, vocabulary 152064) with two
 layers and random weights: float32 logits equal the plain implementation's to
 1e-4 for a whole prompt, token by token and in portions; bfloat16 stays within
 its bar.  Reductions of 3584 and 18944 terms and a group size that is no power
-of two show what the tiny models cannot.  The widths of the smallest and of a
-large model of the family (a width that is no multiple of 256, head size 64 and
-a tied head; 8 kv heads of 5 query heads) run the same kind of schedule."""
+of two show what the tiny models cannot.  The widths of the smallest and of the
+two largest models of the family (a width that is no multiple of 256, head size
+64 and a tied head; 8 kv heads of 5 and of 8 query heads; streams for which the
+fused few-rows kernels end at 8 rows, or are not taken at all) run the same kind
+of schedule."""
 import random
 
 import pytest
@@ -169,12 +171,14 @@ OTHER_WIDTHS = {
                  tie_word_embeddings=True),
     # 8 kv heads of 5 query heads, tiles of 10 rows for the producers of a width of 5,120
     "32b": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, head_dim=128, intermediate_size=27648),
+    # a stream so wide that no step takes the fused few-rows kernels
+    "72b": dict(hidden_size=8192, num_attention_heads=64, num_key_value_heads=8, head_dim=128, intermediate_size=29568),
 }
 
 
 @pytest.mark.parametrize("which", sorted(OTHER_WIDTHS))
 def test_other_widths_of_the_family(tmp_path, which):
-    """Two layers of the widths of the smallest and of a large model of the family (vocabulary cut to
+    """Two layers of the widths of the smallest and of the two largest models of the family (vocabulary cut to
     5,003 rows): a prompt of 300 tokens, then newcomers beside decoded tokens and decode steps of 1, 8,
     16 and 40 requests, in float32 and in bfloat16 against the plain implementation."""
     raw = dict(WIDE, vocab_size=5003, eos_token_id=5002, **OTHER_WIDTHS[which])
