@@ -106,6 +106,11 @@ struct AttnParams {
                                  // product that reads them: element (t, c) at (c / 32) * (out_rows * 32) + t * 32 + c % 32
   int by_chiplet;                // a one-dimensional grid laid out by Place below (else x: workgroup of a pair, y: kv head, z: sequence)
   int grid_x, num_seqs;          // ... its extent per (sequence, kv head) pair, and the sequences
+  // Split single tokens: shares of one length for all sequences of the launch instead of nsplit shares each (see
+  // share_count).  ctx_stats: the sum and the largest of the launch's context lengths, on the device (they change from
+  // step to step under a captured graph); share_waves: the wavefronts the launch aims at; null / 0: nsplit shares each.
+  const int* ctx_stats;
+  int share_waves;
 };
 
 // where element (row, col) of the result goes (col = head * D + channel; runs of four channels stay together)
@@ -451,31 +456,88 @@ __device__ __forceinline__ void walk_blocks(Columns<NB, FOLD>& C, const AttnPara
   }
 }
 
+// Into how many shares the nblk key blocks of a single token's sequence are cut, nsplit at most.  With
+// contexts of different lengths, nsplit shares for every sequence would leave the launch waiting for
+// the shares of its longest sequence while the wavefronts of the short ones have long finished (7B
+// shape, 64 requests of which 8 have 4,096 keys and the others a few hundred, merged in the
+// workgroup or in 4 shares each: 62 and 72 us a layer; streaming their keys takes 18).  So every share
+// of the launch gets about the same number of blocks: the launch's blocks (from the sum of its
+// contexts) over the wavefronts it aims at, no fewer than its longest sequence needs to fit nsplit
+// shares; a long sequence is cut into many, a short one into one, and the wavefronts of the shares a
+// sequence does not use leave at once.  Equal contexts give every sequence share_waves / pairs shares.
+__device__ __forceinline__ int share_count(const AttnParams& P, int nblk) {
+  if (P.ctx_stats == nullptr || P.share_waves <= 0) return P.nsplit;
+  long long total = P.ctx_stats[0];
+  int longest = P.ctx_stats[1];
+  if (P.window > 0) {                                // (a window bounds what a sequence reads)
+    longest = longest < P.window + 31 ? longest : P.window + 31;
+    total = total < (long long)P.num_seqs * longest ? total : (long long)P.num_seqs * longest;
+  }
+  const long long blocks = (total / 32 + P.num_seqs) * P.nkv;                 // key blocks of all pairs, rounded up
+  // (contexts of different lengths: up to twice the wavefronts, of shorter shares, which even out better;
+  // equal contexts keep the count the launch was planned with, whose wavefronts fill whole rounds of the CUs)
+  long long aim = (long long)P.share_waves * longest * P.num_seqs / (total > 0 ? total : 1);
+  aim = aim < P.share_waves ? P.share_waves : aim < 2ll * P.share_waves ? aim : 2ll * P.share_waves;
+  int each = (int)((blocks + aim - 1) / aim);
+  const int fit = (longest / 32 + P.nsplit) / P.nsplit;                         // ceil((longest / 32 + 1) / nsplit)
+  each = each > fit ? each : fit;
+  each = each > 2 ? each : 2;
+  const int n = (nblk + each - 1) / each;
+  return n < 1 ? 1 : n < P.nsplit ? n : P.nsplit;
+}
+
 // One wavefront per workgroup; operands straight from the pages.  Used for
 // decode tokens (SPLIT: the wavefront takes one share of the key blocks) and
 // for prompt portions whose launch does not saturate L2.
 template <int NB, bool SPLIT, bool FOLD, bool PAIRS = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 256 ? 2 : 1))) void attention_mfma_kernel(const AttnParams P) {
   const int lane = threadIdx.x, n = lane & 15, gq = lane >> 4;
-  const int seq = P.seq_begin + blockIdx.z, kvh = blockIdx.y;
+  // Split single tokens come as a one-dimensional grid: all (sequence, kv head) pairs of share 0, then those
+  // of share 1, .., the pairs counted up to a multiple of 8 and, within each eight, rotated by the share.
+  // (and by the number of the eight, so that sequences a multiple of 8 apart do not share a chiplet either).
+  // Workgroups go to the eight chiplets in turn, so workgroup L runs on chiplet L % 8 = (pair + share + pair / 8) % 8:
+  // the shares of one pair go round the chiplets (a long sequence among short ones loads them all), and
+  // so do the pairs of one share (a sequence may use the first few shares only: with the share as the
+  // fastest index, eight slots and two shares in use, two chiplets did all the work).
+  const int pairs = P.nkv * P.num_seqs, pairs8 = (pairs + 7) & ~7;
+  const int share_of = SPLIT ? blockIdx.x / pairs8 : 0, place = SPLIT ? blockIdx.x % pairs8 : 0;
+  const int pair_of = (place & ~7) | ((place - share_of - (place >> 3)) & 7);
+  if (SPLIT && pair_of >= pairs) return;
+  const int seq = P.seq_begin + (SPLIT ? pair_of / P.nkv : (int)blockIdx.z);
+  const int kvh = SPLIT ? pair_of % P.nkv : (int)blockIdx.y;
   const int g = P.nh / P.nkv;
   const int q0 = P.cu_q[seq];
   const int qlen = P.cu_q[seq + 1] - q0;
   const int ncols = qlen * g;
   const int ntiles = (ncols + 16 * NB - 1) / (16 * NB);
-  const int tile_rev = blockIdx.x / P.nsplit, split = blockIdx.x % P.nsplit;
+  const int tile_rev = SPLIT ? 0 : blockIdx.x / P.nsplit, split = SPLIT ? share_of : blockIdx.x % P.nsplit;
   if (tile_rev >= ntiles) return;
   const int tile = ntiles - 1 - tile_rev;          // long (late) tiles first
   const int pos0 = P.positions[q0];
   const int* table = P.block_tables + (size_t)seq * P.max_pages;
+  int shares = P.nsplit;
+  if (SPLIT) {
+    // (a single token: the blocks from its window's first key to its own position, as Columns::init finds them)
+    const int kmin = P.window > 0 && pos0 - P.window + 1 > 0 ? pos0 - P.window + 1 : 0;
+    shares = share_count(P, pos0 / 32 + 1 - kmin / 32);
+    if (split >= shares) {
+      // a share this sequence does not use: nothing but the mark that the combine kernel skips
+      if (lane < g) {
+        const size_t pr = (((size_t)q0 - P.part_row0) * P.nh + kvh * g + lane) * P.nsplit + split;
+        P.part_ml[pr * 2] = -INFINITY;
+        P.part_ml[pr * 2 + 1] = 0.f;
+      }
+      return;
+    }
+  }
 
   Columns<NB, FOLD> C;
   C.init(P, q0, ncols, tile * 16 * NB, pos0, kvh, g, n, gq);
   int kb_begin = C.kb_begin, kb_end = C.kb_end;
   if (SPLIT) {
     const int nblk = kb_end - kb_begin;
-    const int first = kb_begin + (int)((long long)nblk * split / P.nsplit);
-    kb_end = kb_begin + (int)((long long)nblk * (split + 1) / P.nsplit);
+    const int first = kb_begin + (int)((long long)nblk * split / shares);
+    kb_end = kb_begin + (int)((long long)nblk * (split + 1) / shares);
     kb_begin = first;
   }
   walk_blocks<NB, FOLD, PAIRS>(C, P, table, kvh, n, gq, kb_begin, kb_end);
@@ -842,9 +904,9 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
 #pragma unroll
       for (int u = 0; u < 8; ++u) v[u] = po[(size_t)(j + u) * D + d];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) acc += ws[j + u] * v[u];
+      for (int u = 0; u < 8; ++u) acc += ws[j + u] != 0.f ? ws[j + u] * v[u] : 0.f;     // (a share without keys wrote no output)
     }
-    for (; j < nsplit; ++j) acc += ws[j] * po[(size_t)j * D + d];
+    for (; j < nsplit; ++j) acc += ws[j] != 0.f ? ws[j] * po[(size_t)j * D + d] : 0.f;
     out[out_index(out_rows, nh, (size_t)(part_row0 + r), h * D + d)] = (__bf16)(acc * inv);
   }
 }
@@ -871,7 +933,7 @@ extern "C" const char* sl_attention_mfma(
     int max_pages, const int* cu_q, const int* positions, int seq_begin, int num_seqs,
     int max_q_len, int nh, int nkv, int head_dim, int page, float scale, int window, int nsplit,
     int shared_min_waves, int pair_tiles, void* out, float* part_o, float* part_ml, int part_row0, int part_rows,
-    int narrow_below, int out_rows, int group, hipStream_t stream) {
+    int narrow_below, int out_rows, int group, const int* ctx_stats, int share_waves, hipStream_t stream) {
   SL_CHECK(head_dim == D, "attention_mfma: built for another head size");
   SL_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: heads must be a multiple of kv heads");
   SL_CHECK(page == 16 || page == 32 || page == 64, "attention_mfma: page size must be 16, 32 or 64");
@@ -884,7 +946,7 @@ extern "C" const char* sl_attention_mfma(
   const int g = nh / nkv;
   AttnParams P{(const __bf16*)qkv, row_stride, (const __bf16*)kc, (const __bf16*)vc, block_tables,
                max_pages, cu_q, positions, seq_begin, nh, nkv, page, scale, window, nsplit,
-               (__bf16*)out, part_o, part_ml, part_row0, pair_tiles, out_rows, 0, 0, 0};
+               (__bf16*)out, part_o, part_ml, part_row0, pair_tiles, out_rows, 0, 0, num_seqs, nullptr, 0};
   SL_CHECK(out_rows >= 0 && (out_rows == 0 || (max_q_len == 1 && seq_begin == 0 && out_rows == num_seqs)),
            "attention_mfma: a result laid out by k-step is that of a step of single tokens, all of its rows");
   const long long cols = (long long)max_q_len * g;
@@ -909,7 +971,11 @@ extern "C" const char* sl_attention_mfma(
              "attention_mfma: a split launch needs partial buffers for its rows");
     SL_CHECK(g <= 64, "attention_mfma: more than 64 query heads per kv head");
     SL_CHECK(nsplit <= 64 * COMBINE_PER_LANE, "attention_mfma: too many splits of the context");
-    const dim3 grid(nsplit, nkv, num_seqs);
+    const long long pairs8 = ((long long)nkv * num_seqs + 7) / 8 * 8;
+    SL_CHECK(nsplit * pairs8 < (1ll << 31), "attention_mfma: too many shares");
+    const dim3 grid((unsigned)(nsplit * pairs8));
+    P.ctx_stats = ctx_stats;
+    P.share_waves = share_waves;
     if (fold) {
       if (g <= 16) attention_mfma_kernel<1, true, true, true><<<grid, 64, 0, stream>>>(P);
       else if (g <= 32) attention_mfma_kernel<2, true, true><<<grid, 64, 0, stream>>>(P);

@@ -50,6 +50,9 @@ class StepBatch:
     state_slots: torch.Tensor    # [S]
     logit_rows: torch.Tensor     # [R]
     groups: List[GroupMeta]
+    # [2] the sum and the largest of the context lengths of the single-token sequences (what a kernel that
+    # shares out their keys balances by; on the device because a captured step is fed new lengths)
+    ctx_stats: torch.Tensor = None
     # host copies for parts that plan on the host
     q_lens: List[int] = field(default_factory=list)
     starts: List[int] = field(default_factory=list)
@@ -123,6 +126,8 @@ def build_arrays(entries: List[StepEntry], starts: List[int], rows: List[int], m
         parts += [slots, tables.reshape(-1)]
         group_pages.append(max_pages)
 
+    single = ctx[np.asarray(q_lens) == 1]
+    parts.append(np.asarray([single.sum(), single.max()] if single.size else [0, 0], dtype=np.int32))
     sizes = [p.size for p in parts]
     offsets = np.concatenate([[0], np.cumsum([-(-s // 4) * 4 for s in sizes])])   # 16-byte aligned
     flat = np.zeros(int(offsets[-1]), dtype=np.int32)
@@ -147,7 +152,7 @@ def batch_on_device(arr: BatchArrays, dev: torch.Tensor, max_ctx_len: int = 0) -
         num_prefill_tokens=sum(q for q in arr.q_lens if q > 1), num_logit_rows=arr.num_rows,
         max_q_len=max(arr.q_lens), max_ctx_len=max_ctx_len or arr.max_ctx_len,
         ids=views[0], positions=views[1], tok_seq=views[2], cu_q=views[3], ctx_len=views[4],
-        state_slots=views[5], logit_rows=views[6], groups=groups,
+        state_slots=views[5], logit_rows=views[6], groups=groups, ctx_stats=views[-1],
         q_lens=arr.q_lens, starts=arr.starts, requests=arr.requests,
         host_state_slots=arr.state_slots)
 

@@ -420,18 +420,37 @@ class AttentionOps:
                 part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
                        0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
-                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS if triangle else 0, 0, 0)
+                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS if triangle else 0, 0, 0, None, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:
                 blocks = min(blocks, -(-int(window) // 32) + 1)
             most = int(self._lib[lib].sl_attention_mfma_max_splits())
             fits = nh // nkv <= int(self._lib[lib].sl_attention_mfma_group_heads())
-            for first, count, group, nsplit in self._decode_launches(n_dec, nkv, blocks, D, fits, most):
+            launches = self._decode_launches(n_dec, nkv, blocks, D, fits, most)
+            # (Tuning.shares_of_one_length) More pairs than CUs in one launch, and the step says how long its
+            # contexts are: shares of one length for all its sequences (see share_count in the kernel).  The launch is planned as for
+            # equal contexts, in shares (workgroups that merge in LDS wait for their longest sequence), aims
+            # at the wavefronts of that plan, and has room for SHARE_SLOTS_GROWTH times as many shares of a
+            # long sequence among short ones (up to SHARE_SLOTS_WAVES wavefronts launched in all).  7B shape,
+            # 128 requests, us a layer: contexts of 4,096 all 174 (173 in two shares each); uniform in 64..4,096:
+            # 117 against 135; one in eight at 4,096 and the others below 512: 77-87 against 131.  With fewer
+            # pairs the plans above are as good or better (64 requests, uniform: 79 against 71 merged).
+            stats = getattr(batch, "ctx_stats", None) if self.SHARES_OF_ONE_LENGTH else None
+            if stats is not None and len(launches) == 1 and n_dec * nkv > self._num_cus:
+                shares = launches[0][3] if not launches[0][2] else \
+                    self._decode_many(n_dec * nkv, blocks, D, False, min(most, blocks // 2))[1]
+                room = min(self.SHARE_SLOTS_GROWTH * shares, self.SHARE_SLOTS_WAVES // (n_dec * nkv))
+                slots = max(1, min(most, max(1, blocks // 2), max(shares, room)))
+                launches = [(0, n_dec, False, slots)] if slots > 1 else launches
+                aim = shares * n_dec * nkv if slots > 1 else 0
+            else:
+                aim = 0
+            for first, count, group, nsplit in launches:
                 part_o = part_ml = None
                 if nsplit > 1:
                     part_o = self._new((count, nh, nsplit, D), torch.float32)
                     part_ml = self._new((count, nh, nsplit, 2), torch.float32)
                 self._call(lib, name, *common, n_pre + first, count, 1, *tail, nsplit, 0, 0, _p(out),
                            _p(part_o), _p(part_ml), n_pre_tok + first, count if nsplit > 1 else 0, 0,
-                           int(out_rows), int(group))
+                           int(out_rows), int(group), _p(stats) if aim else None, aim)

@@ -137,6 +137,19 @@ class Tuning:
     # of 4 kv heads: 96 / 107 / 188 / 283 us against 108 / 115 / 199 / 298 in one launch; 80 and 144: as
     # fast either way, one launch).
     many_second_launch_us: float = 9.0
+    # single tokens of more pairs than CUs in a step that says how long its contexts are: shares of one
+    # length for all sequences (a long sequence among short ones is cut into up to share_slots_growth times
+    # the shares of the plan for equal contexts, no more than share_slots_waves wavefronts launched in all;
+    # those a sequence does not use leave at once).  Off by default: it pays where contexts differ (7B
+    # shape, 128 requests, us a layer: lengths uniform in 64..4,096 117 against 135, one request in eight at
+    # 4,096 among short ones 77-87 against 131; 256 requests 112-161 against 184-240; a serving load of 128
+    # in flight with prompts of 64 to 3,500 tokens: 5,288 against 5,230 tok/s, its steps being mostly
+    # prompt portions) and costs where they are equal (a decode step of 96 / 128 / 256 requests at
+    # contexts of 4,096: +2.9 / +1.0 / +7.5 %: more share slots to combine, and a combine kernel where one
+    # share a pair needed none), which is what the decode benchmarks measure.
+    shares_of_one_length: bool = False
+    share_slots_growth: int = 4
+    share_slots_waves: int = 4096
     # prompt launches share keys through LDS from this many 32-column wavefronts and this context
     # on (7B shape, laid out by chiplet, a workgroup per tile: as fast or faster than a wavefront
     # per 32 columns straight from the pages at every size measured, from 8 tokens to 32 k)

@@ -98,6 +98,38 @@ def test_long_decoding_across_graph_captures(tmp_path, which, page, dtype, monke
     assert worst < bar, f"max abs err {worst} at {where}, bar {bar}"
 
 
+def test_long_decoding_in_shares_of_one_length(tmp_path, monkeypatch):
+    """Four requests of very different lengths decoded side by side through the captured graphs with the
+    single tokens' keys in shares of one length for all sequences (a table told that it has 2 CUs, so
+    that four pairs are more than it has; the sums the kernel balances by change with every replay)."""
+    from servelab_amd.kernels import HipOps, Tuning
+    monkeypatch.setattr(ModelRunner, "GRAPH_MIN_CONTEXT", 64)
+    folder = make_folder(tmp_path, "B", seed=31, use_sliding_window=False)
+    vocab = TINY["B"]["vocab_size"]
+    rng = random.Random(6)
+    starts = {"p": 400, "q": 3, "r": 70, "s": 33}
+    requests = {r: [rng.randrange(vocab) for _ in range(n + 100)] for r, n in starts.items()}
+    reference = plain_logits(folder, requests)
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": requests[r][:n], "want": [n - 1]} for r, n in starts.items()],
+              "end": []}]
+    for i in range(100):
+        steps.append({"step": i + 1, "entries": [{"id": r, "tokens": [requests[r][n + i]], "want": [0]}
+                                                 for r, n in starts.items()],
+                      "end": list(starts) if i == 99 else []})
+    ops = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(shares_of_one_length=True))
+    ops._num_cus = 2
+    told = []
+    call = ops._call
+    ops._call = lambda stem, name, *args: (told.append(args[-1]) if name.startswith("sl_attention_mfma@") and args[10] == 1
+                                           else None, call(stem, name, *args))[1]
+    out = str(tmp_path / "out")
+    replay_in_process(folder, steps, out, "bfloat16", rs.max_tokens_needed(steps), block_size=16, ops=ops)
+    assert told and any(told)                        # (launches that were told the wavefronts to aim at)
+    worst, where = compare(out, steps, reference, vocab)
+    bar = bfloat16_bar(folder, requests, reference, vocab, "one length")
+    assert worst < bar, f"max abs err {worst} at {where}, bar {bar}"
+
+
 @pytest.mark.parametrize("page,other", [(32, {}), (16, dict(head_dim=64, num_key_value_heads=2, use_sliding_window=False))])
 def test_long_decoding_with_the_keys_merged_inside_the_workgroup(tmp_path, page, other, monkeypatch):
     """The decode attention that a large batch takes by itself (a workgroup of eight wavefronts per
@@ -122,7 +154,7 @@ def test_long_decoding_with_the_keys_merged_inside_the_workgroup(tmp_path, page,
     ops = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(group_attention_fill=0.0))
     merged = []
     call = ops._call
-    ops._call = lambda stem, name, *args: (merged.append(args[-1]) if name.startswith("sl_attention_mfma@") and args[10] == 1
+    ops._call = lambda stem, name, *args: (merged.append(args[-3]) if name.startswith("sl_attention_mfma@") and args[10] == 1
                                            else None, call(stem, name, *args))[1]
     out = str(tmp_path / "out")
     replay_in_process(folder, steps, out, "bfloat16", rs.max_tokens_needed(steps), block_size=page, ops=ops)

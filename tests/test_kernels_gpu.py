@@ -3,6 +3,7 @@
 tiny models': widths and vocabularies that are no power of two, several head
 sizes, group sizes and page sizes."""
 import math
+import random
 import types
 
 import pytest
@@ -855,7 +856,8 @@ def test_attention_over_random_batches(seed):
     """Seeded random batches through the launches the table chooses by itself: whole prompts, portions
     deep in their contexts (two tokens to hundreds), single tokens after them; 1 to 16 kv heads (laid
     out by chiplet or not), with and without a window; on a table that believes in 8 CUs, so that a few
-    single tokens already merge inside their workgroups.  Against the plain computation."""
+    single tokens already merge inside their workgroups or, for every third seed, take shares of one
+    length.  Against the plain computation."""
     import random
     from servelab_amd.kernels import HipOps
     rnd = random.Random(seed)
@@ -871,15 +873,19 @@ def test_attention_over_random_batches(seed):
         prompts.append((q + rnd.choice([0, 0, 5, 200, 900]), q))
     singles = [(rnd.randint(1, 1500), 1) for _ in range(rnd.choice([0, 1, 3, 9]))]
     seqs = prompts + singles or [(77, 77)]
-    ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
+    from servelab_amd.kernels import Tuning
+    ops, emu = HipOps(dt, "cuda:0", tuning=Tuning(shares_of_one_length=seed % 3 == 0)), EmulatedOps(dt)
     ops._num_cus = 8
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=seed)
     qkv, scale = in_units(UNITS[seed % 2], qkv, nh, D, 1.0 / math.sqrt(D))
-    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
     ref = emu.paged_attention(qkv.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(),
                               types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v)
                                                        for k, v in vars(batch).items()}),
                               scale, window)
+    # (what the engine's batches say of their single tokens: the sum and the largest of their contexts)
+    batch.ctx_stats = torch.tensor([sum(c for c, _ in singles), max([c for c, _ in singles] or [0])],
+                                   dtype=torch.int32, device="cuda")
+    got = ops.paged_attention(qkv, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt], (nh, nkv, D, page, window, seqs)
 
 
@@ -973,7 +979,7 @@ def test_decode_attention_merged_inside_the_workgroup(nh, nkv, D, page, window, 
 
     def spy(stem, name, *args):
         if name.startswith("sl_attention_mfma@"):
-            seen.append((args[17], args[-1]))                    # shares, merged inside the workgroup
+            seen.append((args[17], args[-3]))                    # shares, merged inside the workgroup
         return call(stem, name, *args)
     ops._call = spy
     seqs = [(1, 1), (5, 1), (64, 1), (65, 1), (333, 1), (700, 1), (129, 1), (4100, 1)]
@@ -992,12 +998,56 @@ def test_decode_attention_merged_inside_the_workgroup(nh, nkv, D, page, window, 
     for n_seqs, ctx, merged in ((-(-24 // nkv), 4000, True), (max(1, 23 // nkv), 4000, False), (-(-12 // nkv), 900, True),
                                 (-(-12 // nkv), 1100, False)) if window is None else ():      # (a window makes every context short)
         seen.clear()
-        plain._call = lambda stem, name, *args: (seen.append((args[17], args[-1])) if name.startswith("sl_attention_mfma@") else None,
+        plain._call = lambda stem, name, *args: (seen.append((args[17], args[-3])) if name.startswith("sl_attention_mfma@") else None,
                                                  HipOps._call(plain, stem, name, *args))[1]
         case = make_attention_case(dt, nh, nkv, D, page, [(ctx - 3 * i, 1) for i in range(n_seqs)], seed=3)
         q2, s2 = in_units(units, case[0], nh, D, 1.0 / math.sqrt(D))
         plain.paged_attention(q2, nh, nkv, D, case[1], case[2], page, case[3], case[4], s2, window)
         assert len(seen) == 1 and bool(seen[0][1]) == bool(merged) and (seen[0][0] == 1 or not merged), (n_seqs, ctx, seen)
+
+
+@pytest.mark.parametrize("nh,nkv,D,page,window", [(28, 4, 128, 16, None), (8, 1, 64, 32, None), (40, 8, 128, 16, 700), (20, 1, 128, 64, None)])
+def test_single_tokens_in_shares_of_one_length(nh, nkv, D, page, window):
+    """Contexts of very different lengths in one step that says how long they are: every share of the
+    launch has about as many key blocks, a long sequence is cut into more shares than the plan for
+    equal contexts has, a short one into one, and the wavefronts of the shares a sequence does not
+    use leave a mark that the combine kernel skips.  Against the plain result, and the launch itself:
+    more share slots than the plan's shares, and the step's sums on the device."""
+    from servelab_amd.kernels import HipOps, Tuning
+    dt = torch.bfloat16
+    emu = EmulatedOps(dt)
+    rng = random.Random(nh)
+    told = 0
+    for lens in ([4100] + [rng.randrange(1, 300) for _ in range(23)], [rng.randrange(1, 2000) for _ in range(40)],
+                 [3000] * 12, [1], [5, 4100, 70, 33, 64, 65]):
+        seqs = [(c, 1) for c in lens]
+        qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=len(lens))
+        host = types.SimpleNamespace(**{k: (v.cpu() if torch.is_tensor(v) else v) for k, v in vars(batch).items()})
+        q2, scale = in_units(UNITS[1], qkv, nh, D, 1.0 / math.sqrt(D))
+        ref = emu.paged_attention(q2.cpu(), nh, nkv, D, kc.cpu(), vc.cpu(), page, tables.cpu(), host, scale, window)
+        batch.ctx_stats = torch.tensor([sum(lens), max(lens)], dtype=torch.int32, device="cuda")
+        for tuning in (Tuning(shares_of_one_length=True), Tuning(shares_of_one_length=True, share_slots_growth=1),
+                       Tuning(shares_of_one_length=True, share_slots_growth=16, share_slots_waves=1 << 20)):
+            ops = HipOps(dt, "cuda:0", tuning=tuning)
+            ops._num_cus = 8                      # (more pairs than CUs from three sequences on)
+            seen = []
+            call = ops._call
+            ops._call = lambda stem, name, *args: (seen.append(args) if name.startswith("sl_attention_mfma@") else None,
+                                                   call(stem, name, *args))[1]
+            got = ops.paged_attention(q2, nh, nkv, D, kc, vc, page, tables, batch, scale, window)
+            assert rel_err(got.cpu(), ref) < ATTN_TOL[dt], (lens[:3], tuning.share_slots_growth)
+            if len(lens) * nkv > 8 and len(seen) == 1 and seen[0][17] > 1:
+                # one launch in shares: it is told the step's sums and the wavefronts to aim at
+                slots, merged, stats, aim = seen[0][17], seen[0][-3], seen[0][-2], seen[0][-1]
+                assert not merged and stats.value == batch.ctx_stats.data_ptr()
+                assert aim % (len(lens) * nkv) == 0 and aim // (len(lens) * nkv) <= slots
+                assert slots <= max(aim // (len(lens) * nkv), tuning.share_slots_growth * aim // (len(lens) * nkv))
+                told += 1
+        # without the step's sums: as many shares for every sequence
+        del batch.ctx_stats
+        ops = HipOps(dt, "cuda:0", tuning=Tuning(group_attention_fill=1e9))
+        assert rel_err(ops.paged_attention(q2, nh, nkv, D, kc, vc, page, tables, batch, scale, window).cpu(), ref) < ATTN_TOL[dt]
+    assert told >= 6
 
 
 def test_single_tokens_of_more_pairs_than_cus():
@@ -1020,7 +1070,7 @@ def test_single_tokens_of_more_pairs_than_cus():
     ops._num_cus = 8
     seen = []
     call = ops._call
-    ops._call = lambda stem, name, *args: (seen.append((args[17], args[-1])) if name.startswith("sl_attention_mfma@") else None,
+    ops._call = lambda stem, name, *args: (seen.append((args[17], args[-3])) if name.startswith("sl_attention_mfma@") else None,
                                            call(stem, name, *args))[1]
     for n_seqs, ctx, form in ((4, 700, [(1, 1)]), (5, 3000, [(2, 0)]), (40, 700, [(1, 0)]), (9, 3000, [(1, 1), (46, 0)])):
         seqs = [(ctx - 13 * i, 1) for i in range(n_seqs)]
