@@ -489,34 +489,45 @@ __device__ __forceinline__ int share_count(const AttnParams& P, int nblk) {
 // One wavefront per workgroup; operands straight from the pages.  Used for
 // decode tokens (SPLIT: the wavefront takes one share of the key blocks) and
 // for prompt portions whose launch does not saturate L2.
-template <int NB, bool SPLIT, bool FOLD, bool PAIRS = false>
+template <int NB, bool SPLIT, bool FOLD, bool PAIRS = false, bool ONE_LENGTH = false>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB * D <= 256 ? 2 : 1))) void attention_mfma_kernel(const AttnParams P) {
   const int lane = threadIdx.x, n = lane & 15, gq = lane >> 4;
-  // Split single tokens come as a one-dimensional grid: all (sequence, kv head) pairs of share 0, then those
-  // of share 1, .., the pairs counted up to a multiple of 8 and, within each eight, rotated by the share.
-  // (and by the number of the eight, so that sequences a multiple of 8 apart do not share a chiplet either).
-  // Workgroups go to the eight chiplets in turn, so workgroup L runs on chiplet L % 8 = (pair + share + pair / 8) % 8:
-  // the shares of one pair go round the chiplets (a long sequence among short ones loads them all), and
-  // so do the pairs of one share (a sequence may use the first few shares only: with the share as the
-  // fastest index, eight slots and two shares in use, two chiplets did all the work).
-  const int pairs = P.nkv * P.num_seqs, pairs8 = (pairs + 7) & ~7;
-  const int share_of = SPLIT ? blockIdx.x / pairs8 : 0, place = SPLIT ? blockIdx.x % pairs8 : 0;
-  const int pair_of = (place & ~7) | ((place - share_of - (place >> 3)) & 7);
-  if (SPLIT && pair_of >= pairs) return;
-  const int seq = P.seq_begin + (SPLIT ? pair_of / P.nkv : (int)blockIdx.z);
-  const int kvh = SPLIT ? pair_of % P.nkv : (int)blockIdx.y;
+  // Split single tokens come as a grid of (kv head, sequence, share), which is handed out as all (sequence,
+  // kv head) pairs of share 0, then those of share 1, ...  Workgroups go to the eight chiplets in turn
+  // (workgroup L to chiplet L % 8), and both the shares of one pair and the pairs of one share should go
+  // round them: a long sequence among short ones then loads all chiplets, and so do sequences that use only
+  // the first few of their shares (with the share as the fastest index, eight slots and two shares in use,
+  // two chiplets did all the work).  With a number of pairs that is no multiple of 8 the order does that by
+  // itself (each share begins pairs % 8 chiplets further on); with a multiple of 8 the pairs of every eight
+  // are rotated by the share and by the number of the eight, so that workgroup L is a pair with
+  // (pair + share + pair / 8) % 8 = L % 8.  (No places are left empty to make eights: a workgroup that leaves
+  // at once still takes its turn in the order in which a chiplet hands workgroups to its CUs, and with 4
+  // pairs, one request of the 7B shape, half the CUs then got two wavefronts and half none: 12.0 against
+  // 9.8 us a layer.)  Nothing here may stand between the kernel's arguments and its first read of memory
+  // that need not: with one request the launch is a chain of five trips to memory and little else.
+  int seq = P.seq_begin + blockIdx.y, kvh = SPLIT ? blockIdx.x : blockIdx.y;
+  if (!SPLIT) seq = P.seq_begin + blockIdx.z;
+  if (SPLIT && (gridDim.x * gridDim.y) % 8 == 0) {
+    const int place = blockIdx.x + gridDim.x * blockIdx.y;
+    const int pair_of = (place & ~7) | ((place - (int)blockIdx.z - (place >> 3)) & 7);
+    seq = P.seq_begin + pair_of / (int)gridDim.x;
+    kvh = pair_of % (int)gridDim.x;
+  }
   const int g = P.nh / P.nkv;
   const int q0 = P.cu_q[seq];
   const int qlen = P.cu_q[seq + 1] - q0;
   const int ncols = qlen * g;
   const int ntiles = (ncols + 16 * NB - 1) / (16 * NB);
-  const int tile_rev = SPLIT ? 0 : blockIdx.x / P.nsplit, split = SPLIT ? share_of : blockIdx.x % P.nsplit;
+  const int tile_rev = SPLIT ? 0 : blockIdx.x / P.nsplit, split = SPLIT ? blockIdx.z : blockIdx.x % P.nsplit;
   if (tile_rev >= ntiles) return;
   const int tile = ntiles - 1 - tile_rev;          // long (late) tiles first
   const int pos0 = P.positions[q0];
   const int* table = P.block_tables + (size_t)seq * P.max_pages;
   int shares = P.nsplit;
-  if (SPLIT) {
+  if (SPLIT && ONE_LENGTH) {
+    // (a kernel of its own: the count needs the token's position, and a wavefront that has to wait for it
+    // before it may ask for its queries starts a trip to memory later, 1.6 us of the 9.8 of a launch for one
+    // request of the 7B shape at 4,096 keys)
     // (a single token: the blocks from its window's first key to its own position, as Columns::init finds them)
     const int kmin = P.window > 0 && pos0 - P.window + 1 > 0 ? pos0 - P.window + 1 : 0;
     shares = share_count(P, pos0 / 32 + 1 - kmin / 32);
@@ -864,8 +875,11 @@ void attention_mfma_shared_kernel(const AttnParams P) {
 // out[row, head, :] = sum_j w_j o_j / sum_j w_j l_j,  w_j = exp(m_j - max m).
 // One wavefront per (row, head); lane j takes the (m, l) of splits j, j + 64, ..., so
 // nsplit <= 64 * COMBINE_PER_LANE; then the lanes split the channels and sum the partial
-// outputs with the loads of eight splits in flight at a time.
+// outputs with the loads of eight splits in flight at a time.  SKIP: shares of weight 0 wrote no
+// output, and what lies in their place may be anything (a kernel of its own: the test costs the
+// plain one 1.9 of its 5.4 us for one request of the 7B shape in 16 shares).
 constexpr int COMBINE_PER_LANE = 4;
+template <bool SKIP>
 __global__ __launch_bounds__(64) void attention_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int nsplit, int nh,
     int part_row0, __bf16* __restrict__ out, int out_rows) {
@@ -904,9 +918,9 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
 #pragma unroll
       for (int u = 0; u < 8; ++u) v[u] = po[(size_t)(j + u) * D + d];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) acc += ws[j + u] != 0.f ? ws[j + u] * v[u] : 0.f;     // (a share without keys wrote no output)
+      for (int u = 0; u < 8; ++u) acc += SKIP && ws[j + u] == 0.f ? 0.f : ws[j + u] * v[u];
     }
-    for (; j < nsplit; ++j) acc += ws[j] != 0.f ? ws[j] * po[(size_t)j * D + d] : 0.f;
+    for (; j < nsplit; ++j) acc += SKIP && ws[j] == 0.f ? 0.f : ws[j] * po[(size_t)j * D + d];
     out[out_index(out_rows, nh, (size_t)(part_row0 + r), h * D + d)] = (__bf16)(acc * inv);
   }
 }
@@ -971,24 +985,32 @@ extern "C" const char* sl_attention_mfma(
              "attention_mfma: a split launch needs partial buffers for its rows");
     SL_CHECK(g <= 64, "attention_mfma: more than 64 query heads per kv head");
     SL_CHECK(nsplit <= 64 * COMBINE_PER_LANE, "attention_mfma: too many splits of the context");
-    const long long pairs8 = ((long long)nkv * num_seqs + 7) / 8 * 8;
-    SL_CHECK(nsplit * pairs8 < (1ll << 31), "attention_mfma: too many shares");
-    const dim3 grid((unsigned)(nsplit * pairs8));
+    SL_CHECK(num_seqs <= 65535 && nsplit <= 65535, "attention_mfma: too many sequences in a split launch");
+    const dim3 grid(nkv, num_seqs, nsplit);
+    const bool one_length = ctx_stats != nullptr && share_waves > 0;
     P.ctx_stats = ctx_stats;
     P.share_waves = share_waves;
+#define SL_SPLIT(NB_, FOLD_, PAIRS_)                                                                  \
+  do {                                                                                                \
+    if (one_length) attention_mfma_kernel<NB_, true, FOLD_, PAIRS_, true><<<grid, 64, 0, stream>>>(P); \
+    else attention_mfma_kernel<NB_, true, FOLD_, PAIRS_, false><<<grid, 64, 0, stream>>>(P);           \
+  } while (0)
     if (fold) {
-      if (g <= 16) attention_mfma_kernel<1, true, true, true><<<grid, 64, 0, stream>>>(P);
-      else if (g <= 32) attention_mfma_kernel<2, true, true><<<grid, 64, 0, stream>>>(P);
-      else attention_mfma_kernel<4, true, true><<<grid, 64, 0, stream>>>(P);
+      if (g <= 16) SL_SPLIT(1, true, true);
+      else if (g <= 32) SL_SPLIT(2, true, false);
+      else SL_SPLIT(4, true, false);
     } else {
-      if (g <= 16) attention_mfma_kernel<1, true, false><<<grid, 64, 0, stream>>>(P);
-      else if (g <= 32) attention_mfma_kernel<2, true, false><<<grid, 64, 0, stream>>>(P);
-      else attention_mfma_kernel<4, true, false><<<grid, 64, 0, stream>>>(P);
+      if (g <= 16) SL_SPLIT(1, false, false);
+      else if (g <= 32) SL_SPLIT(2, false, false);
+      else SL_SPLIT(4, false, false);
     }
+#undef SL_SPLIT
     const char* e = sl_launch_status();
     if (e) return e;
-    attention_combine_kernel<<<dim3(num_seqs, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh,
-                                                                  part_row0, (__bf16*)out, out_rows);
+    if (one_length) attention_combine_kernel<true><<<dim3(num_seqs, nh), 64, 0, stream>>>(
+        part_o, part_ml, nsplit, nh, part_row0, (__bf16*)out, out_rows);
+    else attention_combine_kernel<false><<<dim3(num_seqs, nh), 64, 0, stream>>>(
+        part_o, part_ml, nsplit, nh, part_row0, (__bf16*)out, out_rows);
     return sl_launch_status();
   }
   // Prompt portions.  The workgroups that share a block through LDS, or one
@@ -1040,7 +1062,7 @@ extern "C" const char* sl_attention_mfma(
     if (nsplit > 1) {
       const char* e = sl_launch_status();
       if (e) return e;
-      attention_combine_kernel<<<dim3(part_rows, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh,
+      attention_combine_kernel<false><<<dim3(part_rows, nh), 64, 0, stream>>>(part_o, part_ml, nsplit, nh,
                                                                     part_row0, (__bf16*)out, out_rows);
     }
   }
