@@ -104,7 +104,8 @@ struct AttnParams {
   int pair;                      // prompt workgroups take a late tile and its early mirror
   int out_rows;                  // 0: out is [T, nh * D]; else its rows are laid out by k-step for the few-rows
                                  // product that reads them: element (t, c) at (c / 32) * (out_rows * 32) + t * 32 + c % 32
-  int by_chiplet;                // a one-dimensional grid laid out by Place below (else x: workgroup of a pair, y: kv head, z: sequence)
+  int by_chiplet;                // a one-dimensional grid laid out by Place below (else x: workgroup of a pair, y: kv head, z: sequence;
+                                 // split single tokens: x: kv head, y: sequence, z: share)
   int grid_x, num_seqs;          // ... its extent per (sequence, kv head) pair, and the sequences
   // Split single tokens: shares of one length for all sequences of the launch instead of nsplit shares each (see
   // share_count).  ctx_stats: the sum and the largest of the launch's context lengths, on the device (they change from
