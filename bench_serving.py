@@ -150,6 +150,15 @@ def summarise(done: list, elapsed: float, ttft_slo_ms: float, tpot_slo_ms: float
     }
 
 
+class AsksFor:
+    """The output-length predictor of the policy "sjf-predicted" for this load: every request
+    generates exactly the tokens it asks for (eos is ignored), so the prediction is exact
+    (the "oracle" of examples/run_simulator.py:56-58)."""
+
+    def predict_remaining(self, req) -> int:
+        return req.params.max_tokens
+
+
 def build_engine(args):
     from servelab_amd import CacheConfig, LLMEngine, SchedulerConfig, load_config
     from servelab_amd.cli import tune_option
@@ -160,7 +169,8 @@ def build_engine(args):
                             chunked_prefill=not args.no_chunked_prefill,
                             policy=args.scheduler_policy)
     warm = dict(tune_products=tune_option(args), capture_graphs_up_to=args.capture_graphs_up_to,
-                run_ahead=not args.no_run_ahead)
+                run_ahead=not args.no_run_ahead,
+                predictor=AsksFor() if args.scheduler_policy == "sjf-predicted" else None)
     if args.model:
         cfg = load_config(args.model)
         return cfg, LLMEngine(cfg, cache, sched, dtype=args.dtype, **warm)
@@ -226,7 +236,8 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-num-seqs", type=int, default=64)
     ap.add_argument("--max-batched-tokens", type=int, default=2048)
     ap.add_argument("--no-chunked-prefill", action="store_true")
-    ap.add_argument("--scheduler-policy", default="fcfs", choices=["fcfs", "priority"])
+    ap.add_argument("--scheduler-policy", default="fcfs", choices=["fcfs", "priority", "sjf-predicted"],
+                    help="sjf-predicted: fewest tokens still to come first, the output lengths being known here")
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
     ap.add_argument("--ttft-slo-ms", type=float, default=2000)
     ap.add_argument("--tpot-slo-ms", type=float, default=50)

@@ -30,14 +30,14 @@ class SchedulerConfig:
     max_num_seqs: int = 64
     max_num_batched_tokens: int = 2048
     chunked_prefill: bool = True
-    policy: str = "fcfs"                   # fcfs | priority
+    policy: str = "fcfs"                   # fcfs | priority | sjf-predicted (needs the engine's predictor)
 
     def __post_init__(self):
         if self.max_num_seqs < 1:
             raise ValueError("max_num_seqs must be >= 1")
         if self.max_num_batched_tokens < 1:
             raise ValueError("max_num_batched_tokens must be >= 1")
-        if self.policy not in ("fcfs", "priority"):
+        if self.policy not in ("fcfs", "priority", "sjf-predicted"):
             raise ValueError(f"unknown scheduler policy: {self.policy}")
 
 

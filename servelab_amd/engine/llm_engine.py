@@ -67,7 +67,7 @@ class _Flight:
 class LLMEngine:
     def __init__(self, model_config, cache_config: Optional[CacheConfig] = None,
                  scheduler_config: Optional[SchedulerConfig] = None, seed: int = 1234,
-                 device: str = "cuda:0", tokenizer=None,
+                 device: str = "cuda:0", tokenizer=None, predictor=None,
                  clock: Optional[Callable[[], float]] = None, dtype: str = "auto",
                  model=None, ops=None, tune_products=False, random_weights: Optional[int] = None,
                  capture_graphs_up_to: int = 0, run_ahead: bool = True):
@@ -79,7 +79,10 @@ class LLMEngine:
         step sizes (rows) to time the library's matrix kernels for.
         ``capture_graphs_up_to``: a context length up to which the decode graphs
         of 1..max_num_seqs requests are captured now rather than when a request
-        first needs them."""
+        first needs them.  ``predictor``: an object with
+        ``predict_remaining(request) -> int``, the number of tokens a request
+        will generate, for the policy "sjf-predicted"
+        (servelab/engine/engine.py:51,131)."""
         self.model_config = model_config
         self.cache_config = cache_config or CacheConfig()
         self.scheduler_config = scheduler_config or SchedulerConfig()
@@ -127,7 +130,7 @@ class LLMEngine:
                 range(1, self.scheduler_config.max_num_seqs + 1), capture_graphs_up_to)
         self.scheduler = Scheduler(self.scheduler_config, self.runner.manager, self.clock,
                                    eos_token_id=model.spec.eos_token_id,
-                                   max_positions=model.spec.max_position_embeddings)
+                                   max_positions=model.spec.max_position_embeddings, predictor=predictor)
         self.sampler = Sampler(model.rt.ops, self.device, seed)
         self.run_ahead = bool(run_ahead)
         self._flight: Optional[_Flight] = None

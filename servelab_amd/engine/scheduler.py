@@ -46,7 +46,32 @@ def priority_key(req: Request):
     return (req.priority, req.times.arrived, req.number)
 
 
+def shortest_predicted_key(predictor):
+    """Fewest predicted tokens still to come first (servelab/engine/scheduler.py:51-70).
+    ``predictor.predict_remaining(request)`` says how many tokens the request
+    will generate in all (servelab/engine/scheduler.py:19-22); what it has
+    generated already is taken off, also for a request that lost its cache
+    to a preemption and keeps its tokens (the reference takes it off only
+    once the prompt has run, and forgets it after a preemption)."""
+    def key(req: Request):
+        remaining = int(predictor.predict_remaining(req)) - req.num_output
+        return (max(1, remaining), req.times.arrived, req.number)
+    return key
+
+
 POLICIES = {"fcfs": fcfs_key, "priority": priority_key}
+PREDICTED_POLICY = "sjf-predicted"
+
+
+def policy_key(name: str, predictor=None):
+    """The sort key of a policy by name (servelab/engine/scheduler.py:74-83)."""
+    if name == PREDICTED_POLICY:
+        if predictor is None:
+            raise ValueError("sjf-predicted policy requires an output-length predictor")
+        return shortest_predicted_key(predictor)
+    if name not in POLICIES:
+        raise ValueError(f"unknown scheduler policy: {name}")
+    return POLICIES[name]
 
 
 @dataclass
@@ -90,13 +115,13 @@ class Plan:
 
 class Scheduler:
     def __init__(self, config: SchedulerConfig, manager, clock: Callable[[], float],
-                 eos_token_id: int = -1, max_positions: Optional[int] = None):
+                 eos_token_id: int = -1, max_positions: Optional[int] = None, predictor=None):
         self.cfg = config
         self.manager = manager
         self.clock = clock
         self.eos_token_id = eos_token_id
         self.max_positions = max_positions
-        self.key = POLICIES[config.policy]
+        self.key = policy_key(config.policy, predictor)
         self.queue: List[Request] = []
         self.active: List[Request] = []
         self.num_preemptions = 0

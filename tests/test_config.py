@@ -100,6 +100,7 @@ def test_engine_configs_validate():
     with pytest.raises(ValueError):
         CacheConfig(block_size=24)
     with pytest.raises(ValueError):
-        SchedulerConfig(policy="sjf-predicted")
+        SchedulerConfig(policy="shortest")
+    assert SchedulerConfig(policy="sjf-predicted").policy == "sjf-predicted"     # (servelab/config.py:93)
     with pytest.raises(ValueError):
         SchedulerConfig(max_num_seqs=0)

@@ -14,11 +14,12 @@ from tiny_configs import make_folder
 
 
 def make_engine(folder, num_blocks=64, max_batched=256, max_seqs=8, block_size=16, chunked=True,
-                policy="fcfs", run_ahead=True):
+                policy="fcfs", run_ahead=True, predictor=None):
     return LLMEngine(load_config(folder), CacheConfig(block_size=block_size, num_blocks=num_blocks),
                      SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched,
                                      chunked_prefill=chunked, policy=policy),
-                     device="cpu", dtype="float32", ops=EmulatedOps(), run_ahead=run_ahead)
+                     device="cpu", dtype="float32", ops=EmulatedOps(), run_ahead=run_ahead,
+                     predictor=predictor)
 
 
 PROMPTS = [list(range(10, 40)), [5, 9, 200, 31], list(range(300, 377)), [7]]
@@ -108,6 +109,27 @@ def test_priority_policy_serves_the_smaller_value_first(folder_and_plain):
             order.append(out.request_id)
             done[out.request_id] = out.outputs[0].token_ids
     assert order == [ids[1], ids[3], ids[2], ids[0]]
+    assert [done[i] for i in ids] == want
+
+
+def test_predicted_shortest_job_first_through_the_engine(folder_and_plain):
+    # servelab/engine/engine.py:51,131: the engine hands its predictor to the scheduler
+    folder, want = folder_and_plain
+
+    class ByPromptLength:
+        def predict_remaining(self, req):
+            return req.prompt_len
+
+    with pytest.raises(ValueError, match="requires an output-length predictor"):
+        make_engine(folder, policy="sjf-predicted")
+    eng = make_engine(folder, policy="sjf-predicted", max_seqs=1, predictor=ByPromptLength())
+    ids = [eng.add_request(prompt_token_ids=p, sampling_params=SamplingParams.greedy(12)) for p in PROMPTS]
+    order, done = [], {}
+    while eng.has_unfinished():
+        for out in eng.step():
+            order.append(out.request_id)
+            done[out.request_id] = out.outputs[0].token_ids
+    assert order == [ids[3], ids[1], ids[0], ids[2]]          # prompts of 1, 4, 30 and 77 tokens
     assert [done[i] for i in ids] == want
 
 

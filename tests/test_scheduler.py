@@ -21,7 +21,7 @@ class Driver:
     'samples' token 7, and checks the invariants after every step."""
 
     def __init__(self, num_pages=16, page_size=4, max_batched=32, max_seqs=8, policy="fcfs",
-                 chunked=True, eos=-1, max_positions=None, window=None):
+                 chunked=True, eos=-1, max_positions=None, window=None, predictor=None):
         self.clock = FakeClock()
         specs = {0: PagedKVSpec(1, 16, None)}
         if window:
@@ -30,7 +30,7 @@ class Driver:
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched,
                             chunked_prefill=chunked, policy=policy),
-            self.manager, self.clock, eos_token_id=eos, max_positions=max_positions)
+            self.manager, self.clock, eos_token_id=eos, max_positions=max_positions, predictor=predictor)
         self.finished, self.aborted, self.n, self.plans = [], [], 0, []
         self.token = 7
 
@@ -122,6 +122,47 @@ def test_fcfs_and_priority_order():
     d.submit("low", 20, 1, priority=5)
     d.submit("high", 20, 1, priority=0)
     assert d.scheduler.schedule().portions[0].request.request_id == "high"
+
+
+class KnowsTheLength:
+    """The predictor of the policy "sjf-predicted": here it knows what each request asks for."""
+
+    def predict_remaining(self, req):
+        return req.params.max_tokens
+
+
+def test_shortest_predicted_job_first():
+    # servelab/engine/scheduler.py:51-70,79-81
+    with pytest.raises(ValueError, match="requires an output-length predictor"):
+        Driver(policy="sjf-predicted")
+    with pytest.raises(ValueError, match="unknown scheduler policy"):
+        SchedulerConfig(policy="shortest")
+    d = Driver(max_batched=8, max_seqs=2, policy="sjf-predicted", predictor=KnowsTheLength())
+    d.submit("long", 8, 9)
+    d.submit("short", 8, 2)
+    d.submit("middle", 8, 5)
+    # admission: the shortest predicted output first, whatever the order of arrival
+    assert [p.request.request_id for p in d.step().portions] == ["short"]
+    assert [p.request.request_id for p in d.step().portions] == ["middle"]
+    d.step()
+    d.step()
+    # what a request has generated counts off its prediction: "middle" (5 predicted, 2 made) now goes
+    # before a fresh request that predicts 4, and the victim of a preemption is the one with most to come
+    key = d.scheduler.key
+    middle = next(r for r in d.scheduler.active if r.request_id == "middle")
+    fresh = Request("fresh", [1, 2], SamplingParams(max_tokens=4), arrived=d.clock.t, number=99)
+    assert middle.num_output == 2 and key(middle) < key(fresh)
+    d.run()
+    assert [r.request_id for r in d.finished] == ["short", "middle", "long"]
+    # equal predictions: first come first served; a prediction at or below what is made counts as 1
+    a = Request("a", [1], SamplingParams(max_tokens=3), arrived=1.0, number=1)
+    b = Request("b", [1], SamplingParams(max_tokens=3), arrived=0.5, number=2)
+    assert key(b) < key(a)
+    a.cached = 1
+    for _ in range(5):
+        a.sampled(7, 2.0)
+        a.cached += 1
+    assert key(a)[0] == 1
 
 
 def test_request_numbers_not_id_strings_break_ties():
