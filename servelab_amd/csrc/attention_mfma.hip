@@ -876,7 +876,7 @@ void attention_mfma_shared_kernel(const AttnParams P) {
 // out[row, head, :] = sum_j w_j o_j / sum_j w_j l_j,  w_j = exp(m_j - max m).
 // One wavefront per (row, head); lane j takes the (m, l) of splits j, j + 64, ..., so
 // nsplit <= 64 * COMBINE_PER_LANE; then the lanes split the channels and sum the partial
-// outputs with the loads of eight splits in flight at a time.  SKIP: shares of weight 0 wrote no
+// outputs, share after share.  SKIP: shares of weight 0 wrote no
 // output, and what lies in their place may be anything (a kernel of its own: the test costs the
 // plain one 1.9 of its 5.4 us for one request of the 7B shape in 16 shares).
 constexpr int COMBINE_PER_LANE = 4;
@@ -911,18 +911,36 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(
   __syncthreads();
   const float inv = 1.f / denom;
   const float* po = part_o + base * D;
-  for (int d = lane; d < D; d += 64) {
-    float acc = 0.f;
-    int j = 0;
-    for (; j + 8 <= nsplit; j += 8) {
-      float v[8];
+  // A lane takes channels lane, lane + 64, ...; the partial outputs of sixteen shares are asked for
+  // together, all channels of a lane at once (a batch is a trip to memory: with eight shares a batch
+  // and the channels one after the other, 64 shares took 2 us longer than 32; with the last shares
+  // below a whole batch one by one, 21 took 3 us longer than 16 or 24).  Added in the order of the
+  // shares, whatever the batches.
+  constexpr int DI = (D + 63) / 64, BATCH = 16;
+  float acc[DI];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = po[(size_t)(j + u) * D + d];
+  for (int di = 0; di < DI; ++di) acc[di] = 0.f;
+  for (int j = 0; j < nsplit; j += BATCH) {
+    float v[BATCH][DI];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) acc += SKIP && ws[j + u] == 0.f ? 0.f : ws[j + u] * v[u];
+    for (int u = 0; u < BATCH; ++u) {
+      const float* row = po + (size_t)(j + u < nsplit ? j + u : nsplit - 1) * D;
+#pragma unroll
+      for (int di = 0; di < DI; ++di) v[u][di] = 64 * di + 64 <= D || lane + 64 * di < D ? row[lane + 64 * di] : 0.f;
     }
-    for (; j < nsplit; ++j) acc += SKIP && ws[j] == 0.f ? 0.f : ws[j] * po[(size_t)j * D + d];
-    out[out_index(out_rows, nh, (size_t)(part_row0 + r), h * D + d)] = (__bf16)(acc * inv);
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      // (no branch here: under one the compiler may move each load down to its use; beyond the last share the
+      // weight is 0 and the value that of the last share)
+      const float w = j + u < nsplit ? ws[j + u] : 0.f;
+#pragma unroll
+      for (int di = 0; di < DI; ++di) acc[di] += SKIP && w == 0.f ? 0.f : w * v[u][di];
+    }
+  }
+#pragma unroll
+  for (int di = 0; di < DI; ++di) {
+    const int d = lane + 64 * di;
+    if (d < D) out[out_index(out_rows, nh, (size_t)(part_row0 + r), h * D + d)] = (__bf16)(acc[di] * inv);
   }
 }
 

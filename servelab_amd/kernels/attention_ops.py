@@ -281,22 +281,31 @@ class AttentionOps:
             self._lib[key] = lib
         return key
 
-    def _decode_shares(self, units, most) -> int:
-        """Into how many shares the keys of each of ``units`` (request, kv head) pairs are cut, ``most`` at
-        most.  A share is a wavefront, and a wavefront streams its keys at the pace of its round trips to
-        memory, so the launch takes what its busiest CU holds: TARGET_WAVES wavefronts (two a CU) are best,
-        and a launch slightly above a whole number of wavefronts per CU is the worst (7B shape, contexts of
-        4,096: 14 requests in 10 shares, 560 wavefronts: 30.6 us a layer; in 9, 504 wavefronts: about 22 us;
-        24 requests 576 against 480 wavefronts: 4.73 against 4.40 ms a step; 48 requests 384 / 576 / 768
-        wavefronts: 5.62 / 5.77 / 5.49 ms).  Taken: the count whose wavefronts fill their rounds over the CUs
-        best, less a fifth of its relative distance from the target; no more than half again the target."""
-        cus, target = self._num_cus, self.TARGET_WAVES
-        best, best_score = 1, None
-        for shares in range(1, max(1, min(most, (3 * target // 2) // units)) + 1):
+    def _decode_shares(self, units, most, blocks, D) -> int:
+        """Into how many shares the ``blocks`` key blocks of each of ``units`` (request, kv head) pairs, no
+        more pairs than CUs, are cut, ``most`` at most: the count with the lowest estimate of the launch's
+        time, fewest shares first among equals.  A share is a wavefront; it asks for two blocks at a time,
+        so its keys take ceil(blocks of the longest share / 2) trips to memory (FEW_TRIP_US each), unless
+        the stream of all keys and values through the fullest CU takes longer (a launch takes what its
+        busiest CU holds: 7B shape, contexts of 4,096, 14 requests in 10 shares, 560 wavefronts on 256
+        CUs: 30.6 us a layer; in 9, 504 wavefronts: about 22 us); every wavefront a CU costs FEW_WAVE_US,
+        and the combine kernel reads the partial results sixteen shares at a time, FEW_BATCH_US a batch.
+        Fitted to 1,500 launches of 1 to 24 requests of the 7B shape at contexts of 512 to 32,768 (mean
+        error 4 %); the count taken costs 0.7 % more than the best measured one on average and 7 % at worst.
+        (Filling whole rounds of the CUs near two wavefronts each, the rule before: 1.1 % and 18 %: it took
+        128 shares for one request at 8,192 to 16,384 keys where 64 are faster, 12.0 against 10.2 us, and
+        fewer than the context allows at 512 and 1,024 keys, where one trip beats full rounds.)"""
+        cus = self._num_cus
+        stream = units * blocks * 32 * D * 4 / (self.FEW_STREAM_GBS_PER_CU * 1e3 * cus)       # us for K and V
+        best, lowest = 1, None
+        for shares in range(1, max(1, min(most, 8 * cus // units)) + 1):
             waves = units * shares
-            score = waves / (-(-waves // cus) * cus) - 0.2 * abs(waves - target) / target
-            if best_score is None or score > best_score + 1e-9:
-                best, best_score = shares, score
+            trips = -(-(-(-blocks // shares)) // 2)
+            t = max(self.FEW_TRIP_US * trips, stream * (-(-waves // cus) * cus / waves)) + self.FEW_WAVE_US * waves / cus
+            if shares > 1:
+                t += self.FEW_BATCH_US * -(-shares // 16) + self.MANY_COMBINE_US
+            if lowest is None or t < lowest - 1e-9:
+                best, lowest = shares, t
         return best
 
     def _decode_many(self, pairs, blocks, D, merged_fits, most):
@@ -329,7 +338,7 @@ class AttentionOps:
         no partial results in memory and no second kernel.  With fewer pairs that would leave a
         pair's keys to the one CU that runs its workgroup, and a CU pulls 50 GB/s whatever is in
         flight (7B shape, contexts of 4,096, 8 requests: 61 us against 16 us): then a wavefront of a
-        workgroup of its own takes a share, shares enough for TARGET_WAVES wavefronts spread over all
+        workgroup of its own takes a share, as many shares as ``_decode_shares`` estimates to be fastest, spread over all
         CUs, and the combine kernel merges them (a few requests with long contexts: up to 256 shares;
         one request at 32,000 tokens: 64 shares leave one wavefront per CU).  Short contexts merge in
         the workgroup from half as many pairs on.  More pairs than CUs: one launch in the form
@@ -342,7 +351,7 @@ class AttentionOps:
         def few(n):
             need = self.GROUP_ATTENTION_FILL * cus
             merged = merged_fits and (n * nkv >= need or (2 * n * nkv >= need and blocks <= self.GROUP_ATTENTION_SHORT_BLOCKS))
-            return merged, 1 if merged else self._decode_shares(n * nkv, min(most, blocks // 2))
+            return merged, 1 if merged else self._decode_shares(n * nkv, min(most, blocks // 2), blocks, D)
 
         if pairs <= cus:
             return [(0, n_dec) + few(n_dec)]

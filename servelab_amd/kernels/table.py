@@ -26,7 +26,7 @@ class KernelTable:
     # ``plan_weights(total_bytes)`` picks "dual" while two copies stay below
     # DUAL_MEMORY_SHARE of the device's memory, else "tiled".
     #
-    # The numbers that choose between kernels (DUAL_MEMORY_SHARE, WIDE_MIN_M, MID_*, TARGET_WAVES,
+    # The numbers that choose between kernels (DUAL_MEMORY_SHARE, WIDE_MIN_M, MID_*, FEW_*, MANY_*,
     # SHARED_ATTENTION_*, ...) are the fields of ``tuning.Tuning``, set on the table at construction.
 
     def __init__(self, act_dtype: torch.dtype, device="cuda:0", tuning: Optional[Tuning] = None):

@@ -4,9 +4,9 @@ Kernel *limits* (how many rows a kernel can take, which head sizes) stay with
 the kernels' wrappers in the kernel table (``*_ops.py``): they are facts of the code.  What is here
 are *choices* that were measured on one MI355X with the projection sizes of the
 Qwen2.5 7B, 32B and 72B shapes; another GPU or another architecture's sizes may
-want others.  ``HipOps(dtype, device, tuning=Tuning(target_waves=...))`` takes a
+want others.  ``HipOps(dtype, device, tuning=Tuning(wide_min_m=...))`` takes a
 changed set; every field becomes an attribute of the kernel table under its
-upper-case name (``ops.TARGET_WAVES``), which is what the routing code reads.
+upper-case name (``ops.WIDE_MIN_M``), which is what the routing code reads.
 """
 from dataclasses import dataclass, fields
 
@@ -97,8 +97,14 @@ class Tuning:
     # ---- attention
     # wavefronts a decode launch of the general (float32) kernel aims for when it splits the context
     general_attention_waves: int = 4096
-    # the same for the matrix-core kernel (384, 768 and 1,024 measured within noise or slower)
-    target_waves: int = 512
+    # single tokens of no more (request, kv head) pairs than CUs, a wavefront per share of a pair's keys:
+    # the estimate of a launch's time that picks the number of shares (HipOps._decode_shares): a trip
+    # to memory of a wavefront (two key blocks), the rate at which a CU streams keys and values, a
+    # wavefront more on every CU, and a batch of sixteen partial results in the combine kernel
+    few_trip_us: float = 1.675
+    few_stream_gbs_per_cu: float = 28.05
+    few_wave_us: float = 0.922
+    few_batch_us: float = 0.463
     # single tokens, no more (request, kv head) pairs than CUs: with this many pairs per CU, a workgroup of eight
     # wavefronts takes a pair's keys and merges in LDS; below, a wavefront takes a share and a second kernel merges
     # (7B shape, a layer: contexts of 4,096, 64 / 128 requests: 89.7 / 177 against 91.1 / 209 us, 32 requests

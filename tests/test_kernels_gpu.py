@@ -889,15 +889,23 @@ def test_attention_over_random_batches(seed):
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt], (nh, nkv, D, page, window, seqs)
 
 
-def test_decode_shares_fill_whole_rounds_over_the_cus():
-    """The number of shares of a request's keys at the batch sizes it was measured at (4 kv heads, 256 CUs,
-    contexts of 4,096: 64 shares at most): never slightly more wavefronts than a whole number per CU."""
+def test_decode_shares_by_the_estimate_of_the_launch():
+    """The number of shares of a request's keys at sizes it was measured at (4 kv heads, head size 128, 256
+    CUs): never slightly more wavefronts than a whole number per CU where the stream of keys decides; one
+    trip to memory a share where the context is short; no more shares than the combine kernel's batches
+    are worth for one request with a long context."""
     from servelab_amd.kernels import HipOps
     ops = HipOps(torch.bfloat16, "cuda:0")
     ops._num_cus = 256
-    shares = {b: ops._decode_shares(4 * b, 64) for b in (1, 8, 14, 16, 17, 24, 48, 64, 128, 200)}
-    assert shares == {1: 64, 8: 16, 14: 9, 16: 8, 17: 7, 24: 5, 48: 4, 64: 2, 128: 1, 200: 1}
-    assert ops._decode_shares(4, 1) == 1 and ops._decode_shares(4, 256) == 128
+    at = lambda requests, ctx: ops._decode_shares(4 * requests, min(256, max(1, ctx // 64)), -(-ctx // 32), 128)
+    assert {b: at(b, 4096) for b in (1, 2, 4, 8, 14, 16, 24, 48, 64)} == \
+        {1: 64, 2: 32, 4: 32, 8: 16, 14: 9, 16: 8, 24: 8, 48: 4, 64: 2}
+    assert {b: at(b, 1024) for b in (1, 5, 7, 8, 12, 16)} == {1: 16, 5: 16, 7: 16, 8: 16, 12: 10, 16: 8}
+    assert {c: at(1, c) for c in (2048, 8192, 16384, 32768)} == {2048: 32, 8192: 64, 16384: 64, 32768: 128}
+    assert ops._decode_shares(4, 1, 128, 128) == 1 and ops._decode_shares(256, 64, 128, 128) == 2
+    for requests in range(1, 65):
+        waves = 4 * requests * at(requests, 4096)
+        assert waves <= 256 or (waves - 1) % 256 >= 128, (requests, waves)      # (no round of the CUs less than half full)
 
 
 def test_whole_prompts_pair_their_tiles_unless_the_rounds_are_uneven():
@@ -1056,7 +1064,7 @@ def test_single_tokens_of_more_pairs_than_cus():
     CU and two, merged in the workgroup where two rounds are nearly full and the context is short, one
     share once there are four wavefronts for every CU), and every form gives the plain result
     (a table told that it has 8 CUs; 4, 5, 40 and 9 requests of 4 kv heads: merged, two shares, one share,
-    and two launches: eight requests, which fill whole rounds, merged and the ninth in 46 shares)."""
+    and two launches: eight requests, which fill whole rounds, merged and the ninth in 4 shares)."""
     from servelab_amd.kernels import HipOps
     dt = torch.bfloat16
     ops, emu = HipOps(dt, "cuda:0"), EmulatedOps(dt)
@@ -1072,7 +1080,7 @@ def test_single_tokens_of_more_pairs_than_cus():
     call = ops._call
     ops._call = lambda stem, name, *args: (seen.append((args[17], args[-3])) if name.startswith("sl_attention_mfma@") else None,
                                            call(stem, name, *args))[1]
-    for n_seqs, ctx, form in ((4, 700, [(1, 1)]), (5, 3000, [(2, 0)]), (40, 700, [(1, 0)]), (9, 3000, [(1, 1), (46, 0)])):
+    for n_seqs, ctx, form in ((4, 700, [(1, 1)]), (5, 3000, [(2, 0)]), (40, 700, [(1, 0)]), (9, 3000, [(1, 1), (4, 0)])):
         seqs = [(ctx - 13 * i, 1) for i in range(n_seqs)]
         qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=ctx)
         qkv, scale = in_units(UNITS[1], qkv, nh, D, 1.0 / math.sqrt(D))
@@ -1093,13 +1101,13 @@ def test_single_tokens_of_more_pairs_than_cus():
 @pytest.mark.parametrize("contexts", [(9000,), (9000, 5000)])
 def test_decode_attention_with_more_shares_than_lanes(nh, nkv, D, page, contexts):
     """One or two requests with long contexts are cut into more than 64 shares (up to 141 here, with a
-    launch that aims at 2,048 wavefronts), of which a lane of the merging wavefront takes several; the key
-    that carries the weight of request 0 lies in a late share."""
+    launch whose estimate counts nothing but the trips to memory), of which a lane of the
+    merging wavefront takes several; the key that carries the weight of request 0 lies in a late share."""
     from servelab_amd.kernels import HipOps, Tuning
     dt = torch.bfloat16
-    ops, emu = HipOps(dt, "cuda:0", tuning=Tuning(target_waves=2048)), EmulatedOps(dt)
+    ops, emu = HipOps(dt, "cuda:0", tuning=Tuning(few_wave_us=0.0, few_batch_us=0.0, few_stream_gbs_per_cu=1e9)), EmulatedOps(dt)
     blocks = -(-max(contexts) // 32)
-    assert 64 < ops._decode_shares(len(contexts) * nkv, min(256, blocks // 2)) <= 141
+    assert 64 < ops._decode_shares(len(contexts) * nkv, min(256, blocks // 2), blocks, D) <= 141
     seqs = [(c, 1) for c in contexts]
     qkv, kc, vc, tables, batch = make_attention_case(dt, nh, nkv, D, page, seqs, seed=21)
     at = 8000

@@ -10,8 +10,8 @@ def test_every_choice_lands_on_the_table_under_its_upper_case_name():
     class Table:
         pass
     t = Table()
-    Tuning(target_waves=64, wide_min_m=33).apply(t)
-    assert t.TARGET_WAVES == 64 and t.WIDE_MIN_M == 33
+    Tuning(few_wave_us=2.5, wide_min_m=33).apply(t)
+    assert t.FEW_WAVE_US == 2.5 and t.WIDE_MIN_M == 33
     assert t.NARROW_ATTENTION_WORKGROUPS == Tuning().narrow_attention_workgroups
     assert {n for n in vars(t)} == {f.name.upper() for f in fields(Tuning)}
 
@@ -23,9 +23,10 @@ def test_a_kernel_table_with_other_choices_gives_the_same_numbers():
     import torch
     from servelab_amd.kernels import HipOps
     a = HipOps(torch.bfloat16, "cuda:0")
-    b = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(target_waves=32, mid_min_elements=1 << 40,
+    b = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(few_wave_us=20.0, mid_min_elements=1 << 40,
                                                        mid_min_elements_many=1 << 40, resident_min_rounds=1 << 20))
-    assert b.TARGET_WAVES == 32 and a.TARGET_WAVES == Tuning().target_waves
+    assert b.FEW_WAVE_US == 20.0 and a.FEW_WAVE_US == Tuning().few_wave_us
+    assert b._decode_shares(32, 64, 128, 128) < a._decode_shares(32, 64, 128, 128)
     g = torch.Generator(device="cuda").manual_seed(0)
     x = torch.randn(40, 1024, device="cuda", generator=g).bfloat16()
     w = (torch.randn(12288, 1024, device="cuda", generator=g) * 0.03).bfloat16()
