@@ -244,9 +244,18 @@ __global__ __launch_bounds__(64) void attention_general_combine_kernel(
   ws[lane] = w;
   __syncthreads();
   act_t* o = out + ((size_t)t * nh + h) * D;
+  // (the partial outputs of sixteen shares are asked for together: one after the other each is a trip to
+  // memory; beyond the last share the weight is 0 and the value that of the last share; added in the
+  // order of the shares)
   for (int d = lane; d < D; d += 64) {
     float a = 0.f;
-    for (int j = 0; j < nsplit; ++j) a += ws[j] * part_o[(base + j) * D + d];
+    for (int j = 0; j < nsplit; j += 16) {
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = part_o[(base + (j + u < nsplit ? j + u : nsplit - 1)) * D + d];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) a += (j + u < nsplit ? ws[j + u] : 0.f) * v[u];
+    }
     o[d] = from_f<act_t>(a / denom);
   }
 }
