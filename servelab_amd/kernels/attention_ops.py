@@ -338,19 +338,19 @@ class AttentionOps:
         no partial results in memory and no second kernel.  With fewer pairs that would leave a
         pair's keys to the one CU that runs its workgroup, and a CU pulls 50 GB/s whatever is in
         flight (7B shape, contexts of 4,096, 8 requests: 61 us against 16 us): then a wavefront of a
-        workgroup of its own takes a share, as many shares as ``_decode_shares`` estimates to be fastest, spread over all
-        CUs, and the combine kernel merges them (a few requests with long contexts: up to 256 shares;
-        one request at 32,000 tokens: 64 shares leave one wavefront per CU).  Short contexts merge in
-        the workgroup from half as many pairs on.  More pairs than CUs: one launch in the form
-        ``_decode_many`` estimates to be the fastest, or two, the sequences that fill whole rounds of
+        workgroup of its own takes a share, as many shares as ``_decode_shares`` estimates to be
+        fastest, spread over all CUs, and the combine kernel merges them (a few requests with long
+        contexts: up to 256 shares; one request at 32,000 tokens: 128).  The shorter the contexts, the
+        fewer pairs it takes for merging in the workgroup to pay (``Tuning.group_attention_from``).
+        More pairs than CUs: one launch in the form ``_decode_many`` estimates to be the fastest, or two, the sequences that fill whole rounds of
         the CUs merged in the workgroup and the others as a launch of few pairs, if the estimates say
         that is faster (the first launch then runs at the rate of a stream, whatever the number of
         sequences)."""
         pairs, cus = n_dec * nkv, self._num_cus
 
         def few(n):
-            need = self.GROUP_ATTENTION_FILL * cus
-            merged = merged_fits and (n * nkv >= need or (2 * n * nkv >= need and blocks <= self.GROUP_ATTENTION_SHORT_BLOCKS))
+            share = next(s for b, s in self.GROUP_ATTENTION_FROM if blocks <= b)
+            merged = merged_fits and n * nkv >= self.GROUP_ATTENTION_FILL * share * cus
             return merged, 1 if merged else self._decode_shares(n * nkv, min(most, blocks // 2), blocks, D)
 
         if pairs <= cus:

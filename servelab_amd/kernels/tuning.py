@@ -105,13 +105,19 @@ class Tuning:
     few_stream_gbs_per_cu: float = 28.05
     few_wave_us: float = 0.922
     few_batch_us: float = 0.463
-    # single tokens, no more (request, kv head) pairs than CUs: with this many pairs per CU, a workgroup of eight
-    # wavefronts takes a pair's keys and merges in LDS; below, a wavefront takes a share and a second kernel merges
-    # (7B shape, a layer: contexts of 4,096, 64 / 128 requests: 89.7 / 177 against 91.1 / 209 us, 32 requests
-    # 76 against 50; contexts of 640, 32 / 64 / 128 requests: 13.8 / 16.9 / 32.2 against 15.1 / 20.0 / 35.8 us,
-    # 16 requests 12.7 against 9.8); contexts of at most short_blocks key blocks from half as many pairs on
+    # single tokens, no more (request, kv head) pairs than CUs: a workgroup of eight wavefronts takes a pair's keys
+    # and merges in LDS (no partial results in memory, no second kernel) once there are group_attention_fill
+    # times the share of group_attention_from pairs a CU, by the length of the longest context in key blocks;
+    # below, a wavefront takes a share and the combine kernel merges.  Merged, a pair's keys come through one
+    # CU, so it pays where contexts are short or nearly every CU has a pair.  7B and 32B shapes, us a layer,
+    # merged against the best number of shares: contexts of 512, 112 / 144 / 256 pairs: 10.9 / 11.3 / 13.4
+    # against 11.2 / 12.8 / 16.3; of 1,024, 128 / 192 / 224 pairs: 18.4 / 22.4 / 23.1 against 16.0 / 21.7 / 25.9;
+    # of 2,048, 192 / 224 / 256 pairs: 41.4 / 42.9 / 45.8 against 37.4 / 45.3 / 47.7; of 4,096, 224 / 240 / 256
+    # pairs: 83.1 / 85.6 / 89.4 against 81.8 / 87.1 / 89.4; of 8,192 and 16,384, 256 pairs: 175 and 345 against
+    # 168 and 329 (a share above 1: never).  Whole decode steps of the 7B shape: 32 requests at 1,024 keys
+    # 3.92 -> 3.84 ms (in shares), 60 at 2,048 keys 4.98 -> 4.81 ms (merged); 48 at 1,024 keys 3.95 ms merged, 4.03 in shares.
     group_attention_fill: float = 1.0
-    group_attention_short_blocks: int = 32
+    group_attention_from: tuple = ((16, 0.45), (32, 0.7), (64, 0.85), (128, 0.97), (1 << 30, 1.01))
     # With more pairs than CUs the form is taken by an estimate of the launch's time, whose constants
     # are fitted to 63 launches of 288 to 1,024 pairs over contexts of 640 to 4,096 (3.5 % rms; the form
     # taken is 0.8 % slower than the best measured one on average, 6 % at worst).  The keys and values
