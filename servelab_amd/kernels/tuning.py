@@ -114,10 +114,12 @@ class Tuning:
     # against 11.2 / 12.8 / 16.3; of 1,024, 128 / 192 / 224 pairs: 18.4 / 22.4 / 23.1 against 16.0 / 21.7 / 25.9;
     # of 2,048, 192 / 224 / 256 pairs: 41.4 / 42.9 / 45.8 against 37.4 / 45.3 / 47.7; of 4,096, 224 / 240 / 256
     # pairs: 83.1 / 85.6 / 89.4 against 81.8 / 87.1 / 89.4; of 8,192 and 16,384, 256 pairs: 175 and 345 against
-    # 168 and 329 (a share above 1: never).  Whole decode steps of the 7B shape: 32 requests at 1,024 keys
+    # 168 and 329 (a share above 1: never).  Contexts of up to 256 keys merge from one pair on (1 to 24
+    # requests at 128 / 192 / 256 keys: 4.6-4.9 / 5.1-6.0 / 5.6-7.2 against 5.1-6.0 / 6.6-8.3 / 6.5-8.1 us; at 384 keys
+    # both forms take the same time, from 512 on shares win: 8 requests 7.1 against 10.0 us).  Whole decode steps of the 7B shape: 32 requests at 1,024 keys
     # 3.92 -> 3.84 ms (in shares), 60 at 2,048 keys 4.98 -> 4.81 ms (merged); 48 at 1,024 keys 3.95 ms merged, 4.03 in shares.
     group_attention_fill: float = 1.0
-    group_attention_from: tuple = ((16, 0.45), (32, 0.7), (64, 0.85), (128, 0.97), (1 << 30, 1.01))
+    group_attention_from: tuple = ((8, 1 / 1024), (16, 0.45), (32, 0.7), (64, 0.85), (128, 0.97), (1 << 30, 1.01))
     # With more pairs than CUs the form is taken by an estimate of the launch's time, whose constants
     # are fitted to 63 launches of 288 to 1,024 pairs over contexts of 640 to 4,096 (3.5 % rms; the form
     # taken is 0.8 % slower than the best measured one on average, 6 % at worst).  The keys and values

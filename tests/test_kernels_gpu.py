@@ -1001,12 +1001,13 @@ def test_decode_attention_merged_inside_the_workgroup(nh, nkv, D, page, window, 
                               scale, window)
     assert rel_err(got.cpu(), ref) < ATTN_TOL[dt]
     # by itself: with a pair for nearly every CU (here: a table told that it has 24 CUs), or fewer of shorter contexts
-    # (0.97 of the CUs up to 4,096 keys, 0.7 up to 1,024, 0.45 up to 512; never beyond 4,096 with no more pairs than CUs)
+    # (0.97 of the CUs up to 4,096 keys, 0.7 up to 1,024, 0.45 up to 512, one pair up to 256; never beyond 4,096 with no more pairs than CUs)
     plain = HipOps(dt, "cuda:0")
     plain._num_cus = 24
     for n_seqs, ctx, merged in ((-(-24 // nkv), 4000, True), (max(1, 23 // nkv), 4000, False), (-(-24 // nkv), 5000, False),
                                 (-(-17 // nkv), 900, True), (max(1, 16 // nkv), 900, False),
-                                (-(-11 // nkv), 500, True), (max(1, 10 // nkv), 500, False)) if window is None else ():      # (a window makes every context short)
+                                (-(-11 // nkv), 500, True), (max(1, 10 // nkv), 500, False),
+                                (1, 200, True), (1, 300, False)) if window is None else ():      # (a window makes every context short)
         seen.clear()
         plain._call = lambda stem, name, *args: (seen.append((args[17], args[-3])) if name.startswith("sl_attention_mfma@") else None,
                                                  HipOps._call(plain, stem, name, *args))[1]
