@@ -272,7 +272,7 @@ class ProductOps:
         """How the block kernel takes a product of M rows: (shares of K, square tiles), or None
         when the product is not one of its own: bfloat16, a row-major copy of the weight, K in
         chunks of 64, a matrix of few rows (its tiles alone would leave most CUs idle, which is
-        what the split repairs) but of MID_MIN_ELEMENTS_MANY elements at least (smaller ones stay
+        what the split repairs) but of BLOCK_MIN_ELEMENTS elements at least (smaller ones stay
         with the kernels they were measured on).  Tiles of 256 x 128 for BLOCK_MIN_M to BLOCK_MAX_M
         rows of x; tiles of 256 x 256 for matrices with long rows (K of BLOCK_SQUARE_MIN_K and
         more: the down projection) from 257 to BLOCK_SQUARE_MAX_M rows, if their tiles and shares
@@ -283,7 +283,7 @@ class ProductOps:
         kernel; at 1,024 rows 111 us in 4 shares, 144 us in 6)."""
         w = weight.w if isinstance(weight, LinearWeight) else weight
         if (self.act_dtype != torch.bfloat16 or not self.use_block_products or w is None
-                or K % 64 or N % 4 or N > self.BLOCK_MAX_N or N * K < self.MID_MIN_ELEMENTS_MANY):
+                or K % 64 or N % 4 or N > self.BLOCK_MAX_N or N * K < self.BLOCK_MIN_ELEMENTS):
             return None
         if K >= self.BLOCK_SQUARE_MIN_K and 256 < M <= self.BLOCK_SQUARE_MAX_M:
             tiles = -(-N // 256) * -(-M // 256)

@@ -58,9 +58,17 @@ class Tuning:
     # workgroups of 8 wavefronts (16 tiles of W per pass over x) if this many remain, else 4
     mid_wide_workgroups: int = 128
     # matrices of this many elements take the LDS-staged kernel at 17..32 rows ...
-    mid_min_elements: int = 48 << 20
-    # ... and of this many at 33..128 rows, where re-reading x costs more
-    mid_min_elements_many: int = 8 << 20
+    mid_min_elements: int = 1 << 19
+    # ... and of this many at 33..128 rows (smaller ones: two tiles a workgroup straight from L2, up to 64 rows).
+    # Both were 48 M and 8 M elements while the kernel had workgroups of four wavefronts only; as it is, it
+    # wins at every size measured: decode steps of 24 / 32 requests, 7B shape (the output projection, 12.8 M
+    # elements) 4.33 -> 4.23 / 4.65 -> 4.54 ms, 32B shape 16.3 -> 16.0 / 17.7 -> 17.2 ms; the 0.5B shape (matrices
+    # of 0.8 to 8.7 M elements) at 24 / 48 / 80 / 128 requests 1.58 -> 1.32 / 2.05 -> 1.61 / 5.46 -> 1.75 / 5.11 ->
+    # 2.12 ms (beyond 64 rows its products went to the library, outside the captured step), 1.5B at 48 /
+    # 128: 2.83 -> 2.70 / 5.21 -> 3.59 ms, 3B at 48 / 128: 4.16 -> 4.02 / 6.24 -> 5.35 ms
+    mid_min_elements_many: int = 1 << 19
+    # matrices of fewer elements than this stay off the block kernel (tiles of 256 rows of x) at 129 rows and more
+    block_min_elements: int = 8 << 20
 
     # ---- the wavefront-per-column products (float32 table, bfloat16 fallbacks)
     # up to 16 rows of x go through LDS once per 32 columns of W instead of through L1 once per 4

@@ -235,9 +235,11 @@ def test_tiled_only_weights(M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(17, 50, 64), (33, 1000, 3584), (64, 3584, 1024), (40, 130, 352), (64, 70, 2048)])
 def test_linear_wide(M, N, K):
-    """The 17..64-row kernel alone: ragged M and N, an odd number of tiles."""
-    from servelab_amd.kernels import HipOps
-    ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
+    """The 17..64-row kernel alone: ragged M and N, an odd number of tiles; and that ``linear`` takes it
+    for matrices below the size from which the LDS-staged kernel takes over."""
+    from servelab_amd.kernels import HipOps, Tuning
+    ops = HipOps(torch.bfloat16, "cuda:0", tuning=Tuning(mid_min_elements=1 << 40, mid_min_elements_many=1 << 40))
+    emu = EmulatedOps(torch.bfloat16)
     x = randn(M, K, dtype=torch.bfloat16, seed=4)
     weight = ops.prepare_weight(randn(N, K, dtype=torch.bfloat16, scale=0.1, seed=5))
     b = randn(N, seed=6)
@@ -687,7 +689,7 @@ def test_a_row_gives_the_same_keys_whichever_path_its_step_takes():
     from servelab_amd.kernels import HipOps
     dt = torch.bfloat16
     ops = HipOps(dt, "cuda:0")
-    nh, nkv, D, page, H, M = 8, 2, 64, 16, 3072, 300       # 768 x 3072 = 2.4 M elements: library above 64 rows
+    nh, nkv, D, page, H, M = 8, 2, 64, 16, 3072, 300       # (the library takes products of more than 128 rows)
     N = (nh + 2 * nkv) * D
     x = randn(M, H, dtype=dt, seed=1)
     w = ops.prepare_weight(randn(N, H, dtype=dt, scale=0.02, seed=2))
@@ -709,7 +711,7 @@ def test_a_row_gives_the_same_keys_whichever_path_its_step_takes():
                                      sin[a:b].contiguous(), slots[a:b].contiguous(), kc, vc, page)
             q.append(qkv[:, :nh * D].float())
         return torch.cat(q), kc.float(), vc.float()
-    assert ops._few_rows_limit(w) == 64
+    assert ops._few_rows_limit(w) == 128
     whole, by8, by40 = run(M), run(8), run(40)
     for other in (by8, by40):
         for a, b in zip(whole, other):
@@ -1375,9 +1377,9 @@ def test_sampling_rows_with_different_rules_in_one_call(V):
 
 
 def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
-    """Large matrices take the LDS-staged kernel up to 128 rows (plain, gated,
-    deferred to the norm, with rotation and cache write, float32 logits of more
-    rows in slices of 128); small ones go to the library from 65 rows on."""
+    """Matrices of half a million elements and more take the LDS-staged kernel up to 128 rows
+    (plain, gated, deferred to the norm, with rotation and cache write, float32 logits of more
+    rows in slices of 128); smaller ones go to the library from 65 rows on."""
     from servelab_amd.kernels import HipOps
     from servelab_amd.kernels.ops import PartialSums
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
@@ -1386,7 +1388,8 @@ def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
     w = randn(N, K, dtype=torch.bfloat16, scale=0.05, seed=2)
     weight, b = ops.prepare_weight(w), randn(N, seed=3)
     assert ops._few_rows_limit(weight) == 128
-    assert ops._few_rows_limit(ops.prepare_weight(w[:256].contiguous())) == 64
+    assert ops._few_rows_limit(ops.prepare_weight(w[:256].contiguous())) == 128      # (0.9 M elements)
+    assert ops._few_rows_limit(ops.prepare_weight(w[:128].contiguous())) == 64
     assert torch.equal(ops.linear(x, weight, b), ops.linear_mid(x, weight, b))
     assert rel_err(ops.linear(x, weight, b), emu.linear(x, w, b)) < 2 ** -7
     assert rel_err(ops.gated_linear(x, weight, 8), emu.silu_mul(emu.linear(x, w, None), 8)) < 2 ** -6
