@@ -427,9 +427,12 @@ class AttentionOps:
             if nsplit > 1:
                 part_o = self._new((n_pre_tok, nh, nsplit, D), torch.float32)
                 part_ml = self._new((n_pre_tok, nh, nsplit, 2), torch.float32)
+            # workgroups of 64 columns instead of 128 for launches below this many of the latter
+            narrow_below = (self.NARROW_ATTENTION_SHORT_WORKGROUPS if batch.max_q_len <= self.NARROW_ATTENTION_SHORT_TOKENS
+                            else self.NARROW_ATTENTION_WORKGROUPS)
             self._call(lib, name, *common, 0, n_pre, batch.max_q_len, *tail, nsplit,
                        0 if shared else 1 << 30, int(pair), _p(out), _p(part_o), _p(part_ml), 0,
-                       n_pre_tok if nsplit > 1 else 0, self.NARROW_ATTENTION_WORKGROUPS if triangle else 0, 0, 0, None, 0)
+                       n_pre_tok if nsplit > 1 else 0, narrow_below if triangle else 0, 0, 0, None, 0)
         if n_dec:
             blocks = -(-batch.max_ctx_len // 32)
             if window:

@@ -196,6 +196,13 @@ class Tuning:
     # per tile: 2,048 tokens 57.5 against 71.4 us, 2,560: 78 against 86, 3,072: 113 against 102; portions
     # deep in a context keep 128 columns: 2,048 tokens after 6,144: 290 against 332 us)
     narrow_attention_workgroups: int = 600
+    # ... and prompts of at most narrow_attention_short_tokens tokens up to narrow_attention_short_workgroups:
+    # several short prompts have as many workgroups as one long one, but no long tiles for which the
+    # wider workgroups' fewer reads of the keys would pay (us, 64 against 128 columns: 7B shape, four
+    # prompts of 1,024 tokens 62 against 76; 32B shape, two of 1,024: 43 against 51, four: 80 against 85;
+    # 72B shape, four of 1,024: 118 against 120; two prompts of 2,048 tokens take the same time either way)
+    narrow_attention_short_tokens: int = 1024
+    narrow_attention_short_workgroups: int = 2000
     # where the launch is not laid out by chiplet (3, 5, 6, 7, 9.. kv heads), a workgroup of a whole
     # prompt takes a late tile of the causal triangle and its early mirror, unless the pairs would
     # fill the chip (two workgroups a CU) in several rounds, the last of them mostly empty: below
