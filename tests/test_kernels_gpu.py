@@ -1378,8 +1378,9 @@ def test_sampling_rows_with_different_rules_in_one_call(V):
 
 def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
     """Matrices of half a million elements and more take the LDS-staged kernel up to 128 rows
-    (plain, gated, deferred to the norm, with rotation and cache write, float32 logits of more
-    rows in slices of 128); smaller ones go to the library from 65 rows on."""
+    (plain, gated, deferred to the norm, with rotation and cache write; float32 logits of more
+    rows come from the library's float32 sums, or, without a row-major copy of the weight, in
+    slices of 128 rows); smaller ones go to the library from 65 rows on."""
     from servelab_amd.kernels import HipOps
     from servelab_amd.kernels.ops import PartialSums
     ops, emu = HipOps(torch.bfloat16, "cuda:0"), EmulatedOps(torch.bfloat16)
@@ -1398,6 +1399,11 @@ def test_products_of_65_to_128_rows_stay_with_the_tiled_weight():
     assert rel_err(ops.materialize(delta), emu.linear(x, w, b)) < 2 ** -7
     many = randn(300, K, dtype=torch.bfloat16, seed=4)
     got = ops.linear(many, weight, b, out_f32=True)
+    assert got.shape == (300, N) and rel_err(got, emu.linear(many, w, b, True)) < 2e-5
+    ops.weight_layout = "tiled"
+    tiled_only = ops.prepare_weight(w.clone())
+    assert tiled_only.w is None
+    got = ops.linear(many, tiled_only, b, out_f32=True)
     assert got.shape == (300, N) and rel_err(got, emu.linear(many, w, b, True)) < 2e-5
 
 
