@@ -291,8 +291,9 @@ class AttentionOps:
         CUs: 30.6 us a layer; in 9, 504 wavefronts: about 22 us); every wavefront a CU costs FEW_WAVE_US,
         and the combine kernel reads the partial results sixteen shares at a time, FEW_BATCH_US a batch.
         Fitted to 1,500 launches of 1 to 24 requests of the 7B shape at contexts of 512 to 32,768 (mean
-        error 4 %); the count taken costs 0.7 % more than the best measured one on average and 7 % at worst.
-        (Filling whole rounds of the CUs near two wavefronts each, the rule before: 1.1 % and 18 %: it took
+        error 4 %); over those and four further contexts the count taken costs 0.5 % more than the best
+        measured one on average and 4 % at worst.
+        (Filling whole rounds of the CUs near two wavefronts each, the rule before: 1.2 % and 20 %: it took
         128 shares for one request at 8,192 to 16,384 keys where 64 are faster, 12.0 against 10.2 us, and
         fewer than the context allows at 512 and 1,024 keys, where one trip beats full rounds.)"""
         cus = self._num_cus
